@@ -1,0 +1,84 @@
+// Internal device helpers: bf16 <-> f32, 128-bit packets, wave64 and block reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(bf16_t x) { return (float)x; }
+template <typename T> __device__ __forceinline__ T from_f32(float x);
+template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return (bf16_t)x; }  // RNE (v_cvt_pk_bf16_f32)
+
+// A 16-byte packet of T: 4 floats or 8 bf16.
+template <typename T> struct Pack;
+template <> struct Pack<float> {
+    static constexpr int N = 4;
+    float4 raw;
+    __device__ __forceinline__ float get(int i) const { return (&raw.x)[i]; }
+    __device__ __forceinline__ void set(int i, float v) { (&raw.x)[i] = v; }
+};
+template <> struct Pack<bf16_t> {
+    static constexpr int N = 8;
+    bf16x8 raw;
+    __device__ __forceinline__ float get(int i) const { return (float)raw[i]; }
+    __device__ __forceinline__ void set(int i, float v) { raw[i] = (bf16_t)v; }
+};
+template <typename T> __device__ __forceinline__ Pack<T> load_pack(const T* p) {
+    return *reinterpret_cast<const Pack<T>*>(p);
+}
+template <typename T> __device__ __forceinline__ void store_pack(T* p, const Pack<T>& v) {
+    *reinterpret_cast<Pack<T>*>(p) = v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// Block-wide reductions; every thread gets the result.  `smem` holds >= blockDim.x/64 floats.
+// The result is the same in every thread and independent of timing (fixed tree).
+template <int THREADS> __device__ __forceinline__ float block_sum(float v, float* smem) {
+    constexpr int W = THREADS / kWave;
+    v = wave_sum(v);
+    if (W == 1) return v;
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) smem[wid] = v;
+    __syncthreads();
+    float r = 0.f;
+#pragma unroll
+    for (int i = 0; i < W; i++) r += smem[i];
+    return r;
+}
+template <int THREADS> __device__ __forceinline__ float block_max(float v, float* smem) {
+    constexpr int W = THREADS / kWave;
+    v = wave_max(v);
+    if (W == 1) return v;
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) smem[wid] = v;
+    __syncthreads();
+    float r = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < W; i++) r = fmaxf(r, smem[i]);
+    return r;
+}

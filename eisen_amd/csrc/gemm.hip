@@ -1,0 +1,300 @@
+// GEMM family: C[M,N] (+)= op(A) * op(B), row-major, optional batch.
+//
+//   forward  Y  = X * W          (A [M,K], B [K,N])            Graph::matmul, src/graph/ops/linear.rs:254-262
+//   dX       dA = dC * B^T       (A [M,K'], B stored [N',K'])   src/graph/ops/linear.rs:269-277
+//   dW       dB = A^T * dC       (A stored [K',M'], B [K',N'])  src/graph/ops/linear.rs:279-287
+//   tied lm_head / bmm with trans_b                             src/graph/ops/linear.rs:456-481, :1430-1446
+//
+// bf16 path: MFMA v_mfma_f32_32x32x16_bf16, f32 accumulate.  A workgroup of 4 waves owns a
+// BM x BN tile of C; each wave owns a (BM/2) x (BN/2) quadrant made of 32x32 MFMA tiles.  K is walked in slabs of
+// 32 through double-buffered LDS (one barrier per slab) with the next slab's global loads in
+// flight during the current slab's MFMAs.  LDS always holds both operands K-contiguous, which
+// is the order the MFMA operand registers want (8 consecutive k per lane, one ds_read_b128);
+// an operand whose memory order is the other way round is transposed on its way into LDS.
+//
+// f32 path and odd shapes: a plain LDS-tiled FMA kernel (64x64 tile, 4x4 per thread).
+#include "device_utils.cuh"
+#include "runtime.h"
+
+namespace {
+
+constexpr int kGemmThreads = 256;
+constexpr int BK = 32;
+constexpr int LDS_PITCH = BK + 8;  // bf16 elements; 80-byte rows keep 16-byte alignment and spread banks
+
+struct GemmArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int M, N, K;
+    int lda, ldb, ldc;                 // leading dimensions in elements
+    long long sA, sB, sC;              // batch strides in elements
+    int accumulate;
+};
+
+// ---- MFMA kernel -------------------------------------------------------------------------
+// A_KC: A is stored [M][K] (k contiguous); otherwise [K][M].  B_KC: B is stored [N][K];
+// otherwise [K][N].
+template <int BM, int BN, bool A_KC, bool B_KC, typename TC>
+__global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
+    constexpr int WM = BM / 2, WN = BN / 2;          // wave quadrant
+    constexpr int TM = WM / 32, TN = WN / 32;        // 32x32 tiles per wave
+    constexpr int A_CHUNKS = BM * BK / 8 / kGemmThreads;  // 16-byte chunks per thread per slab
+    constexpr int B_CHUNKS = BN * BK / 8 / kGemmThreads;
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2][(BM + BN) * LDS_PITCH];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    // neighbouring workgroups share an A row-block: walk N fastest inside a strip of M
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const bf16_t* A = static_cast<const bf16_t*>(g.A) + (long long)blockIdx.z * g.sA;
+    const bf16_t* B = static_cast<const bf16_t*>(g.B) + (long long)blockIdx.z * g.sB;
+    TC* C = static_cast<TC*>(g.C) + (long long)blockIdx.z * g.sC;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    bf16x8 ra[A_CHUNKS], rb[B_CHUNKS];
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < A_CHUNKS; c++) {
+            const int chunk = c * kGemmThreads + tid;
+            if (A_KC) {
+                const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
+                const int m = m0 + row, k = k0 + kc * 8;
+                ra[c] = (m < g.M && k < g.K) ? *reinterpret_cast<const bf16x8*>(A + (long long)m * g.lda + k) : zero8;
+            } else {
+                const int kk = chunk / (BM / 8), mc = chunk % (BM / 8);
+                const int m = m0 + mc * 8, k = k0 + kk;
+                ra[c] = (m < g.M && k < g.K) ? *reinterpret_cast<const bf16x8*>(A + (long long)k * g.lda + m) : zero8;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < B_CHUNKS; c++) {
+            const int chunk = c * kGemmThreads + tid;
+            if (B_KC) {
+                const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
+                const int n = n0 + row, k = k0 + kc * 8;
+                rb[c] = (n < g.N && k < g.K) ? *reinterpret_cast<const bf16x8*>(B + (long long)n * g.ldb + k) : zero8;
+            } else {
+                const int kk = chunk / (BN / 8), nc = chunk % (BN / 8);
+                const int n = n0 + nc * 8, k = k0 + kk;
+                rb[c] = (n < g.N && k < g.K) ? *reinterpret_cast<const bf16x8*>(B + (long long)k * g.ldb + n) : zero8;
+            }
+        }
+    };
+    auto store_lds = [&](int buf) {
+        bf16_t* As = lds[buf];
+        bf16_t* Bs = lds[buf] + BM * LDS_PITCH;
+#pragma unroll
+        for (int c = 0; c < A_CHUNKS; c++) {
+            const int chunk = c * kGemmThreads + tid;
+            if (A_KC) {
+                const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
+                *reinterpret_cast<bf16x8*>(As + row * LDS_PITCH + kc * 8) = ra[c];
+            } else {
+                const int kk = chunk / (BM / 8), mc = chunk % (BM / 8);
+#pragma unroll
+                for (int j = 0; j < 8; j++) As[(mc * 8 + j) * LDS_PITCH + kk] = ra[c][j];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < B_CHUNKS; c++) {
+            const int chunk = c * kGemmThreads + tid;
+            if (B_KC) {
+                const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
+                *reinterpret_cast<bf16x8*>(Bs + row * LDS_PITCH + kc * 8) = rb[c];
+            } else {
+                const int kk = chunk / (BN / 8), nc = chunk % (BN / 8);
+#pragma unroll
+                for (int j = 0; j < 8; j++) Bs[(nc * 8 + j) * LDS_PITCH + kk] = rb[c][j];
+            }
+        }
+    };
+
+    const int nk = (g.K + BK - 1) / BK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) load_global((kt + 1) * BK);
+        const bf16_t* As = lds[buf] + (wm * WM + (lane & 31)) * LDS_PITCH + (lane >> 5) * 8;
+        const bf16_t* Bs = lds[buf] + BM * LDS_PITCH + (wn * WN + (lane & 31)) * LDS_PITCH + (lane >> 5) * 8;
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 16) {
+            bf16x8 a[TM], b[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) a[i] = *reinterpret_cast<const bf16x8*>(As + i * 32 * LDS_PITCH + ks);
+#pragma unroll
+            for (int j = 0; j < TN; j++) b[j] = *reinterpret_cast<const bf16x8*>(Bs + j * 32 * LDS_PITCH + ks);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WN + j * 32 + (lane & 31);
+            if (n >= g.N) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (m < g.M) {
+                    TC* dst = C + (long long)m * g.ldc + n;
+                    const float val = acc[i][j][v];
+                    *dst = from_f32<TC>(g.accumulate ? to_f32(*dst) + val : val);
+                }
+            }
+        }
+}
+
+// ---- generic kernel (f32, or bf16 with shapes the MFMA kernel does not take) ---------------
+template <typename TA, typename TC>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g, int trans_a, int trans_b) {
+    constexpr int T = 64, KT = 16;
+    __shared__ float As[KT][T + 1], Bs[KT][T + 1];
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+    const TA* A = static_cast<const TA*>(g.A) + (long long)blockIdx.z * g.sA;
+    const TA* B = static_cast<const TA*>(g.B) + (long long)blockIdx.z * g.sB;
+    TC* C = static_cast<TC*>(g.C) + (long long)blockIdx.z * g.sC;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < g.K; k0 += KT) {
+        for (int e = tid; e < T * KT; e += 256) {
+            // read along the operand's contiguous dimension
+            int kk, mm;
+            if (trans_a) { kk = e / T; mm = e % T; } else { mm = e / KT; kk = e % KT; }
+            const int m = m0 + mm, k = k0 + kk;
+            float v = 0.f;
+            if (m < g.M && k < g.K) v = to_f32(trans_a ? A[(long long)k * g.lda + m] : A[(long long)m * g.lda + k]);
+            As[kk][mm] = v;
+            int kb, nn;
+            if (trans_b) { nn = e / KT; kb = e % KT; } else { kb = e / T; nn = e % T; }
+            const int n = n0 + nn, k2 = k0 + kb;
+            float w = 0.f;
+            if (n < g.N && k2 < g.K) w = to_f32(trans_b ? B[(long long)n * g.ldb + k2] : B[(long long)k2 * g.ldb + n]);
+            Bs[kb][nn] = w;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KT; kk++) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; j++) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] += a[i] * b[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+            if (m < g.M && n < g.N) {
+                TC* dst = C + (long long)m * g.ldc + n;
+                *dst = from_f32<TC>(g.accumulate ? to_f32(*dst) + acc[i][j] : acc[i][j]);
+            }
+        }
+}
+
+template <int BM, int BN, typename TC>
+void launch_mfma(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int batch) {
+    dim3 grid((unsigned)eisen_ceil_div(g.N, BN), (unsigned)eisen_ceil_div(g.M, BM), (unsigned)batch);
+    if (a_kc && b_kc) gemm_mfma_kernel<BM, BN, true, true, TC><<<grid, kGemmThreads, 0, ctx->stream>>>(g);
+    else if (a_kc && !b_kc) gemm_mfma_kernel<BM, BN, true, false, TC><<<grid, kGemmThreads, 0, ctx->stream>>>(g);
+    else if (!a_kc && b_kc) gemm_mfma_kernel<BM, BN, false, true, TC><<<grid, kGemmThreads, 0, ctx->stream>>>(g);
+    else gemm_mfma_kernel<BM, BN, false, false, TC><<<grid, kGemmThreads, 0, ctx->stream>>>(g);
+}
+
+template <typename TA, typename TC>
+void launch_generic(eisen_ctx* ctx, const GemmArgs& g, int trans_a, int trans_b, int batch) {
+    dim3 grid((unsigned)eisen_ceil_div(g.N, 64), (unsigned)eisen_ceil_div(g.M, 64), (unsigned)batch);
+    gemm_generic_kernel<TA, TC><<<grid, 256, 0, ctx->stream>>>(g, trans_a, trans_b);
+}
+
+}  // namespace
+
+// Internal entry shared by eisen_hip_gemm and eisen_hip_bmm.
+static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
+                       int trans_b, size_t M, size_t N, size_t K, size_t batch, long long sA, long long sB, long long sC,
+                       int accumulate, const char* who) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, A && B && C, EISEN_E_ARG, "%s: null pointer", who);
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype_ab) && eisen_dtype_ok(dtype_c), EISEN_E_ARG, "%s: unknown dtype", who);
+    EISEN_REQUIRE(ctx, !(dtype_ab == EISEN_F32 && dtype_c == EISEN_BF16), EISEN_E_ARG, "%s: f32 operands with bf16 output is not a supported combination", who);
+    EISEN_REQUIRE(ctx, M < (size_t(1) << 30) && N < (size_t(1) << 30) && K < (size_t(1) << 30) && batch < 65536, EISEN_E_SHAPE, "%s: dimension out of range", who);
+    if (M == 0 || N == 0 || batch == 0) return 0;
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C;
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.lda = (int)(trans_a ? M : K);
+    g.ldb = (int)(trans_b ? K : N);
+    g.ldc = (int)N;
+    g.sA = sA; g.sB = sB; g.sC = sC;
+    g.accumulate = accumulate;
+    if (K == 0) {  // empty contraction: C (+)= 0
+        if (!accumulate) {
+            for (size_t b = 0; b < batch; b++) {
+                int rc = eisen_hip_memset_zero(ctx, (char*)C + b * sC * eisen_dtype_size(dtype_c), M * N * eisen_dtype_size(dtype_c));
+                if (rc) return rc;
+            }
+        }
+        return 0;
+    }
+    const bool a_kc = !trans_a, b_kc = trans_b != 0;
+    bool mfma_ok = dtype_ab == EISEN_BF16 && eisen_aligned(A, 16) && eisen_aligned(B, 16) && g.lda % 8 == 0 && g.ldb % 8 == 0 &&
+                   sA % 8 == 0 && sB % 8 == 0;
+    // the contiguous dimension of each operand must be a whole number of 8-element chunks
+    if (a_kc) mfma_ok = mfma_ok && K % 8 == 0; else mfma_ok = mfma_ok && M % 8 == 0;
+    if (b_kc) mfma_ok = mfma_ok && K % 8 == 0; else mfma_ok = mfma_ok && N % 8 == 0;
+    if (mfma_ok) {
+        // 128x128 tiles unless the problem is too small to give every CU a tile
+        const size_t tiles128 = eisen_ceil_div(M, 128) * eisen_ceil_div(N, 128) * batch;
+        if (tiles128 >= 256 || (M >= 128 && N >= 128 && tiles128 >= 128)) {
+            if (dtype_c == EISEN_BF16) launch_mfma<128, 128, bf16_t>(ctx, g, a_kc, b_kc, (int)batch);
+            else launch_mfma<128, 128, float>(ctx, g, a_kc, b_kc, (int)batch);
+        } else {
+            if (dtype_c == EISEN_BF16) launch_mfma<64, 64, bf16_t>(ctx, g, a_kc, b_kc, (int)batch);
+            else launch_mfma<64, 64, float>(ctx, g, a_kc, b_kc, (int)batch);
+        }
+    } else if (dtype_ab == EISEN_F32) {
+        launch_generic<float, float>(ctx, g, trans_a, trans_b, (int)batch);
+    } else if (dtype_c == EISEN_BF16) {
+        launch_generic<bf16_t, bf16_t>(ctx, g, trans_a, trans_b, (int)batch);
+    } else {
+        launch_generic<bf16_t, float>(ctx, g, trans_a, trans_b, (int)batch);
+    }
+    EISEN_LAUNCH_CHECK(ctx, who);
+    return 0;
+}
+
+extern "C" int eisen_hip_gemm(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
+                              int trans_b, size_t M, size_t N, size_t K, int accumulate) {
+    return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, 1, 0, 0, 0, accumulate, "eisen_hip_gemm");
+}
+
+extern "C" int eisen_hip_bmm(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
+                             int trans_b, size_t batch, size_t M, size_t N, size_t K, int accumulate) {
+    return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, batch, (long long)(M * K), (long long)(K * N),
+                       (long long)(M * N), accumulate, "eisen_hip_bmm");
+}

@@ -1,0 +1,306 @@
+// RMSNorm forward/backward and row softmax forward/backward.
+// One 64-lane wave owns one row; lanes stride the row in 16-byte packets so every global
+// access is a fully coalesced 1 KiB wave transaction.  Reductions are wave shuffles.
+#include "device_utils.cuh"
+#include "runtime.h"
+
+namespace {
+
+constexpr int kRowThreads = 256;  // 4 waves = 4 rows per block
+constexpr int kRowWaves = kRowThreads / kWave;
+
+// y = x * rrms * w,  rrms = 1/sqrt(mean(x^2) + eps)   (src/graph/ops/normalization.rs:141-151)
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void rms_norm_fwd_kernel(const T* __restrict__ x, const float* __restrict__ w,
+                                                                   T* __restrict__ out, float* __restrict__ rrms_out,
+                                                                   size_t rows, int dim, float eps) {
+    constexpr int N = VEC ? Pack<T>::N : 1;
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * kRowWaves + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * dim;
+    T* orow = out + row * dim;
+    float ss = 0.f;
+    for (int c = lane * N; c < dim; c += kWave * N) {
+        if (VEC) {
+            const Pack<T> p = load_pack(xr + c);
+#pragma unroll
+            for (int j = 0; j < N; j++) ss += p.get(j) * p.get(j);
+        } else {
+            const float v = to_f32(xr[c]);
+            ss += v * v;
+        }
+    }
+    ss = wave_sum(ss);
+    const float rrms = 1.0f / sqrtf(ss / (float)dim + eps);
+    if (lane == 0) rrms_out[row] = rrms;
+    for (int c = lane * N; c < dim; c += kWave * N) {
+        if (VEC) {
+            const Pack<T> p = load_pack(xr + c);  // second read of a row this wave just streamed: L2/TCP hit
+            Pack<T> o;
+#pragma unroll
+            for (int j = 0; j < N; j++) o.set(j, p.get(j) * rrms * w[c + j]);
+            store_pack(orow + c, o);
+        } else {
+            orow[c] = from_f32<T>(to_f32(xr[c]) * rrms * w[c]);
+        }
+    }
+}
+
+// dx = rrms*(go*w) - x*(rrms^3/D)*sum_d(go*x*w);  dw_partial[d] += go*x*rrms
+// (src/graph/ops/normalization.rs:157-171).  Each wave walks rows wave_id, wave_id+W, ...
+// and keeps its dw partial in registers; partials meet in LDS and leave as one row of
+// `partial` per block.  A second kernel sums the block rows in fixed order.
+template <typename T, int MAXP>
+__global__ __launch_bounds__(kRowThreads) void rms_norm_bwd_kernel(const T* __restrict__ x, const float* __restrict__ w,
+                                                                   const float* __restrict__ rrms_in,
+                                                                   const T* __restrict__ go, T* __restrict__ gx,
+                                                                   float* __restrict__ partial, size_t rows, int dim,
+                                                                   int accumulate_x) {
+    constexpr int N = Pack<T>::N;
+    extern __shared__ float lds[];  // [kRowWaves][dim]
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const size_t wave_global = (size_t)blockIdx.x * kRowWaves + wid;
+    const size_t wave_stride = (size_t)gridDim.x * kRowWaves;
+    float dw[MAXP][N];
+#pragma unroll
+    for (int p = 0; p < MAXP; p++)
+#pragma unroll
+        for (int j = 0; j < N; j++) dw[p][j] = 0.f;
+
+    for (size_t row = wave_global; row < rows; row += wave_stride) {
+        const T* xr = x + row * dim;
+        const T* gr = go + row * dim;
+        T* gxr = gx + row * dim;
+        const float rrms = rrms_in[row];
+        Pack<T> xp[MAXP], gp[MAXP];
+        float gdxw = 0.f;
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) {
+            const int c = (p * kWave + lane) * N;
+            if (c < dim) {
+                xp[p] = load_pack(xr + c);
+                gp[p] = load_pack(gr + c);
+#pragma unroll
+                for (int j = 0; j < N; j++) gdxw += gp[p].get(j) * xp[p].get(j) * w[c + j];
+            }
+        }
+        gdxw = wave_sum(gdxw);
+        const float rrc_d = rrms * rrms * rrms / (float)dim;
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) {
+            const int c = (p * kWave + lane) * N;
+            if (c < dim) {
+                Pack<T> o;
+                if (accumulate_x) o = load_pack(gxr + c);
+#pragma unroll
+                for (int j = 0; j < N; j++) {
+                    const float xv = xp[p].get(j), gv = gp[p].get(j);
+                    const float dx = rrms * (gv * w[c + j]) - xv * rrc_d * gdxw;
+                    o.set(j, accumulate_x ? o.get(j) + dx : dx);
+                    dw[p][j] += gv * xv * rrms;
+                }
+                store_pack(gxr + c, o);
+            }
+        }
+    }
+    // combine the block's waves in a fixed order
+#pragma unroll
+    for (int p = 0; p < MAXP; p++) {
+        const int c = (p * kWave + lane) * N;
+        if (c < dim)
+#pragma unroll
+            for (int j = 0; j < N; j++) lds[wid * dim + c + j] = dw[p][j];
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < dim; c += kRowThreads) {
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < kRowWaves; k++) s += lds[k * dim + c];
+        partial[(size_t)blockIdx.x * dim + c] = s;
+    }
+}
+
+__global__ void rms_norm_dw_reduce_kernel(const float* __restrict__ partial, float* __restrict__ gw, int nblocks, int dim) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= dim) return;
+    float s = 0.f;
+    for (int b = 0; b < nblocks; b++) s += partial[(size_t)b * dim + c];
+    gw[c] += s;
+}
+
+// Scalar fallback for rows that are not packet-aligned: one wave per row, same arithmetic.
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void rms_norm_bwd_scalar_kernel(const T* __restrict__ x, const float* __restrict__ w,
+                                                                          const float* __restrict__ rrms_in,
+                                                                          const T* __restrict__ go, T* __restrict__ gx,
+                                                                          size_t rows, int dim, int accumulate_x) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * kRowWaves + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * dim;
+    const T* gr = go + row * dim;
+    T* gxr = gx + row * dim;
+    const float rrms = rrms_in[row];
+    float gdxw = 0.f;
+    for (int c = lane; c < dim; c += kWave) gdxw += to_f32(gr[c]) * to_f32(xr[c]) * w[c];
+    gdxw = wave_sum(gdxw);
+    const float rrc_d = rrms * rrms * rrms / (float)dim;
+    for (int c = lane; c < dim; c += kWave) {
+        const float dx = rrms * (to_f32(gr[c]) * w[c]) - to_f32(xr[c]) * rrc_d * gdxw;
+        gxr[c] = from_f32<T>(accumulate_x ? to_f32(gxr[c]) + dx : dx);
+    }
+}
+// dw for the scalar fallback: one thread per column walks the rows in order.
+template <typename T>
+__global__ void rms_norm_dw_scalar_kernel(const T* __restrict__ x, const float* __restrict__ rrms_in,
+                                          const T* __restrict__ go, float* __restrict__ gw, size_t rows, int dim) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= dim) return;
+    float s = 0.f;
+    for (size_t r = 0; r < rows; r++) s += to_f32(go[r * dim + c]) * to_f32(x[r * dim + c]) * rrms_in[r];
+    gw[c] += s;
+}
+
+// softmax over the last dim (src/graph/ops/reduction.rs:483-496): max, exp(x-max), divide.
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ out, size_t rows,
+                                                                  int n) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * kRowWaves + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * n;
+    T* orow = out + row * n;
+    float mx = -INFINITY;
+    for (int c = lane; c < n; c += kWave) mx = fmaxf(mx, to_f32(xr[c]));
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int c = lane; c < n; c += kWave) sum += __expf(to_f32(xr[c]) - mx);
+    sum = wave_sum(sum);
+    for (int c = lane; c < n; c += kWave) orow[c] = from_f32<T>(__expf(to_f32(xr[c]) - mx) / sum);
+}
+
+// gx += y*(go - sum(go*y))   (src/graph/ops/reduction.rs:504-512)
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void softmax_bwd_kernel(const T* __restrict__ y, const T* __restrict__ go,
+                                                                  T* __restrict__ gx, size_t rows, int n, int accumulate) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * kRowWaves + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* yr = y + row * n;
+    const T* gr = go + row * n;
+    T* gxr = gx + row * n;
+    float dot = 0.f;
+    for (int c = lane; c < n; c += kWave) dot += to_f32(gr[c]) * to_f32(yr[c]);
+    dot = wave_sum(dot);
+    for (int c = lane; c < n; c += kWave) {
+        const float v = to_f32(yr[c]) * (to_f32(gr[c]) - dot);
+        gxr[c] = from_f32<T>(accumulate ? to_f32(gxr[c]) + v : v);
+    }
+}
+
+template <typename T>
+int rms_norm_fwd(eisen_ctx* ctx, const void* x, const float* w, void* out, float* rrms, size_t rows, size_t dim, float eps) {
+    const unsigned blocks = (unsigned)eisen_ceil_div(rows, kRowWaves);
+    const bool vec = dim % Pack<T>::N == 0 && eisen_aligned(x, 16) && eisen_aligned(out, 16);
+    if (vec)
+        rms_norm_fwd_kernel<T, true><<<blocks, kRowThreads, 0, ctx->stream>>>((const T*)x, w, (T*)out, rrms, rows, (int)dim, eps);
+    else
+        rms_norm_fwd_kernel<T, false><<<blocks, kRowThreads, 0, ctx->stream>>>((const T*)x, w, (T*)out, rrms, rows, (int)dim, eps);
+    EISEN_LAUNCH_CHECK(ctx, "rms_norm_fwd_kernel");
+    return 0;
+}
+
+template <typename T, int MAXP>
+int rms_norm_bwd_vec(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* gw,
+                     size_t rows, size_t dim, int accumulate_x) {
+    // enough waves to cover the chip a few times over, few enough that the partial rows stay small
+    unsigned blocks = (unsigned)std::min<size_t>(eisen_ceil_div(rows, kRowWaves), 512);
+    void* ws = nullptr;
+    int rc = eisen_workspace(ctx, (size_t)blocks * dim * sizeof(float), &ws);
+    if (rc) return rc;
+    const size_t lds = (size_t)kRowWaves * dim * sizeof(float);
+    rms_norm_bwd_kernel<T, MAXP><<<blocks, kRowThreads, lds, ctx->stream>>>((const T*)x, w, rrms, (const T*)go, (T*)gx,
+                                                                            (float*)ws, rows, (int)dim, accumulate_x);
+    EISEN_LAUNCH_CHECK(ctx, "rms_norm_bwd_kernel");
+    rms_norm_dw_reduce_kernel<<<(unsigned)eisen_ceil_div(dim, 256), 256, 0, ctx->stream>>>((const float*)ws, gw, (int)blocks, (int)dim);
+    EISEN_LAUNCH_CHECK(ctx, "rms_norm_dw_reduce_kernel");
+    return 0;
+}
+
+template <typename T>
+int rms_norm_bwd(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* gw,
+                 size_t rows, size_t dim, int accumulate_x) {
+    constexpr int N = Pack<T>::N;
+    const bool vec = dim % N == 0 && eisen_aligned(x, 16) && eisen_aligned(go, 16) && eisen_aligned(gx, 16) &&
+                     dim <= (size_t)kWave * N * 8 && (size_t)kRowWaves * dim * sizeof(float) <= 64 * 1024;
+    if (vec) {
+        const size_t packs = eisen_ceil_div(dim, (size_t)kWave * N);
+        if (packs <= 1) return rms_norm_bwd_vec<T, 1>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
+        if (packs <= 2) return rms_norm_bwd_vec<T, 2>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
+        if (packs <= 4) return rms_norm_bwd_vec<T, 4>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
+        return rms_norm_bwd_vec<T, 8>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
+    }
+    rms_norm_bwd_scalar_kernel<T><<<(unsigned)eisen_ceil_div(rows, kRowWaves), kRowThreads, 0, ctx->stream>>>(
+        (const T*)x, w, rrms, (const T*)go, (T*)gx, rows, (int)dim, accumulate_x);
+    EISEN_LAUNCH_CHECK(ctx, "rms_norm_bwd_scalar_kernel");
+    rms_norm_dw_scalar_kernel<T><<<(unsigned)eisen_ceil_div(dim, 256), 256, 0, ctx->stream>>>((const T*)x, rrms, (const T*)go, gw, rows, (int)dim);
+    EISEN_LAUNCH_CHECK(ctx, "rms_norm_dw_scalar_kernel");
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int eisen_hip_rms_norm(eisen_ctx* ctx, const void* x, const float* w, void* out, float* rrms, int dtype,
+                                  size_t rows, size_t dim, float eps) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, x && w && out && rrms, EISEN_E_ARG, "eisen_hip_rms_norm: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_rms_norm: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, dim > 0 && dim < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_rms_norm: dim %zu out of range", dim);
+    if (rows == 0) return 0;
+    return dtype == EISEN_F32 ? rms_norm_fwd<float>(ctx, x, w, out, rrms, rows, dim, eps)
+                              : rms_norm_fwd<bf16_t>(ctx, x, w, out, rrms, rows, dim, eps);
+}
+
+extern "C" int eisen_hip_rms_norm_backward(eisen_ctx* ctx, const void* x, const float* w, const float* rrms,
+                                           const void* go, void* gx, float* gw, int dtype, size_t rows, size_t dim,
+                                           int accumulate_x) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, x && w && rrms && go && gx && gw, EISEN_E_ARG, "eisen_hip_rms_norm_backward: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_rms_norm_backward: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, dim > 0 && dim < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_rms_norm_backward: dim %zu out of range", dim);
+    if (rows == 0) return 0;
+    return dtype == EISEN_F32 ? rms_norm_bwd<float>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x)
+                              : rms_norm_bwd<bf16_t>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
+}
+
+extern "C" int eisen_hip_softmax(eisen_ctx* ctx, const void* x, void* out, int dtype, size_t rows, size_t n) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, x && out, EISEN_E_ARG, "eisen_hip_softmax: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_softmax: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, n > 0 && n < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_softmax: n %zu out of range", n);
+    if (rows == 0) return 0;
+    const unsigned blocks = (unsigned)eisen_ceil_div(rows, kRowWaves);
+    if (dtype == EISEN_F32)
+        softmax_fwd_kernel<float><<<blocks, kRowThreads, 0, ctx->stream>>>((const float*)x, (float*)out, rows, (int)n);
+    else
+        softmax_fwd_kernel<bf16_t><<<blocks, kRowThreads, 0, ctx->stream>>>((const bf16_t*)x, (bf16_t*)out, rows, (int)n);
+    EISEN_LAUNCH_CHECK(ctx, "softmax_fwd_kernel");
+    return 0;
+}
+
+extern "C" int eisen_hip_softmax_backward(eisen_ctx* ctx, const void* out, const void* go, void* gx, int dtype,
+                                          size_t rows, size_t n, int accumulate) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, out && go && gx, EISEN_E_ARG, "eisen_hip_softmax_backward: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_softmax_backward: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, n > 0 && n < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_softmax_backward: n %zu out of range", n);
+    if (rows == 0) return 0;
+    const unsigned blocks = (unsigned)eisen_ceil_div(rows, kRowWaves);
+    if (dtype == EISEN_F32)
+        softmax_bwd_kernel<float><<<blocks, kRowThreads, 0, ctx->stream>>>((const float*)out, (const float*)go, (float*)gx, rows, (int)n, accumulate);
+    else
+        softmax_bwd_kernel<bf16_t><<<blocks, kRowThreads, 0, ctx->stream>>>((const bf16_t*)out, (const bf16_t*)go, (bf16_t*)gx, rows, (int)n, accumulate);
+    EISEN_LAUNCH_CHECK(ctx, "softmax_bwd_kernel");
+    return 0;
+}

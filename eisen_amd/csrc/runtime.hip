@@ -1,0 +1,290 @@
+// Runtime half of the C-ABI: context, one stream, stream-ordered pool, copies, module
+// load / launch by name, event timer.  Replaces the cudarc calls of the reference
+// (src/graph/mod.rs:152-307, src/graph/memory.rs:189-266, src/tensor.rs:145-223).
+#include "runtime.h"
+
+int eisen_set_error(eisen_ctx* ctx, int code, const char* fmt, ...) {
+    if (ctx) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(ctx->last_error, sizeof(ctx->last_error), fmt, ap);
+        va_end(ap);
+    }
+    return code;
+}
+
+extern "C" const char* eisen_hip_last_error(eisen_ctx* ctx) { return ctx ? ctx->last_error : "null context"; }
+
+extern "C" int eisen_hip_init(int device, eisen_ctx** out) {
+    if (!out) return EISEN_E_ARG;
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess) return (int)e;
+    if (device < 0 || device >= count) return EISEN_E_ARG;
+    e = hipSetDevice(device);
+    if (e != hipSuccess) return (int)e;
+    eisen_ctx* ctx = new eisen_ctx();
+    ctx->device = device;
+    // default priority, non-blocking with respect to the legacy null stream
+    e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&ctx->ev_start);
+    if (e == hipSuccess) e = hipEventCreate(&ctx->ev_stop);
+    if (e == hipSuccess) {
+        // keep freed blocks inside the driver pool instead of returning them to the OS
+        hipMemPool_t pool;
+        if (hipDeviceGetDefaultMemPool(&pool, device) == hipSuccess) {
+            uint64_t threshold = UINT64_MAX;
+            (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &threshold);
+        }
+        (void)hipGetLastError();
+    }
+    if (e != hipSuccess) {
+        delete ctx;
+        return (int)e;
+    }
+    *out = ctx;
+    return 0;
+}
+
+extern "C" int eisen_hip_pool_trim(eisen_ctx* ctx) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_HIP_TRY(ctx, hipSetDevice(ctx->device));
+    for (auto& kv : ctx->free_lists)
+        for (void* p : kv.second) EISEN_HIP_TRY(ctx, hipFreeAsync(p, ctx->stream));
+    ctx->free_lists.clear();
+    ctx->cached_bytes = 0;
+    return 0;
+}
+
+extern "C" int eisen_hip_destroy(eisen_ctx* ctx) {
+    EISEN_CHECK_CTX(ctx);
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)eisen_hip_pool_trim(ctx);
+    for (auto& kv : ctx->live) (void)hipFreeAsync(kv.first, ctx->stream);
+    for (auto& t : ctx->rope_tables) (void)hipFreeAsync(t.cos_sin, ctx->stream);
+    if (ctx->ws) (void)hipFreeAsync(ctx->ws, ctx->stream);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->stage) (void)hipHostFree(ctx->stage);
+    (void)hipEventDestroy(ctx->ev_start);
+    (void)hipEventDestroy(ctx->ev_stop);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return 0;
+}
+
+extern "C" int eisen_hip_stream_sync(eisen_ctx* ctx) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return 0;
+}
+
+extern "C" void* eisen_hip_stream(eisen_ctx* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
+
+extern "C" int eisen_hip_malloc(eisen_ctx* ctx, size_t bytes, void** out) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, out != nullptr, EISEN_E_ARG, "eisen_hip_malloc: out is null");
+    if (bytes == 0) bytes = 4;
+    bytes = (bytes + 255) & ~size_t(255);  // 256-byte granules keep every block 16-byte aligned
+    void* p = nullptr;
+    auto it = ctx->free_lists.find(bytes);
+    if (it != ctx->free_lists.end() && !it->second.empty()) {
+        p = it->second.back();
+        it->second.pop_back();
+        ctx->cached_bytes -= bytes;
+    } else {
+        hipError_t e = hipMallocAsync(&p, bytes, ctx->stream);
+        if (e != hipSuccess) {
+            // out of memory: give cached blocks back and retry once
+            (void)hipGetLastError();
+            (void)eisen_hip_pool_trim(ctx);
+            (void)hipStreamSynchronize(ctx->stream);
+            e = hipMallocAsync(&p, bytes, ctx->stream);
+            if (e != hipSuccess)
+                return eisen_set_error(ctx, (int)e, "hipMallocAsync(%zu bytes) failed: %s", bytes,
+                                       hipGetErrorString(e));
+        }
+    }
+    ctx->live[p] = bytes;
+    ctx->in_use_bytes += bytes;
+    *out = p;
+    return 0;
+}
+
+extern "C" int eisen_hip_malloc_zeroed(eisen_ctx* ctx, size_t bytes, void** out) {
+    int rc = eisen_hip_malloc(ctx, bytes, out);
+    if (rc) return rc;
+    EISEN_HIP_TRY(ctx, hipMemsetAsync(*out, 0, ctx->live[*out], ctx->stream));
+    return 0;
+}
+
+extern "C" int eisen_hip_free(eisen_ctx* ctx, void* ptr) {
+    EISEN_CHECK_CTX(ctx);
+    if (!ptr) return 0;
+    auto it = ctx->live.find(ptr);
+    EISEN_REQUIRE(ctx, it != ctx->live.end(), EISEN_E_ARG, "eisen_hip_free: %p was not allocated by this context", ptr);
+    const size_t bytes = it->second;
+    ctx->live.erase(it);
+    ctx->in_use_bytes -= bytes;
+    ctx->free_lists[bytes].push_back(ptr);
+    ctx->cached_bytes += bytes;
+    return 0;
+}
+
+extern "C" int eisen_hip_mem_info(eisen_ctx* ctx, size_t* free_bytes, size_t* total_bytes) {
+    EISEN_CHECK_CTX(ctx);
+    size_t f = 0, t = 0;
+    EISEN_HIP_TRY(ctx, hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return 0;
+}
+
+extern "C" int eisen_hip_pool_stats(eisen_ctx* ctx, size_t* in_use_bytes, size_t* cached_bytes) {
+    EISEN_CHECK_CTX(ctx);
+    if (in_use_bytes) *in_use_bytes = ctx->in_use_bytes;
+    if (cached_bytes) *cached_bytes = ctx->cached_bytes;
+    return 0;
+}
+
+int eisen_workspace(eisen_ctx* ctx, size_t bytes, void** out) {
+    if (bytes > ctx->ws_bytes) {
+        // stream order makes the old block safe to free while earlier kernels still read it
+        if (ctx->ws) EISEN_HIP_TRY(ctx, hipFreeAsync(ctx->ws, ctx->stream));
+        ctx->ws = nullptr;
+        ctx->ws_bytes = 0;
+        size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        hipError_t e = hipMallocAsync(&ctx->ws, want, ctx->stream);
+        if (e != hipSuccess)
+            return eisen_set_error(ctx, EISEN_E_NOMEM, "workspace of %zu bytes: %s", want, hipGetErrorString(e));
+        ctx->ws_bytes = want;
+    }
+    *out = ctx->ws;
+    return 0;
+}
+
+int eisen_staging(eisen_ctx* ctx, size_t bytes, void** out) {
+    // an earlier asynchronous upload may still be reading the staging buffer
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    if (bytes > ctx->stage_bytes) {
+        if (ctx->stage) EISEN_HIP_TRY(ctx, hipHostFree(ctx->stage));
+        ctx->stage = nullptr;
+        ctx->stage_bytes = 0;
+        size_t want = (bytes + (size_t(1) << 16) - 1) & ~((size_t(1) << 16) - 1);
+        EISEN_HIP_TRY(ctx, hipHostMalloc(&ctx->stage, want, hipHostMallocDefault));
+        ctx->stage_bytes = want;
+    }
+    *out = ctx->stage;
+    return 0;
+}
+
+static constexpr size_t kStageLimit = size_t(8) << 20;
+
+extern "C" int eisen_hip_htod(eisen_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, dst && src, EISEN_E_ARG, "eisen_hip_htod: null pointer");
+    if (bytes == 0) return 0;
+    if (bytes <= kStageLimit) {
+        // small uploads (token ids, targets, tables) go through pinned staging and stay asynchronous
+        void* st = nullptr;
+        if (bytes > ctx->stage_bytes || true) {
+            int rc = eisen_staging(ctx, bytes, &st);
+            if (rc) return rc;
+        }
+        memcpy(st, src, bytes);
+        EISEN_HIP_TRY(ctx, hipMemcpyAsync(dst, st, bytes, hipMemcpyHostToDevice, ctx->stream));
+        return 0;
+    }
+    EISEN_HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return 0;
+}
+
+extern "C" int eisen_hip_dtoh(eisen_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, dst && src, EISEN_E_ARG, "eisen_hip_dtoh: null pointer");
+    if (bytes == 0) return 0;
+    EISEN_HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return 0;
+}
+
+extern "C" int eisen_hip_dtod(eisen_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, dst && src, EISEN_E_ARG, "eisen_hip_dtod: null pointer");
+    if (bytes == 0) return 0;
+    EISEN_HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return 0;
+}
+
+extern "C" int eisen_hip_memset_zero(eisen_ctx* ctx, void* dst, size_t bytes) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, dst != nullptr, EISEN_E_ARG, "eisen_hip_memset_zero: null pointer");
+    if (bytes == 0) return 0;
+    EISEN_HIP_TRY(ctx, hipMemsetAsync(dst, 0, bytes, ctx->stream));
+    return 0;
+}
+
+extern "C" int eisen_hip_module_load(eisen_ctx* ctx, const void* image, size_t len, eisen_module** out) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, image && len && out, EISEN_E_ARG, "eisen_hip_module_load: null image or out");
+    hipModule_t mod;
+    EISEN_HIP_TRY(ctx, hipModuleLoadData(&mod, image));
+    *out = new eisen_module{mod};
+    return 0;
+}
+
+extern "C" int eisen_hip_module_unload(eisen_ctx* ctx, eisen_module* mod) {
+    EISEN_CHECK_CTX(ctx);
+    if (!mod) return 0;
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    EISEN_HIP_TRY(ctx, hipModuleUnload(mod->mod));
+    delete mod;
+    return 0;
+}
+
+extern "C" int eisen_hip_get_function(eisen_ctx* ctx, eisen_module* mod, const char* name, eisen_function** out) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, mod && name && out, EISEN_E_ARG, "eisen_hip_get_function: null argument");
+    hipFunction_t fn;
+    hipError_t e = hipModuleGetFunction(&fn, mod->mod, name);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return eisen_set_error(ctx, (int)e, "kernel '%s' not found in module: %s", name, hipGetErrorString(e));
+    }
+    *out = new eisen_function{fn};  // lives as long as the process; a handful per module
+    return 0;
+}
+
+extern "C" int eisen_hip_launch(eisen_ctx* ctx, eisen_function* fn, const unsigned grid[3], const unsigned block[3],
+                                unsigned shared_bytes, void** args) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, fn && grid && block, EISEN_E_ARG, "eisen_hip_launch: null argument");
+    EISEN_REQUIRE(ctx, grid[0] && grid[1] && grid[2] && block[0] && block[1] && block[2], EISEN_E_ARG,
+                  "eisen_hip_launch: zero grid or block dimension");
+    EISEN_REQUIRE(ctx, (size_t)block[0] * block[1] * block[2] <= 1024, EISEN_E_SHAPE,
+                  "eisen_hip_launch: more than 1024 threads per block");
+    EISEN_HIP_TRY(ctx, hipModuleLaunchKernel(fn->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                             shared_bytes, ctx->stream, args, nullptr));
+    return 0;
+}
+
+extern "C" int eisen_hip_timer_start(eisen_ctx* ctx) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_HIP_TRY(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+    ctx->timer_running = true;
+    return 0;
+}
+
+extern "C" int eisen_hip_timer_stop(eisen_ctx* ctx, float* ms_out) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, ctx->timer_running, EISEN_E_STATE, "eisen_hip_timer_stop without eisen_hip_timer_start");
+    EISEN_HIP_TRY(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
+    EISEN_HIP_TRY(ctx, hipEventSynchronize(ctx->ev_stop));
+    float ms = 0.f;
+    EISEN_HIP_TRY(ctx, hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop));
+    ctx->timer_running = false;
+    if (ms_out) *ms_out = ms;
+    return 0;
+}

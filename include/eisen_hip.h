@@ -1,0 +1,249 @@
+/*
+ * eisen_hip.h -- C-ABI of libeisen_hip.so, the MI355X (gfx950) device backend for eisen's
+ * training step.
+ *
+ * This is the surface a `Device::Gpu` backend binds over FFI in place of the cudarc driver
+ * calls and the by-name CUDA kernels of the reference.  Plain C: opaque handles, raw device
+ * pointers, sizes; no C++ or torch types.  Every function returns 0 on success, a positive
+ * hipError_t on a HIP failure, or a negative EISEN_E_* code on an argument error; none of
+ * them aborts.  `eisen_hip_last_error(ctx)` returns the message of the last failure.
+ *
+ * Conventions
+ *   - One context = one device + one HIP stream (the reference is single-stream:
+ *     src/tensor.rs:18-22 `Device::Gpu(ctx, stream)`).  Every op is enqueued on that stream
+ *     and returns without synchronising unless stated.
+ *   - `dtype` arguments take EISEN_F32 or EISEN_BF16 and name the element type of the
+ *     activation buffers of the call.  Parameter gradients, norm gains, moments and master
+ *     weights are always f32.
+ *   - `accumulate` != 0 means `dst += value` (the reference's backward semantics,
+ *     every backward_fn adds into `.grad`), 0 means `dst = value` (first writer of a
+ *     gradient buffer; saves the zero-fill and the read).
+ *   - Matrices are row-major and contiguous; linear weights are [in, out]
+ *     (src/nn/linear.rs:40).
+ */
+#ifndef EISEN_HIP_H
+#define EISEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct eisen_ctx eisen_ctx;
+typedef struct eisen_module eisen_module;
+typedef struct eisen_function eisen_function;
+
+enum { EISEN_F32 = 0, EISEN_BF16 = 1 };
+
+enum {
+    EISEN_E_ARG = -1,      /* null pointer, zero/negative size, unknown dtype */
+    EISEN_E_SHAPE = -2,    /* shape the kernel family does not support (message says which) */
+    EISEN_E_ALIGN = -3,    /* pointer or row pitch not aligned as the kernel needs */
+    EISEN_E_NOMEM = -4,    /* workspace could not be allocated */
+    EISEN_E_STATE = -5     /* call order violated (e.g. timer stop without start) */
+};
+
+#define EISEN_IGNORE_INDEX (-1) /* target id of a masked row (reference: usize::MAX, src/data/fim.rs:173) */
+
+/* ---- runtime: replaces the cudarc calls counted at src/graph/mod.rs:152-307 ------------- */
+
+/* CudaContext::new(0) + ctx.default_stream() (tests/gpu_kernels.rs:6-14, src/main.rs:9-11). */
+int eisen_hip_init(int device, eisen_ctx** out);
+int eisen_hip_destroy(eisen_ctx* ctx);
+const char* eisen_hip_last_error(eisen_ctx* ctx);
+/* stream.synchronize() (e.g. src/graph/mod.rs:776-788). */
+int eisen_hip_stream_sync(eisen_ctx* ctx);
+/* The hipStream_t of the context, as void*, for callers that enqueue their own work. */
+void* eisen_hip_stream(eisen_ctx* ctx);
+
+/* stream.alloc_zeros / Graph::safe_alloc_zeros (src/graph/memory.rs:189-266) and the
+ * size-keyed vram_pool in front of it (src/graph/mod.rs:437-556).  Stream-ordered:
+ * a freed block may be handed out again to a later call on the same stream. */
+int eisen_hip_malloc(eisen_ctx* ctx, size_t bytes, void** out);
+int eisen_hip_malloc_zeroed(eisen_ctx* ctx, size_t bytes, void** out);
+int eisen_hip_free(eisen_ctx* ctx, void* ptr);
+/* Drop every cached block back to the driver (the OOM fallback's "clear pools" step). */
+int eisen_hip_pool_trim(eisen_ctx* ctx);
+/* ctx.mem_get_info() (src/graph/memory.rs:429-470). */
+int eisen_hip_mem_info(eisen_ctx* ctx, size_t* free_bytes, size_t* total_bytes);
+/* Bytes currently handed out / cached by the pool (diagnostics, tests). */
+int eisen_hip_pool_stats(eisen_ctx* ctx, size_t* in_use_bytes, size_t* cached_bytes);
+
+/* stream.memcpy_htod / clone_htod (src/graph/mod.rs:368-430, src/tensor.rs:156-160):
+ * asynchronous on the stream; the host buffer is copied to a staging area first, so it may
+ * be reused as soon as the call returns. */
+int eisen_hip_htod(eisen_ctx* ctx, void* dst_device, const void* src_host, size_t bytes);
+/* stream.clone_dtoh (src/tensor.rs:177-223): synchronises the stream before returning. */
+int eisen_hip_dtoh(eisen_ctx* ctx, void* dst_host, const void* src_device, size_t bytes);
+int eisen_hip_dtod(eisen_ctx* ctx, void* dst_device, const void* src_device, size_t bytes);
+int eisen_hip_memset_zero(eisen_ctx* ctx, void* dst_device, size_t bytes);
+
+/* ctx.load_module(ptx) / module.load_function(name) / stream.launch_builder(f)...launch(cfg)
+ * (src/graph/mod.rs:155-266; e.g. src/graph/ops/normalization.rs:47-88).  `image` is a
+ * gfx950 code object (hipcc --genco).  `args` follows hipModuleLaunchKernel: an array of
+ * pointers to the argument values, in order. */
+int eisen_hip_module_load(eisen_ctx* ctx, const void* image, size_t len, eisen_module** out);
+int eisen_hip_module_unload(eisen_ctx* ctx, eisen_module* mod);
+int eisen_hip_get_function(eisen_ctx* ctx, eisen_module* mod, const char* name, eisen_function** out);
+int eisen_hip_launch(eisen_ctx* ctx, eisen_function* fn, const unsigned grid[3], const unsigned block[3],
+                     unsigned shared_bytes, void** args);
+
+/* HIP-event stopwatch on the context's stream (the reference only has host Instant timers,
+ * examples/train_llm.rs:484-496).  stop() synchronises and returns milliseconds. */
+int eisen_hip_timer_start(eisen_ctx* ctx);
+int eisen_hip_timer_stop(eisen_ctx* ctx, float* ms_out);
+
+/* ---- elementwise ---------------------------------------------------------------------- */
+
+/* fill_f32 / scale_f32 (kernels/ops_f32.cu:101,107; callers src/graph/mod.rs:683-693,
+ * src/nn/optim.rs:183-192,224-235). */
+int eisen_hip_fill(eisen_ctx* ctx, void* dst, int dtype, float value, size_t n);
+int eisen_hip_scale(eisen_ctx* ctx, void* dst, int dtype, float factor, size_t n);
+/* dst *= *factor_device (factor read on the device: no host round trip). */
+int eisen_hip_scale_by_device_scalar(eisen_ctx* ctx, void* dst, int dtype, const float* factor_device, size_t n);
+/* cast_f32_to_bf16 / cast_bf16_to_f32 (kernels/ops_bf16.cu:4,11), round-to-nearest-even. */
+int eisen_hip_cast(eisen_ctx* ctx, const void* src, int src_dtype, void* dst, int dst_dtype, size_t n);
+/* accumulate_f32 without broadcast (kernels/ops_f32.cu:84; add/reshape/copy backward,
+ * src/graph/ops/elementwise.rs:116-137, transform.rs:365-380): dst (+)= src. */
+int eisen_hip_accumulate(eisen_ctx* ctx, void* dst, const void* src, int dtype, size_t n, int accumulate);
+/* add_f32 / mul_f32 same-shape fast path (kernels/ops_f32.cu:66,113). */
+int eisen_hip_add(eisen_ctx* ctx, const void* a, const void* b, void* out, int dtype, size_t n);
+int eisen_hip_mul(eisen_ctx* ctx, const void* a, const void* b, void* out, int dtype, size_t n);
+/* Broadcasting add/mul, rank <= 4 (Graph::add / Graph::mul, src/graph/ops/elementwise.rs:15-145,
+ * :188-293).  out_shape has `rank` entries; a_strides/b_strides are element strides in the
+ * broadcast shape (0 on broadcast dims, src/tensor.rs:249-263). */
+int eisen_hip_add_bcast(eisen_ctx* ctx, const void* a, const void* b, void* out, int dtype, int rank,
+                        const size_t* out_shape, const size_t* a_strides, const size_t* b_strides);
+int eisen_hip_mul_bcast(eisen_ctx* ctx, const void* a, const void* b, void* out, int dtype, int rank,
+                        const size_t* out_shape, const size_t* a_strides, const size_t* b_strides);
+/* Backward of a broadcast operand: dst[bcast_idx(i)] += src[i] * (mul ? other[other_idx(i)] : 1),
+ * reduced deterministically (one thread owns one dst element and walks its sources in
+ * ascending i) -- replaces accumulate_f32's atomicAdd (kernels/ops_f32.cu:84-99). */
+int eisen_hip_bcast_backward(eisen_ctx* ctx, void* dst, const void* grad_out, const void* other, int dtype,
+                             int rank, const size_t* out_shape, const size_t* dst_strides,
+                             const size_t* other_strides, size_t dst_numel, int accumulate);
+/* mul_backward_f32 same-shape (kernels/ops_f32.cu:119): ga (+)= b*go, gb (+)= a*go.
+ * ga or gb may be NULL (constant operand). */
+int eisen_hip_mul_backward(eisen_ctx* ctx, const void* a, const void* b, const void* go, void* ga, void* gb,
+                           int dtype, size_t n, int accumulate_a, int accumulate_b);
+/* silu_f32 / silu_backward_f32 (kernels/ops_f32.cu:135,142; src/graph/ops/elementwise.rs:337-465). */
+int eisen_hip_silu(eisen_ctx* ctx, const void* x, void* out, int dtype, size_t n);
+int eisen_hip_silu_backward(eisen_ctx* ctx, const void* x, const void* go, void* gx, int dtype, size_t n,
+                            int accumulate);
+/* Fused silu(gate)*up and its backward: the gate/silu/up/mul chain of
+ * TransformerBlock::forward_with_mask (src/nn/transformer.rs:40-43) in one pass each way. */
+int eisen_hip_swiglu(eisen_ctx* ctx, const void* gate, const void* up, void* out, int dtype, size_t n);
+int eisen_hip_swiglu_backward(eisen_ctx* ctx, const void* gate, const void* up, const void* go, void* dgate,
+                              void* dup, int dtype, size_t n, int accumulate_gate, int accumulate_up);
+
+/* ---- normalisation, rotary, layout ----------------------------------------------------- */
+
+/* rmsnorm_f32 / rmsnorm_backward_f32 (kernels/ops_f32.cu:539-578; Graph::rms_norm,
+ * src/graph/ops/normalization.rs:8-184).  w, rrms, gw are f32.  rrms [rows] is written by the
+ * forward and read by the backward.  gw += sum over rows (two-stage, fixed order, no atomics). */
+int eisen_hip_rms_norm(eisen_ctx* ctx, const void* x, const float* w, void* out, float* rrms, int dtype,
+                       size_t rows, size_t dim, float eps);
+int eisen_hip_rms_norm_backward(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go,
+                                void* gx, float* gw, int dtype, size_t rows, size_t dim, int accumulate_x);
+/* rope_f32 / rope_backward_f32 (kernels/ops_f32.cu:724-760; Graph::rope,
+ * src/graph/ops/transform.rs:467-610): x [batch, seq, hidden], interleaved pairs within each
+ * head of `head_dim`, base 10000, position = index along dim 1. */
+int eisen_hip_rope(eisen_ctx* ctx, const void* x, void* out, int dtype, size_t batch, size_t seq, size_t hidden,
+                   size_t head_dim);
+int eisen_hip_rope_backward(eisen_ctx* ctx, const void* go, void* gx, int dtype, size_t batch, size_t seq,
+                            size_t hidden, size_t head_dim, int accumulate);
+/* transpose_0213_f32 / _backward (kernels/ops_f32.cu:694,709; src/graph/ops/transform.rs:7-127):
+ * [b, s, h, d] -> [b, h, s, d]; the backward is the same permutation applied to the grad. */
+int eisen_hip_transpose_0213(eisen_ctx* ctx, const void* in, void* out, int dtype, size_t b, size_t s, size_t h,
+                             size_t d, int accumulate);
+/* repeat_kv_f32 / _backward (kernels/ops_f32.cu:787-838; src/graph/ops/gqa.rs:13-194). */
+int eisen_hip_repeat_kv(eisen_ctx* ctx, const void* in, void* out, int dtype, size_t batch, size_t kv_heads,
+                        size_t seq, size_t head_dim, size_t repeats);
+int eisen_hip_repeat_kv_backward(eisen_ctx* ctx, const void* go, void* gin, int dtype, size_t batch,
+                                 size_t kv_heads, size_t seq, size_t head_dim, size_t repeats, int accumulate);
+/* softmax_f32 / softmax_backward_f32 over the last dim (kernels/ops_f32.cu:625,636;
+ * src/graph/ops/reduction.rs:397-523). */
+int eisen_hip_softmax(eisen_ctx* ctx, const void* x, void* out, int dtype, size_t rows, size_t n);
+int eisen_hip_softmax_backward(eisen_ctx* ctx, const void* out, const void* go, void* gx, int dtype, size_t rows,
+                               size_t n, int accumulate);
+
+/* ---- contractions ---------------------------------------------------------------------- */
+
+/* C[M,N] (+)= op(A) * op(B), row-major.  op(A) = A stored [M,K], or A stored [K,M] when
+ * trans_a; op(B) = B stored [K,N], or B stored [N,K] when trans_b.  Covers
+ *   Graph::matmul forward (matmul_f32 / matmul_bf16_f32, kernels/ops_f32.cu:158, ops_bf16.cu:26;
+ *     src/graph/ops/linear.rs:35-263):                       trans_a=0, trans_b=0
+ *   dX = dY * W^T (matmul_backward_a_f32, ops_f32.cu:192; linear.rs:266-277):  trans_b=1
+ *   dW += X^T * dY (matmul_backward_b_f32, ops_f32.cu:225; linear.rs:278-287): trans_a=1, accumulate=1
+ *   tied lm_head (matmul_trans_b_f32 / matmul_trans_a_f32, ops_f32.cu:842-882; linear.rs:301-517).
+ * dtype_ab: element type of A and B; dtype_c: element type of C (f32 operands need f32 C).
+ * bf16 operands run on MFMA with f32 accumulation; f32 operands on an FMA kernel. */
+int eisen_hip_gemm(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
+                   int trans_b, size_t M, size_t N, size_t K, int accumulate);
+/* Batched form with contiguous batches (bmm_f32 and its four backward kernels,
+ * kernels/ops_f32.cu:342-510; Graph::bmm, src/graph/ops/linear.rs:1198-1511). */
+int eisen_hip_bmm(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
+                  int trans_b, size_t batch, size_t M, size_t N, size_t K, int accumulate);
+
+/* ---- embedding ------------------------------------------------------------------------- */
+
+/* gather_f32 (kernels/ops_f32.cu:513; Graph::gather, src/graph/ops/transform.rs:132-324).
+ * ids are int32 on the device (the reference stores them as f32 and casts, :294). */
+int eisen_hip_gather(eisen_ctx* ctx, const void* weight, const int32_t* ids, void* out, int dtype, size_t n_ids,
+                     size_t vocab, size_t hidden);
+/* Embedding-gradient scatter, deterministic (replaces gather_backward_f32's atomicAdd,
+ * kernels/ops_f32.cu:526-537).  gw[ids[i], :] += go[i, :], every row receiving its addends
+ * in ascending i exactly like the CPU arm (src/graph/ops/transform.rs:306-315).
+ * `ids_host` is the host copy of the ids (they originate on the host in every caller,
+ * examples/train_llm.rs:433-435); the call builds a stable position index from it. */
+int eisen_hip_gather_backward(eisen_ctx* ctx, const int32_t* ids_host, const void* go, float* gw, int dtype,
+                              size_t n_ids, size_t vocab, size_t hidden);
+
+/* ---- loss ------------------------------------------------------------------------------ */
+
+/* Fused softmax-cross-entropy forward+backward in one pass over the logits
+ * (cross_entropy_f32 + cross_entropy_backward_f32, kernels/ops_f32.cu:580-623, and the masked
+ * pair :5-64; Graph::cross_entropy / cross_entropy_masked, src/graph/ops/reduction.rs:529-944).
+ *   loss_out[0] = normalizer * sum_rows -ln(p_target + 1e-8)      (rows with target -1 skipped)
+ *   dlogits     = (p - onehot(target)) * normalizer * grad_scale  (zero for skipped rows)
+ * normalizer = 1/rows, or 1/valid_rows when any target is EISEN_IGNORE_INDEX.
+ * targets: int32 on the device.  row_loss [rows] f32 scratch owned by the caller.
+ * argmax_out (int32 [rows]) and target_logit_out (f32 [rows]) may be NULL; when given they
+ * receive the first index of the row maximum and the logit at the target (0 for skipped rows). */
+int eisen_hip_cross_entropy(eisen_ctx* ctx, const void* logits, const int32_t* targets, void* dlogits,
+                            float* row_loss, float* loss_out, int32_t* argmax_out, float* target_logit_out,
+                            int dtype, size_t rows, size_t classes, float normalizer, float grad_scale);
+
+/* ---- optimiser ------------------------------------------------------------------------- */
+
+/* One parameter tensor of a fused multi-tensor optimiser call. */
+typedef struct {
+    float* w;          /* f32 master weight */
+    const float* g;    /* f32 gradient */
+    float* m;          /* f32 first moment */
+    float* v;          /* f32 second moment */
+    void* w_bf16;      /* optional bf16 copy of the updated weight (NULL: none) */
+    size_t n;          /* elements */
+} eisen_param_slot;
+
+/* adamw_step_f32 (kernels/ops_f32.cu:762-784; AdamW::step, src/nn/optim.rs:334-562) over all
+ * tensors in one launch.  bc1/bc2 are the reciprocal bias corrections 1/(1-beta^t) computed
+ * by the caller (src/nn/optim.rs:336-338).  grad_scale_device: optional device f32 the
+ * gradient is multiplied with first (the clip coefficient); NULL = 1. */
+int eisen_hip_adamw_step(eisen_ctx* ctx, const eisen_param_slot* slots, size_t n_slots, float lr, float beta1,
+                         float beta2, float eps, float weight_decay, float bc1, float bc2,
+                         const float* grad_scale_device);
+/* AdamW::clip_grad_norm without the D2H of every gradient (src/nn/optim.rs:250-321):
+ * out_device[0] = sqrt(sum g^2) with f64 accumulation, out_device[1] = clip coefficient
+ * min(1, max_norm/(norm+1e-6)) (1 when norm == 0).  Deterministic two-stage reduction. */
+int eisen_hip_grad_norm(eisen_ctx* ctx, const eisen_param_slot* slots, size_t n_slots, float max_norm,
+                        float* out_device);
+/* AdamW::zero_grad over all tensors in one launch (src/nn/optim.rs:207-245). */
+int eisen_hip_zero_grads(eisen_ctx* ctx, const eisen_param_slot* slots, size_t n_slots);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EISEN_HIP_H */

@@ -1,0 +1,48 @@
+"""Helpers for the GPU parity tests: a session Context and tolerance checks.
+
+Tolerances (stated once, used by every GPU test):
+  f32 kernels   : |a - e| <= 1e-4 * |e| + 1e-4 * rms(e)      ("rtol 1e-4", near-zero elements measured
+                  against the tensor's RMS instead of their own magnitude)
+  bf16 kernels  : |a - e| <= 2e-2 * |e| + 2e-2 * rms(e)      ("rtol 2e-2 on gradients")
+  integer/index : bit-exact
+"""
+import numpy as np
+import pytest
+
+RTOL_F32 = 1e-4
+RTOL_BF16 = 2e-2
+
+
+@pytest.fixture(scope="session")
+def ctx():
+    from eisen_amd import hip
+    c = hip.Context(0)
+    yield c
+    c.close()
+
+
+def assert_close(actual, expected, rtol, name=""):
+    a = np.asarray(actual, np.float64).reshape(-1)
+    e = np.asarray(expected, np.float64).reshape(-1)
+    assert a.shape == e.shape, f"{name}: shape {a.shape} vs {e.shape}"
+    assert np.isfinite(a).all(), f"{name}: non-finite values in the result"
+    rms = float(np.sqrt(np.mean(e * e))) if e.size else 0.0
+    tol = rtol * np.abs(e) + rtol * rms + 1e-30
+    err = np.abs(a - e)
+    bad = err > tol
+    if bad.any():
+        i = int(np.argmax(err / tol))
+        raise AssertionError(f"{name}: {int(bad.sum())}/{a.size} elements outside rtol {rtol:g}; worst at {i}: "
+                             f"got {a[i]:.8g}, expected {e[i]:.8g}, rms {rms:.4g}")
+
+
+def tol_for(dtype):
+    from eisen_amd import hip
+    return RTOL_BF16 if dtype == hip.BF16 else RTOL_F32
+
+
+def prep(x, dtype):
+    """Input as the device will see it: bf16 inputs are rounded first so oracle and GPU start equal."""
+    from eisen_amd import hip
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    return hip.round_bf16(x) if dtype == hip.BF16 else x

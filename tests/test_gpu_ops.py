@@ -1,0 +1,557 @@
+"""GPU parity tests: every C-ABI op against the CPU oracle on the same seeded inputs.
+
+Run on an MI355X with `pytest -m gpu`.  All calls go through libeisen_hip.so's C-ABI
+(eisen_amd.hip is a ctypes mirror of include/eisen_hip.h); the oracle is only the checker.
+"""
+import numpy as np
+import pytest
+
+from eisen_amd import hip
+from oracle import cpu_ref as R
+from tests import gen
+from tests.gpu_util import assert_close, ctx, prep, tol_for  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+F32, BF16 = hip.F32, hip.BF16
+DTYPES = [F32, BF16]
+_ids = {F32: "f32", BF16: "bf16"}
+
+
+def up(ctx, x, dtype):
+    return ctx.upload(x, dtype)
+
+
+def dn(ctx, buf, shape, dtype):
+    return ctx.download(buf, tuple(shape), dtype)
+
+
+# ---------------------------------------------------------------------------
+# runtime
+# ---------------------------------------------------------------------------
+
+def test_runtime_roundtrip_pool_and_errors(ctx):
+    x = gen.normal(1, (1000,))
+    b = ctx.upload(x)
+    assert np.array_equal(ctx.download(b, (1000,)), x)
+    in_use0, _ = ctx.pool_stats()
+    b.free()
+    in_use1, cached1 = ctx.pool_stats()
+    assert in_use1 == in_use0 - 4096 and cached1 >= 4096      # 256-byte granules: 4000 -> 4096
+    b2 = ctx.malloc(4000, zero=True)                           # same bucket comes back, zero-filled
+    assert not ctx.download(b2, (1000,)).any()
+    free, total = ctx.mem_info()
+    assert 0 < free <= total and total > 200 * 2 ** 30          # 288 GB part
+    with pytest.raises(hip.EisenHipError):
+        ctx.fill(None, F32, 1.0, 10)
+    with pytest.raises(hip.EisenHipError):
+        ctx.rope(b2, b2, BF16, 1, 4, 12, 6)                    # head_dim 6 is not a packet multiple
+    big = gen.normal(2, (5 * 2 ** 20,))                        # > staging limit: direct copy path
+    bb = ctx.upload(big)
+    assert np.array_equal(ctx.download(bb, big.shape), big)
+    bb.free()
+    b2.free()
+    ctx.timer_start()
+    ms = ctx.timer_stop()
+    assert ms >= 0.0
+
+
+def test_module_load_and_launch_by_name(ctx):
+    """The reference's load_module / load_function / launch_builder path (src/graph/mod.rs:155-266)."""
+    import ctypes as C
+    mod = ctx.module_load()
+    fill = ctx.get_function(mod, "fill_f32")
+    scale = ctx.get_function(mod, "scale_f32")
+    cast = ctx.get_function(mod, "cast_f32_to_bf16")
+    n = 5000
+    buf = ctx.malloc(n * 4)
+    ctx.launch(fill, (8, 1, 1), (256, 1, 1), [C.c_void_p(buf.ptr), C.c_float(2.5), C.c_size_t(n)])
+    ctx.launch(scale, (8, 1, 1), (256, 1, 1), [C.c_void_p(buf.ptr), C.c_float(-2.0), C.c_size_t(n)])
+    assert np.array_equal(ctx.download(buf, (n,)), np.full(n, -5.0, np.float32))
+    x = gen.normal(3, (n,), 10.0)
+    src = ctx.upload(x)
+    dst = ctx.malloc(n * 2)
+    ctx.launch(cast, (8, 1, 1), (256, 1, 1), [C.c_void_p(src.ptr), C.c_void_p(dst.ptr), C.c_size_t(n)])
+    assert np.array_equal(ctx.download(dst, (n,), BF16), hip.round_bf16(x))     # device cast is RNE, bit-exact
+    with pytest.raises(hip.EisenHipError):
+        ctx.get_function(mod, "no_such_kernel")
+    ctx.module_unload(mod)
+
+
+# ---------------------------------------------------------------------------
+# elementwise
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+def test_fill_scale_cast_accumulate(ctx, n):
+    x = gen.normal(4, (n,), 3.0)
+    for dtype in DTYPES:
+        b = ctx.malloc(n * 4)
+        ctx.fill(b, dtype, 1.25, n)
+        ctx.scale(b, dtype, 3.0, n)
+        assert np.array_equal(dn(ctx, b, (n,), dtype), np.full(n, 3.75, np.float32))
+        b.free()
+    src = ctx.upload(x)
+    bf = ctx.malloc(n * 2)
+    back = ctx.malloc(n * 4)
+    ctx.cast(src, F32, bf, BF16, n)
+    ctx.cast(bf, BF16, back, F32, n)
+    assert np.array_equal(dn(ctx, bf, (n,), BF16), hip.round_bf16(x))
+    assert np.array_equal(dn(ctx, back, (n,), F32), hip.round_bf16(x))
+    y = gen.normal(5, (n,))
+    dst = ctx.upload(y)
+    ctx.accumulate(dst, src, F32, n, 1)
+    assert np.array_equal(dn(ctx, dst, (n,), F32), y + x)
+    ctx.accumulate(dst, src, F32, n, 0)
+    assert np.array_equal(dn(ctx, dst, (n,), F32), x)
+    one = ctx.upload(np.array([0.5], np.float32))
+    ctx.scale_by_device_scalar(dst, F32, one, n)
+    assert np.array_equal(dn(ctx, dst, (n,), F32), x * np.float32(0.5))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+def test_add_mul_silu_swiglu(ctx, dtype):
+    n = 3 * 1024 + 5
+    a, b, go = prep(gen.normal(6, (n,), 2.0), dtype), prep(gen.normal(7, (n,), 2.0), dtype), prep(gen.normal(8, (n,)), dtype)
+    da, db, dgo = up(ctx, a, dtype), up(ctx, b, dtype), up(ctx, go, dtype)
+    out = ctx.malloc(n * 4)
+    tol = tol_for(dtype)
+    ctx.add(da, db, out, dtype, n)
+    assert_close(dn(ctx, out, (n,), dtype), a + b, tol, "add")
+    ctx.mul(da, db, out, dtype, n)
+    assert_close(dn(ctx, out, (n,), dtype), a * b, tol, "mul")
+    ga, gb = ctx.malloc(n * 4), ctx.malloc(n * 4)
+    ctx.mul_backward(da, db, dgo, ga, gb, dtype, n)
+    assert_close(dn(ctx, ga, (n,), dtype), b * go, tol, "mul_bwd a")
+    assert_close(dn(ctx, gb, (n,), dtype), a * go, tol, "mul_bwd b")
+    ctx.mul_backward(da, db, dgo, ga, None, dtype, n, acc_a=1)          # constant operand, accumulate
+    assert_close(dn(ctx, ga, (n,), dtype), 2 * b * go, tol, "mul_bwd acc")
+    ctx.silu(da, out, dtype, n)
+    assert_close(dn(ctx, out, (n,), dtype), R.silu_fwd(a), tol, "silu")
+    ctx.silu_backward(da, dgo, out, dtype, n)
+    assert_close(dn(ctx, out, (n,), dtype), R.silu_bwd(a, go), tol, "silu_bwd")
+    # fused SwiGLU == silu -> mul chain of the oracle (src/nn/transformer.rs:40-43)
+    g = R.Graph()
+    gi, ui = g.alloc((n,), a), g.alloc((n,), b)
+    h = g.mul(g.silu(gi), ui)
+    seed = g.alloc((n,), go)
+    g.backward(g.sum(g.mul(h, seed), 0))
+    ctx.swiglu(da, db, out, dtype, n)
+    assert_close(dn(ctx, out, (n,), dtype), g.data(h), tol, "swiglu")
+    ctx.swiglu_backward(da, db, dgo, ga, gb, dtype, n)
+    assert_close(dn(ctx, ga, (n,), dtype), g.grad(gi), tol, "swiglu dgate")
+    assert_close(dn(ctx, gb, (n,), dtype), g.grad(ui), tol, "swiglu dup")
+
+
+def test_broadcast_add_mul_and_backward(ctx):
+    # mask add [1,S,S] onto [BH,S,S] and a [1,3] row onto [2,3] (tests/phase1.rs:14-20)
+    BH, S = 3, 5
+    a, m = gen.normal(9, (BH, S, S)), gen.normal(10, (1, S, S))
+    go = gen.normal(11, (BH, S, S))
+    da, dm, dgo = up(ctx, a, F32), up(ctx, m, F32), up(ctx, go, F32)
+    out = ctx.malloc(a.nbytes)
+    ctx.add_bcast(da, dm, out, F32, (BH, S, S), (S * S, S, 1), (0, S, 1))
+    assert np.array_equal(dn(ctx, out, a.shape, F32), a + m)
+    ctx.mul_bcast(da, dm, out, F32, (BH, S, S), (S * S, S, 1), (0, S, 1))
+    assert np.array_equal(dn(ctx, out, a.shape, F32), a * m)
+    g = R.Graph()
+    ai, mi = g.alloc(a.shape, a), g.alloc(m.shape, m)
+    pr = g.mul(ai, mi)
+    seed = g.alloc(go.shape, go)
+    g.backward(g.sum(g.sum(g.sum(g.mul(pr, seed), 2), 1), 0))
+    gm = ctx.malloc(m.nbytes)
+    ctx.bcast_backward(gm, dgo, da, F32, (BH, S, S), (0, S, 1), (S * S, S, 1), S * S, 0)
+    assert_close(dn(ctx, gm, m.shape, F32), g.grad(mi), 1e-5, "mul bcast bwd")
+    ctx.bcast_backward(gm, dgo, None, F32, (BH, S, S), (0, S, 1), None, S * S, 0)
+    assert_close(dn(ctx, gm, m.shape, F32), go.sum(0, keepdims=True), 1e-5, "add bcast bwd")
+
+
+# ---------------------------------------------------------------------------
+# rmsnorm, rope, softmax, layout
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+@pytest.mark.parametrize("rows,dim", [(2, 4), (64, 64), (37, 256), (130, 2048), (9, 100)])
+def test_rms_norm(ctx, dtype, rows, dim):
+    if rows == 2:   # reference smoke vector (tests/gpu_kernels.rs:219-229)
+        x = prep(np.array([[1, -2, 3, -4], [0.1, 0.2, -0.1, 0.0]], np.float32), dtype)
+    else:
+        x = prep(gen.normal(12, (rows, dim), 1.5), dtype)
+    w = (1.0 + gen.normal(13, (dim,), 0.2)).astype(np.float32)
+    go = prep(gen.normal(14, (rows, dim)), dtype)
+    tol = tol_for(dtype)
+    dx, dw, dgo = up(ctx, x, dtype), up(ctx, w, F32), up(ctx, go, dtype)
+    out, rr = ctx.malloc(x.nbytes), ctx.malloc(rows * 4)
+    ctx.rms_norm(dx, dw, out, rr, dtype, rows, dim, 1e-5)
+    eo, er = R.rms_norm_fwd(x, w, 1e-5)
+    assert_close(dn(ctx, out, x.shape, dtype), eo, tol, "rms fwd")
+    assert_close(dn(ctx, rr, (rows,), F32), er, 1e-5, "rrms")
+    egx, egw = R.rms_norm_bwd(x, w, er, go)
+    gx = ctx.malloc(x.nbytes)
+    gw0 = gen.normal(15, (dim,))
+    gw = ctx.upload(gw0)
+    ctx.rms_norm_backward(dx, dw, rr, dgo, gx, gw, dtype, rows, dim, 0)
+    assert_close(dn(ctx, gx, x.shape, dtype), egx, tol, "rms dx")
+    assert_close(dn(ctx, gw, (dim,), F32) - gw0, egw, tol if dtype == BF16 else 2e-4, "rms dw (+=)")
+    prev = dn(ctx, gx, x.shape, dtype)
+    ctx.rms_norm_backward(dx, dw, rr, dgo, gx, gw, dtype, rows, dim, 1)     # residual fan-in: dx +=
+    assert_close(dn(ctx, gx, x.shape, dtype), 2 * prev, tol, "rms dx +=")
+    # deterministic: a second run gives the same bits
+    gw2 = ctx.upload(gw0)
+    ctx.rms_norm_backward(dx, dw, rr, dgo, gx, gw2, dtype, rows, dim, 0)
+    gw3 = ctx.upload(gw0)
+    ctx.rms_norm_backward(dx, dw, rr, dgo, gx, gw3, dtype, rows, dim, 0)
+    assert np.array_equal(dn(ctx, gw2, (dim,), F32), dn(ctx, gw3, (dim,), F32))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+@pytest.mark.parametrize("b,s,hidden,hd", [(1, 2, 8, 8), (2, 33, 64, 16), (2, 128, 256, 64)])
+def test_rope(ctx, dtype, b, s, hidden, hd):
+    x = prep(gen.normal(16, (b, s, hidden)), dtype)
+    go = prep(gen.normal(17, (b, s, hidden)), dtype)
+    tol = tol_for(dtype)
+    dx, dgo = up(ctx, x, dtype), up(ctx, go, dtype)
+    out = ctx.malloc(x.nbytes)
+    ctx.rope(dx, out, dtype, b, s, hidden, hd)
+    got = dn(ctx, out, x.shape, dtype)
+    assert_close(got, R.rope_fwd(x, hd), tol, "rope fwd")
+    assert np.array_equal(got[:, 0], x[:, 0])                                    # position 0: identity
+    if dtype == F32:   # same angle table and the same two products + one add per output: bit-exact
+        assert np.array_equal(got, R.rope_fwd(x, hd))
+    gx = ctx.malloc(x.nbytes)
+    ctx.rope_backward(dgo, gx, dtype, b, s, hidden, hd, 0)
+    assert_close(dn(ctx, gx, x.shape, dtype), R.rope_bwd(go, hd), tol, "rope bwd")
+    ctx.rope_backward(dgo, gx, dtype, b, s, hidden, hd, 1)
+    assert_close(dn(ctx, gx, x.shape, dtype), 2 * R.rope_bwd(go, hd), tol, "rope bwd +=")
+
+
+def test_rope_reference_vector(ctx):
+    # tests/gpu_kernels.rs:485-513
+    x = np.ones((1, 2, 4), np.float32)
+    dx = up(ctx, x, F32)
+    out = ctx.malloc(x.nbytes)
+    ctx.rope(dx, out, F32, 1, 2, 4, 4)
+    r = dn(ctx, out, (8,), F32)
+    assert r[:4].tolist() == [1.0] * 4
+    assert abs(r[4] - (0.5403 - 0.8414)) < 1e-3 and abs(r[5] - (0.5403 + 0.8414)) < 1e-3
+    ctx.rope_backward(dx, out, F32, 1, 2, 4, 4, 0)
+    r = dn(ctx, out, (8,), F32)
+    assert abs(r[4] - (0.5403 + 0.8414)) < 1e-3 and abs(r[5] - (0.5403 - 0.8414)) < 1e-3
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+def test_softmax(ctx, dtype):
+    rows, n = 37, 133
+    x = prep(gen.normal(18, (rows, n), 3.0), dtype)
+    x[:, 100:] = -1e20 if dtype == F32 else x[:, 100:]                      # masked tail underflows to exactly 0
+    go = prep(gen.normal(19, (rows, n)), dtype)
+    tol = tol_for(dtype)
+    dx, dgo = up(ctx, x, dtype), up(ctx, go, dtype)
+    out = ctx.malloc(x.nbytes)
+    ctx.softmax(dx, out, dtype, rows, n)
+    got = dn(ctx, out, x.shape, dtype)
+    exp = R.softmax_fwd(x)
+    assert_close(got, exp, tol, "softmax")
+    if dtype == F32:
+        assert not got[:, 100:].any()
+    y = prep(exp, dtype)
+    dy = up(ctx, y, dtype)
+    gx = ctx.malloc(x.nbytes)
+    ctx.softmax_backward(dy, dgo, gx, dtype, rows, n, 0)
+    assert_close(dn(ctx, gx, x.shape, dtype), R.softmax_bwd(y, go), tol, "softmax bwd")
+    # reference vector: softmax([2,0]) = [0.88079, 0.11920] (tests/gpu_kernels.rs:374-376)
+    d2 = up(ctx, np.array([[2.0, 0.0]], np.float32), F32)
+    ctx.softmax(d2, out, F32, 1, 2)
+    p = dn(ctx, out, (2,), F32)
+    assert abs(p[0] - 0.88079) < 1e-4 and abs(p[1] - 0.11920) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+def test_transpose_0213_and_repeat_kv_bit_exact(ctx, dtype):
+    b, s, h, d = 2, 9, 4, 16
+    x = prep(gen.normal(20, (b, s, h, d)), dtype)
+    dx = up(ctx, x, dtype)
+    out = ctx.malloc(x.nbytes)
+    ctx.transpose_0213(dx, out, dtype, b, s, h, d, 0)
+    assert np.array_equal(dn(ctx, out, (b, h, s, d), dtype), R.transpose_0213_fwd(x))
+    back = ctx.malloc(x.nbytes)
+    ctx.transpose_0213(out, back, dtype, b, h, s, d, 0)                         # backward = inverse permutation
+    assert np.array_equal(dn(ctx, back, x.shape, dtype), x)
+    ctx.transpose_0213(dx, out, F32, 1, 3, 2, 3, 0) if dtype == F32 else None   # odd d: scalar path
+    kv, rep = 2, 3
+    k = prep(gen.normal(21, (b, kv, s, d)), dtype)
+    dk = up(ctx, k, dtype)
+    rk = ctx.malloc(k.nbytes * rep)
+    ctx.repeat_kv(dk, rk, dtype, b, kv, s, d, rep)
+    assert np.array_equal(dn(ctx, rk, (b, kv * rep, s, d), dtype), R.repeat_kv_fwd(k, rep))
+    go = prep(gen.normal(22, (b, kv * rep, s, d)), dtype)
+    dgo = up(ctx, go, dtype)
+    gk = ctx.malloc(k.nbytes)
+    ctx.repeat_kv_backward(dgo, gk, dtype, b, kv, s, d, rep, 0)
+    exp = R.repeat_kv_bwd(go, rep)
+    if dtype == F32:
+        assert np.array_equal(dn(ctx, gk, k.shape, dtype), exp)                 # same order r = 0,1,2: bit-exact
+    else:
+        assert_close(dn(ctx, gk, k.shape, dtype), exp, tol_for(dtype), "repeat_kv bwd")
+
+
+# ---------------------------------------------------------------------------
+# embedding
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+def test_gather_and_deterministic_scatter(ctx, dtype):
+    # reference vectors: collision on row 2 (tests/gpu_kernels.rs:164-206), dup/single/unused rows
+    # (tests/phase2_embedding.rs:37-43)
+    w = prep(np.array([[0.1, 0.2, 0.3, 0.4], [0.3, 0.4, 0.5, 0.6], [0.5, 0.6, 0.7, 0.8]], np.float32), dtype)
+    ids = np.array([2, 0, 2, 1], np.int32)
+    dw, dids = up(ctx, w, dtype), ctx.upload(ids)
+    out = ctx.malloc(4 * 4 * 4)
+    ctx.gather(dw, dids, out, dtype, 4, 3, 4)
+    assert np.array_equal(dn(ctx, out, (4, 4), dtype), w[ids])
+    ones = up(ctx, np.ones((4, 4), np.float32), dtype)
+    gw = ctx.malloc(3 * 4 * 4, zero=True)
+    ctx.gather_backward(ids, ones, gw, dtype, 3, 4)
+    assert dn(ctx, gw, (3, 4), F32).tolist() == [[1] * 4, [1] * 4, [2] * 4]
+    # Zipf ids (hot rows), hidden 256: ascending-position order -> bit-exact against the CPU arm
+    vocab, hidden, n = 512, 256, 3000
+    ids = gen.zipf_ids(23, (n,), vocab).astype(np.int32)
+    W = prep(gen.normal(24, (vocab, hidden)), dtype)
+    go = prep(gen.normal(25, (n, hidden)), dtype)
+    dW, dids, dgo = up(ctx, W, dtype), ctx.upload(ids), up(ctx, go, dtype)
+    out = ctx.malloc(n * hidden * 4)
+    ctx.gather(dW, dids, out, dtype, n, vocab, hidden)
+    assert np.array_equal(dn(ctx, out, (n, hidden), dtype), R.gather_fwd(W, ids.astype(np.float32)))
+    gw0 = gen.normal(26, (vocab, hidden))
+    gw = ctx.upload(gw0)
+    ctx.gather_backward(ids, dgo, gw, dtype, vocab, hidden)
+    exp = R.gather_bwd(ids.astype(np.float32), go, vocab, gw0.copy())
+    assert np.array_equal(dn(ctx, gw, (vocab, hidden), F32), exp)
+    with pytest.raises(hip.EisenHipError):
+        ctx.gather_backward(np.array([0, 999], np.int32), dgo, gw, dtype, vocab, hidden)
+
+
+# ---------------------------------------------------------------------------
+# fused cross entropy
+# ---------------------------------------------------------------------------
+
+def _ce_case(ctx, dtype, rows, classes, seed, masked=False, grad_scale=1.0):
+    x = prep(gen.normal(seed, (rows, classes), 2.0), dtype)
+    t = gen.uniform_ids(seed + 1, (rows,), classes)
+    if masked:
+        t[::3] = R.IGNORE_INDEX
+    valid = int((t != R.IGNORE_INDEX).sum())
+    normalizer = 1.0 / valid
+    dx, dt = up(ctx, x, dtype), ctx.upload(t.astype(np.int32))
+    dl, rl, lo = ctx.malloc(x.nbytes), ctx.malloc(rows * 4), ctx.malloc(4)
+    am, tl = ctx.malloc(rows * 4), ctx.malloc(rows * 4)
+    ctx.cross_entropy(dx, dt, dl, rl, lo, dtype, rows, classes, normalizer, grad_scale, am, tl)
+    loss = float(dn(ctx, lo, (1,), F32)[0])
+    eloss, egl = R.cross_entropy_masked(x, t, grad_scale)
+    assert abs(loss - eloss) <= 1e-3 * abs(eloss), (loss, eloss)             # config 2: loss within 1e-3 relative
+    if dtype == F32:
+        assert abs(loss - eloss) <= 1e-4 * abs(eloss), (loss, eloss)
+    assert_close(dn(ctx, dl, x.shape, dtype), egl, tol_for(dtype), "dlogits")
+    # integer work is bit-exact: first argmax per row and the gathered target logit
+    eam = np.where(t < 0, -1, x.argmax(-1))
+    etl = np.where(t < 0, 0.0, x[np.arange(rows), np.maximum(t, 0)]).astype(np.float32)
+    assert np.array_equal(ctx.download(am, (rows,), np.int32), eam.astype(np.int32))
+    assert np.array_equal(dn(ctx, tl, (rows,), F32), etl)
+    if masked:
+        assert not dn(ctx, dl, x.shape, dtype)[::3].any()
+    for b in (dx, dt, dl, rl, lo, am, tl):
+        b.free()
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+@pytest.mark.parametrize("rows,classes", [(2, 3), (64, 256), (33, 1000), (16, 8192), (8, 32000), (4, 50257), (3, 70000)])
+def test_cross_entropy_fused(ctx, dtype, rows, classes):
+    _ce_case(ctx, dtype, rows, classes, 100 + classes % 97)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+def test_cross_entropy_masked_and_scaled(ctx, dtype):
+    _ce_case(ctx, dtype, 30, 512, 200, masked=True)
+    _ce_case(ctx, dtype, 30, 512, 201, masked=False, grad_scale=3.0)
+
+
+def test_cross_entropy_reference_vector_and_ties(ctx):
+    # tests/gpu_kernels.rs:262-289
+    x = np.array([[2.0, 1.0, 0.1], [0.0, 3.0, 0.5]], np.float32)
+    dx, dt = up(ctx, x, F32), ctx.upload(np.array([0, 1], np.int32))
+    dl, rl, lo = ctx.malloc(24), ctx.malloc(8), ctx.malloc(4)
+    ctx.cross_entropy(dx, dt, dl, rl, lo, F32, 2, 3, 0.5)
+    loss = dn(ctx, lo, (1,), F32)[0]
+    g = dn(ctx, dl, (6,), F32)
+    assert abs(loss - 0.27) < 0.05
+    assert g[0] < 0 < g[1] and g[2] > 0 and g[3] > 0 and g[4] < 0 < g[5]
+    # ties: the first maximum wins, in every kernel variant
+    for classes in (64, 4096, 32000):
+        x = np.zeros((2, classes), np.float32)
+        x[0, [5, 900 % classes, classes - 1]] = 7.0
+        x[1, classes - 1] = 1.0
+        dx, dt = up(ctx, x, BF16), ctx.upload(np.array([1, 2], np.int32))
+        dl, rl, lo, am = ctx.malloc(x.nbytes), ctx.malloc(8), ctx.malloc(4), ctx.malloc(8)
+        ctx.cross_entropy(dx, dt, dl, rl, lo, BF16, 2, classes, 0.5, 1.0, am)
+        assert ctx.download(am, (2,), np.int32).tolist() == [5, classes - 1]
+
+
+def test_cross_entropy_config2_full_size_properties(ctx):
+    """[8192 x 32000] bf16 (config 2): size-independent properties instead of a full oracle run --
+    gradient rows sum to ~0, loss equals the mean of -ln(p_t + 1e-8) recomputed on sampled rows by
+    the oracle, argmax / target logit bit-exact on every row."""
+    rows, classes = 8192, 32000
+    rng = np.random.default_rng(7)
+    x = hip.round_bf16((rng.standard_normal((rows, classes), dtype=np.float32) * 2.0))
+    t = rng.integers(0, classes, rows)
+    dx, dt = up(ctx, x, BF16), ctx.upload(t.astype(np.int32))
+    dl, rl, lo = ctx.malloc(rows * classes * 2), ctx.malloc(rows * 4), ctx.malloc(4)
+    am, tl = ctx.malloc(rows * 4), ctx.malloc(rows * 4)
+    ctx.cross_entropy(dx, dt, dl, rl, lo, BF16, rows, classes, 1.0 / rows, 1.0, am, tl)
+    assert np.array_equal(ctx.download(am, (rows,), np.int32), x.argmax(-1).astype(np.int32))
+    assert np.array_equal(dn(ctx, tl, (rows,), F32), x[np.arange(rows), t])
+    row_loss = dn(ctx, rl, (rows,), F32)
+    sample = np.arange(0, rows, 64)
+    _, egl, probs = R.cross_entropy(x[sample], t[sample])
+    exp_rows = -np.log(probs[np.arange(sample.size), t[sample]].astype(np.float64) + 1e-8)
+    assert_close(row_loss[sample], exp_rows, 1e-4, "row loss")
+    loss = float(dn(ctx, lo, (1,), F32)[0])
+    assert abs(loss - row_loss.astype(np.float64).mean()) <= 1e-5 * loss
+    g = dn(ctx, dl, (rows, classes), BF16)
+    assert_close(g[sample] * rows, egl * sample.size, 2e-2, "dlogits (sampled rows)")
+    assert np.abs(g.astype(np.float64).sum(-1)).max() < 2e-2 / rows
+    for b in (dx, dt, dl, rl, lo, am, tl):
+        b.free()
+
+
+# ---------------------------------------------------------------------------
+# optimiser
+# ---------------------------------------------------------------------------
+
+def test_adamw_multi_tensor_grad_norm_zero(ctx):
+    sizes = [7, 4096, 100003, 64 * 64, 5]
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.95, 1e-8, 0.1
+    W = [gen.normal(300 + i, (n,)) for i, n in enumerate(sizes)]
+    G = [gen.normal(310 + i, (n,), 0.1) for i, n in enumerate(sizes)]
+    M = [np.zeros(n, np.float32) for n in sizes]
+    V = [np.zeros(n, np.float32) for n in sizes]
+    dW, dG = [ctx.upload(w) for w in W], [ctx.upload(g) for g in G]
+    dM, dV = [ctx.malloc(n * 4, zero=True) for n in sizes], [ctx.malloc(n * 4, zero=True) for n in sizes]
+    dB = [ctx.malloc(n * 2) for n in sizes]
+    slots = [(dW[i], dG[i], dM[i], dV[i], dB[i], sizes[i]) for i in range(len(sizes))]
+    out = ctx.malloc(8)
+    ctx.grad_norm(slots, 1.0, out)
+    norm, coef = dn(ctx, out, (2,), F32)
+    enorm, ecoef = R.grad_norm_clip_coef(G, 1.0)
+    assert abs(norm - enorm) <= 1e-6 * enorm and abs(coef - ecoef) <= 1e-6 * ecoef
+    for t in (1, 2, 3):
+        bc1, bc2 = R.adamw_bias_corrections(b1, b2, t)
+        ctx.adamw_step(slots, lr, b1, b2, eps, wd, bc1, bc2, out)          # clip coefficient read on device
+        for i in range(len(sizes)):
+            R.adamw_update(W[i], G[i] * np.float32(ecoef), M[i], V[i], lr, b1, b2, eps, wd, t)
+    for i, n in enumerate(sizes):
+        got = dn(ctx, dW[i], (n,), F32)
+        assert_close(got, W[i], 1e-4, f"w[{i}]")
+        assert_close(dn(ctx, dM[i], (n,), F32), M[i], 1e-4, f"m[{i}]")
+        assert_close(dn(ctx, dV[i], (n,), F32), V[i], 1e-4, f"v[{i}]")
+        assert np.array_equal(dn(ctx, dB[i], (n,), BF16), hip.round_bf16(got))   # bf16 copy = RNE of the new weight
+    # first step from zero moments: closed form (bias corrections cancel)
+    w0, g0 = gen.normal(320, (1000,)), gen.normal(321, (1000,))
+    dw, dg = ctx.upload(w0), ctx.upload(g0)
+    dm, dv = ctx.malloc(4000, zero=True), ctx.malloc(4000, zero=True)
+    bc1, bc2 = R.adamw_bias_corrections(b1, b2, 1)
+    ctx.adamw_step([(dw, dg, dm, dv, None, 1000)], lr, b1, b2, eps, wd, bc1, bc2)
+    closed = w0.astype(np.float64) * (1 - lr * wd) - lr * g0 / (np.abs(g0.astype(np.float64)) + eps)
+    assert_close(dn(ctx, dw, (1000,), F32), closed, 1e-4, "closed form")
+    ctx.zero_grads(slots)
+    assert all(not dn(ctx, dG[i], (n,), F32).any() for i, n in enumerate(sizes))
+
+
+# ---------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------
+
+def _gemm_case(ctx, M, N, K, ta, tb, dtype_ab, dtype_c, accumulate, seed=400):
+    a = prep(gen.normal(seed, (K, M) if ta else (M, K)), dtype_ab)
+    b = prep(gen.normal(seed + 1, (N, K) if tb else (K, N)), dtype_ab)
+    c0 = prep(gen.normal(seed + 2, (M, N)), dtype_c)
+    am = a.T if ta else a
+    bm = b.T if tb else b
+    exp = am.astype(np.float64) @ bm.astype(np.float64) + (c0 if accumulate else 0)
+    da, db, dc = up(ctx, a, dtype_ab), up(ctx, b, dtype_ab), up(ctx, c0, dtype_c)
+    ctx.gemm(da, db, dc, dtype_ab, dtype_c, int(ta), int(tb), M, N, K, int(accumulate))
+    got = dn(ctx, dc, (M, N), dtype_c)
+    # bf16 operands are exact in f32 products; only the f32 accumulation order and the output rounding differ
+    tol = 2e-2 if dtype_c == BF16 else (2e-4 if dtype_ab == F32 else 1e-3)
+    assert_close(got, exp, tol, f"gemm M{M} N{N} K{K} ta{ta} tb{tb}")
+    for x in (da, db, dc):
+        x.free()
+
+
+def test_gemm_reference_vector(ctx):
+    # tests/gpu_kernels.rs:79-103: forward, dA = dC B^T, dB = A^T dC with dC = ones
+    a = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    b = np.array([[7, 8], [9, 1], [2, 3]], np.float32)
+    ones = np.ones((2, 2), np.float32)
+    for dtype in DTYPES:
+        da, db, dg = up(ctx, a, dtype), up(ctx, b, dtype), up(ctx, ones, dtype)
+        c, ga, gb = ctx.malloc(16), ctx.malloc(24, zero=True), ctx.malloc(24, zero=True)
+        ctx.gemm(da, db, c, dtype, dtype, 0, 0, 2, 2, 3)
+        assert dn(ctx, c, (4,), dtype).tolist() == [31.0, 19.0, 85.0, 55.0]
+        ctx.gemm(dg, db, ga, dtype, F32, 0, 1, 2, 3, 2, 1)
+        assert dn(ctx, ga, (6,), F32).tolist() == [15.0, 10.0, 5.0, 15.0, 10.0, 5.0]
+        ctx.gemm(da, dg, gb, dtype, F32, 1, 0, 3, 2, 2, 1)
+        assert dn(ctx, gb, (6,), F32).tolist() == [5.0, 5.0, 7.0, 7.0, 9.0, 9.0]
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (128, 256, 96), (200, 72, 40), (512, 384, 1024), (2048, 2048, 512), (8, 8, 8)])
+def test_gemm_bf16_mfma(ctx, ta, tb, M, N, K):
+    _gemm_case(ctx, M, N, K, ta, tb, BF16, BF16, False)
+    _gemm_case(ctx, M, N, K, ta, tb, BF16, F32, True)
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0)])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (33, 17, 29), (64, 256, 64)])
+def test_gemm_f32_and_odd_shapes(ctx, ta, tb, M, N, K):
+    _gemm_case(ctx, M, N, K, ta, tb, F32, F32, False)
+    _gemm_case(ctx, M, N, K, ta, tb, F32, F32, True)
+    _gemm_case(ctx, M, N, K, ta, tb, BF16, BF16, False)        # odd shapes fall back to the FMA kernel
+
+
+def test_gemm_f32_matches_oracle_order_tolerance(ctx):
+    # config-1 sized linear against the sequential-order f32 oracle, rtol 1e-4
+    a, b, go = gen.normal(410, (64, 64)), gen.normal(411, (64, 256), 0.02), gen.normal(412, (64, 256))
+    da, db, dgo = up(ctx, a, F32), up(ctx, b, F32), up(ctx, go, F32)
+    c, ga, gb = ctx.malloc(64 * 256 * 4), ctx.malloc(a.nbytes, zero=True), ctx.malloc(b.nbytes, zero=True)
+    ctx.gemm(da, db, c, F32, F32, 0, 0, 64, 256, 64)
+    assert_close(dn(ctx, c, (64, 256), F32), R.matmul_fwd(a, b), 1e-4, "fwd")
+    ctx.gemm(dgo, db, ga, F32, F32, 0, 1, 64, 64, 256, 1)
+    ctx.gemm(da, dgo, gb, F32, F32, 1, 0, 64, 256, 64, 1)
+    ega, egb = R.matmul_bwd(a, b, go)
+    assert_close(dn(ctx, ga, a.shape, F32), ega, 1e-4, "dA")
+    assert_close(dn(ctx, gb, b.shape, F32), egb, 1e-4, "dB")
+
+
+def test_bmm_batched(ctx):
+    # tests/gpu_kernels.rs:344-368: scores [2,0,0,1]
+    q = np.array([1, 0, 1, 0, 1, 0, 1, 1, 1, 0, 0, 1], np.float32).reshape(2, 2, 3)
+    k = np.array([1, 0, 1, 0, 1, 0, 1, 0, 0, 0, 0, 1], np.float32).reshape(2, 2, 3)
+    dq, dk = up(ctx, q, F32), up(ctx, k, F32)
+    s = ctx.malloc(32)
+    ctx.bmm(dq, dk, s, F32, F32, 0, 1, 2, 2, 2, 3)
+    assert dn(ctx, s, (8,), F32)[:4].tolist() == [2.0, 0.0, 0.0, 1.0]
+    for dtype, tol in ((F32, 1e-4), (BF16, 2e-2)):
+        a = prep(gen.normal(420, (6, 64, 32)), dtype)
+        b = prep(gen.normal(421, (6, 48, 32)), dtype)
+        da, db = up(ctx, a, dtype), up(ctx, b, dtype)
+        c = ctx.malloc(6 * 64 * 48 * 4)
+        ctx.bmm(da, db, c, dtype, dtype, 0, 1, 6, 64, 48, 32)
+        assert_close(dn(ctx, c, (6, 64, 48), dtype), R.bmm_fwd(a, b, True), tol, "bmm nt")
+        go = prep(gen.normal(422, (6, 64, 48)), dtype)
+        dgo = up(ctx, go, dtype)
+        ga, gb = ctx.malloc(a.nbytes), ctx.malloc(b.nbytes)
+        ctx.bmm(dgo, db, ga, dtype, dtype, 0, 0, 6, 64, 32, 48)        # dA = dC * B   (B stored [N,K])
+        ctx.bmm(dgo, da, gb, dtype, dtype, 1, 0, 6, 48, 32, 64)        # dB = dC^T * A
+        ega, egb = R.bmm_bwd(a, b, go, True)
+        assert_close(dn(ctx, ga, a.shape, dtype), ega, tol, "bmm dA")
+        assert_close(dn(ctx, gb, b.shape, dtype), egb, tol, "bmm dB")
