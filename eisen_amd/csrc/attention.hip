@@ -1,0 +1,601 @@
+// Causal grouped-query flash attention, forward (saving log-sum-exp) and backward.
+//
+// The reference trains through the unfused chain bmm -> mul(scale) -> add(mask) -> softmax ->
+// bmm with repeat_kv and three transposes around it (src/nn/attention.rs:300-375); its fused
+// kernel is inference-only (src/graph/ops/attention.rs:7-18).  These kernels compute the same
+// function and the same gradients without materialising [B*H, S, S] or the repeated K/V:
+//   P = softmax(scale * Q K^T + causal mask),  O = P V
+//   dV = P^T dO,  dP = dO V^T,  dS = P o (dP - rowsum(dO o O)),  dQ = scale dS K,  dK = scale dS^T Q
+// with dK/dV summed over the query heads of a KV group (the repeat_kv backward,
+// src/graph/ops/gqa.rs:168-184) inside the kernel.
+//
+// Tensors are addressed as base + b*stride_b + s*stride_s + h*stride_h + d, so both
+// [B,S,H,hd] (what the projections produce) and [B,H,S,hd] (the reference's q_t layout) work.
+//
+// bf16 path (head_dim 32/64/128), v_mfma_f32_32x32x16_bf16, one wave = 32 query rows or 32 keys:
+//   forward / dQ kernel: a wave keeps its Q (and dO) rows in registers as MFMA B operands and
+//     walks 64-key K/V tiles staged in LDS.  Scores are produced transposed (S^T = K Q^T), so a
+//     lane owns one query and the softmax statistics never leave the lane pair; P^T is already
+//     in B-operand order for O^T += V^T P^T, and V^T / K^T come out of the row-major LDS tile
+//     through ds_read_b64_tr_b16.
+//   dK/dV kernel: a wave keeps 32 keys of K and V in registers, accumulates their dK/dV over
+//     every query head of the group and every visible query tile; Q/dO tiles go through LDS.
+//     No atomics anywhere: dQ has its own query-stationary pass, so results are reproducible.
+// f32 path (any head_dim): one wave per query row / key row, plain FMA, for small shapes.
+#include "device_utils.cuh"
+#include "runtime.h"
+
+namespace {
+
+struct AttnArgs {
+    const void *Q, *K, *V, *O, *dO;
+    void *Out, *dQ, *dK, *dV;
+    float *LSE, *D;
+    int B, S, Hq, Hkv, G, hd;
+    long long q_sb, q_ss, q_sh;
+    long long k_sb, k_ss, k_sh;
+    float scale, scale_log2e;
+    int causal;
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+typedef bf16x4 __attribute__((address_space(3))) * lds_bf16x4_ptr;
+
+// 4 consecutive rows of a column out of a row-major LDS tile: within each group of 16 lanes,
+// lane i receives rows r0..r0+3 of column c0+i when lane L passes &tile[r0 + L/4][c0 + 4*(L%4)].
+__device__ __forceinline__ bf16x4 lds_read_tr(const bf16_t* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p));
+}
+__device__ __forceinline__ bf16x8 concat4(bf16x4 lo, bf16x4 hi) {
+    bf16x8 r;
+    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+    return r;
+}
+// Row index inside a 32x32 MFMA accumulator tile held by register v of a lane in half g.
+__device__ __forceinline__ int acc_row(int v, int g) { return 8 * (v >> 2) + 4 * g + (v & 3); }
+
+// K-operand (8 values along the contraction) for contraction step t of a [32-row k-dim] x
+// [32-col] block of a row-major LDS tile, in the order the accumulator registers 8t..8t+7 use.
+__device__ __forceinline__ bf16x8 lds_tr_operand(const bf16_t* tile, int pitch, int row0, int col0, int t, int lane) {
+    const int g = lane >> 5, L = lane & 15, half = (lane >> 4) & 1;
+    const bf16_t* p = tile + (row0 + 16 * t + 4 * g + (L >> 2)) * pitch + col0 + 16 * half + 4 * (L & 3);
+    return concat4(lds_read_tr(p), lds_read_tr(p + 8 * pitch));
+}
+
+// Cooperative copy of `rows` x HD bf16 (16-byte chunks) from a strided global tensor into LDS.
+template <int HD, int THREADS>
+__device__ __forceinline__ void load_tile(bf16_t* dst, const bf16_t* src, long long row_stride, int first_row, int rows,
+                                          int limit_rows) {
+    constexpr int PITCH = HD + 8, CPR = HD / 8;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int c = threadIdx.x; c < rows * CPR; c += THREADS) {
+        const int r = c / CPR, cc = c % CPR;
+        const int gr = first_row + r;
+        const bf16x8 v = gr < limit_rows ? *reinterpret_cast<const bf16x8*>(src + (long long)gr * row_stride + cc * 8) : zero8;
+        *reinterpret_cast<bf16x8*>(dst + r * PITCH + cc * 8) = v;
+    }
+}
+
+// ---- forward -------------------------------------------------------------------------------
+template <int HD, int GW>
+__global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
+    constexpr int QS = 4 / GW, BKV = 64, PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[BKV * PITCH];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, c = lane & 31;
+    const int hsub = wave % GW, qsub = wave / GW;
+    const int qblk = gridDim.x - 1 - blockIdx.x;  // long rows first
+    const int groups = a.G / GW;
+    const int kvh = blockIdx.y / groups, hq = kvh * a.G + (blockIdx.y % groups) * GW + hsub, b = blockIdx.z;
+    const int q0 = (qblk * QS + qsub) * 32, q = q0 + c;
+    const bool valid_q = q < a.S;
+    const bf16_t* Qp = static_cast<const bf16_t*>(a.Q) + b * a.q_sb + hq * a.q_sh;
+    const bf16_t* Kp = static_cast<const bf16_t*>(a.K) + b * a.k_sb + kvh * a.k_sh;
+    const bf16_t* Vp = static_cast<const bf16_t*>(a.V) + b * a.k_sb + kvh * a.k_sh;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    bf16x8 qf[KSTEPS];
+#pragma unroll
+    for (int st = 0; st < KSTEPS; st++)
+        qf[st] = valid_q ? *reinterpret_cast<const bf16x8*>(Qp + (long long)q * a.q_ss + st * 16 + 8 * g) : zero8;
+    f32x16 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[dt][v] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    const int block_qmax = min(a.S - 1, (qblk * QS + QS - 1) * 32 + 31);
+    const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
+    const int my_qmax = q0 < a.S ? q0 + 31 : -1;
+
+    for (int kt = 0; kt < n_kt; kt++) {
+        __syncthreads();
+        load_tile<HD, 256>(Ks, Kp, a.k_ss, kt * BKV, BKV, a.S);
+        load_tile<HD, 256>(Vs, Vp, a.k_ss, kt * BKV, BKV, a.S);
+        __syncthreads();
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+            const int k0 = kt * BKV + sub * 32;
+            if (k0 >= a.S || my_qmax < 0 || (a.causal && k0 > my_qmax)) continue;  // wave-uniform
+            f32x16 s;
+#pragma unroll
+            for (int v = 0; v < 16; v++) s[v] = 0.f;
+#pragma unroll
+            for (int st = 0; st < KSTEPS; st++) {
+                const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int key = k0 + acc_row(v, g);
+                float val = s[v] * a.scale_log2e;
+                if ((a.causal && key > q) || key >= a.S) val = -INFINITY;
+                s[v] = val;
+                mx = fmaxf(mx, val);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = exp2f(m - m_use);
+            float rowsum = 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                s[v] = exp2f(s[v] - m_use);
+                rowsum += s[v];
+            }
+            rowsum += __shfl_xor(rowsum, 32, 64);
+            l = l * alpha + rowsum;
+            m = m_new;
+            bf16x8 pf[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) pf[t][e] = (bf16_t)s[8 * t + e];
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) o[dt][v] *= alpha;
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const bf16x8 vt = lds_tr_operand(Vs, PITCH, sub * 32, dt * 32, t, lane);
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt, pf[t], o[dt], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (valid_q) {
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        bf16_t* Op = static_cast<bf16_t*>(a.Out) + b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int vg = 0; vg < 4; vg++) {
+                bf16x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[e] = (bf16_t)(o[dt][vg * 4 + e] * inv);
+                *reinterpret_cast<bf16x4*>(Op + dt * 32 + 8 * vg + 4 * g) = w;
+            }
+        if (g == 0) a.LSE[((long long)b * a.Hq + hq) * a.S + q] = (m + log2f(l)) * kLn2;
+    }
+}
+
+// ---- backward: dQ (query-stationary); also writes D = rowsum(dO o O) for the dK/dV pass ------
+template <int HD, int GW>
+__global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
+    constexpr int QS = 4 / GW, BKV = 64, PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[BKV * PITCH];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, c = lane & 31;
+    const int hsub = wave % GW, qsub = wave / GW;
+    const int qblk = gridDim.x - 1 - blockIdx.x;
+    const int groups = a.G / GW;
+    const int kvh = blockIdx.y / groups, hq = kvh * a.G + (blockIdx.y % groups) * GW + hsub, b = blockIdx.z;
+    const int q0 = (qblk * QS + qsub) * 32, q = q0 + c;
+    const bool valid_q = q < a.S;
+    const long long qoff = b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+    const bf16_t* Kp = static_cast<const bf16_t*>(a.K) + b * a.k_sb + kvh * a.k_sh;
+    const bf16_t* Vp = static_cast<const bf16_t*>(a.V) + b * a.k_sb + kvh * a.k_sh;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    bf16x8 qf[KSTEPS], dof[KSTEPS];
+    float dpart = 0.f;
+#pragma unroll
+    for (int st = 0; st < KSTEPS; st++) {
+        const int d = st * 16 + 8 * g;
+        qf[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.Q) + qoff + d) : zero8;
+        dof[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.dO) + qoff + d) : zero8;
+        const bf16x8 of = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.O) + qoff + d) : zero8;
+#pragma unroll
+        for (int e = 0; e < 8; e++) dpart += (float)dof[st][e] * (float)of[e];
+    }
+    const float Dq = dpart + __shfl_xor(dpart, 32, 64);
+    const long long stat = ((long long)b * a.Hq + hq) * a.S + q;
+    if (valid_q && g == 0) a.D[stat] = Dq;
+    const float lse2 = valid_q ? a.LSE[stat] * kLog2e : INFINITY;
+
+    f32x16 dq[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) dq[dt][v] = 0.f;
+
+    const int block_qmax = min(a.S - 1, (qblk * QS + QS - 1) * 32 + 31);
+    const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
+    const int my_qmax = q0 < a.S ? q0 + 31 : -1;
+
+    for (int kt = 0; kt < n_kt; kt++) {
+        __syncthreads();
+        load_tile<HD, 256>(Ks, Kp, a.k_ss, kt * BKV, BKV, a.S);
+        load_tile<HD, 256>(Vs, Vp, a.k_ss, kt * BKV, BKV, a.S);
+        __syncthreads();
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+            const int k0 = kt * BKV + sub * 32;
+            if (k0 >= a.S || my_qmax < 0 || (a.causal && k0 > my_qmax)) continue;
+            f32x16 s, dp;
+#pragma unroll
+            for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
+#pragma unroll
+            for (int st = 0; st < KSTEPS; st++) {
+                const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
+                const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[st], dp, 0, 0, 0);
+            }
+            bf16x8 dsf[2];
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int key = k0 + acc_row(v, g);
+                const bool masked = (a.causal && key > q) || key >= a.S;
+                const float p = masked ? 0.f : exp2f(s[v] * a.scale_log2e - lse2);
+                dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - Dq));
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const bf16x8 ktr = lds_tr_operand(Ks, PITCH, sub * 32, dt * 32, t, lane);
+                    dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsf[t], dq[dt], 0, 0, 0);
+                }
+        }
+    }
+    if (valid_q) {
+        bf16_t* dQp = static_cast<bf16_t*>(a.dQ) + qoff;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int vg = 0; vg < 4; vg++) {
+                bf16x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[e] = (bf16_t)(dq[dt][vg * 4 + e] * a.scale);
+                *reinterpret_cast<bf16x4*>(dQp + dt * 32 + 8 * vg + 4 * g) = w;
+            }
+    }
+}
+
+// ---- backward: dK, dV (key-stationary, summed over the query heads of the group) -------------
+template <int HD>
+__global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
+    constexpr int PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
+    __shared__ __attribute__((aligned(16))) bf16_t Qs[32 * PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t dOs[32 * PITCH];
+    __shared__ float lse_s[32], d_s[32];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, c = lane & 31;
+    const int kb = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int k0w = kb * 128 + wave * 32, key = k0w + c;
+    const bool valid_k = key < a.S;
+    const long long koff = b * a.k_sb + kvh * a.k_sh + (long long)key * a.k_ss;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8 kf[KSTEPS], vf[KSTEPS];
+#pragma unroll
+    for (int st = 0; st < KSTEPS; st++) {
+        const int d = st * 16 + 8 * g;
+        kf[st] = valid_k ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.K) + koff + d) : zero8;
+        vf[st] = valid_k ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.V) + koff + d) : zero8;
+    }
+    f32x16 dk[DT], dv[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) { dk[dt][v] = 0.f; dv[dt][v] = 0.f; }
+
+    const int n_qt = (a.S + 31) / 32;
+    const int qt_start = a.causal ? kb * 4 : 0;  // first query tile that can see this block's first key
+    for (int hh = 0; hh < a.G; hh++) {
+        const int hq = kvh * a.G + hh;
+        const bf16_t* Qp = static_cast<const bf16_t*>(a.Q) + b * a.q_sb + hq * a.q_sh;
+        const bf16_t* dOp = static_cast<const bf16_t*>(a.dO) + b * a.q_sb + hq * a.q_sh;
+        const long long stat0 = ((long long)b * a.Hq + hq) * a.S;
+        for (int qt = qt_start; qt < n_qt; qt++) {
+            const int q0 = qt * 32;
+            __syncthreads();
+            load_tile<HD, 256>(Qs, Qp, a.q_ss, q0, 32, a.S);
+            load_tile<HD, 256>(dOs, dOp, a.q_ss, q0, 32, a.S);
+            if (threadIdx.x < 32) {
+                const int qq = q0 + threadIdx.x;
+                lse_s[threadIdx.x] = qq < a.S ? a.LSE[stat0 + qq] * kLog2e : INFINITY;
+                d_s[threadIdx.x] = qq < a.S ? a.D[stat0 + qq] : 0.f;
+            }
+            __syncthreads();
+            if (k0w >= a.S || (a.causal && q0 + 31 < k0w)) continue;  // wave-uniform
+            f32x16 s, dp;
+#pragma unroll
+            for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
+#pragma unroll
+            for (int st = 0; st < KSTEPS; st++) {
+                const bf16x8 qa = *reinterpret_cast<const bf16x8*>(Qs + c * PITCH + st * 16 + 8 * g);
+                const bf16x8 da = *reinterpret_cast<const bf16x8*>(dOs + c * PITCH + st * 16 + 8 * g);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[st], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[st], dp, 0, 0, 0);
+            }
+            bf16x8 pf[2], dsf[2];
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int qi = acc_row(v, g), qq = q0 + qi;
+                const bool masked = (a.causal && key > qq) || qq >= a.S || !valid_k;
+                const float p = masked ? 0.f : exp2f(s[v] * a.scale_log2e - lse_s[qi]);
+                pf[v >> 3][v & 7] = (bf16_t)p;
+                dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - d_s[qi]));
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const bf16x8 dotr = lds_tr_operand(dOs, PITCH, 0, dt * 32, t, lane);
+                    const bf16x8 qtr = lds_tr_operand(Qs, PITCH, 0, dt * 32, t, lane);
+                    dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[t], dotr, dv[dt], 0, 0, 0);
+                    dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[t], qtr, dk[dt], 0, 0, 0);
+                }
+        }
+    }
+    bf16_t* dKp = static_cast<bf16_t*>(a.dK) + b * a.k_sb + kvh * a.k_sh;
+    bf16_t* dVp = static_cast<bf16_t*>(a.dV) + b * a.k_sb + kvh * a.k_sh;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int kr = k0w + acc_row(v, g);
+            if (kr < a.S) {
+                dKp[(long long)kr * a.k_ss + dt * 32 + c] = (bf16_t)(dk[dt][v] * a.scale);
+                dVp[(long long)kr * a.k_ss + dt * 32 + c] = (bf16_t)dv[dt][v];
+            }
+        }
+}
+
+// ---- f32 path: one wave per row, any head_dim ---------------------------------------------------
+// forward: scores in LDS (S floats), same arithmetic as the unfused chain
+// (bmm -> *scale -> mask -> softmax -> bmm; src/nn/attention.rs:338-375).
+__global__ __launch_bounds__(64) void attn_f32_fwd_kernel(AttnArgs a) {
+    extern __shared__ float sc[];
+    const int q = blockIdx.x, hq = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const int kvh = hq / a.G;
+    const float* Qr = static_cast<const float*>(a.Q) + b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+    const float* Kp = static_cast<const float*>(a.K) + b * a.k_sb + kvh * a.k_sh;
+    const float* Vp = static_cast<const float*>(a.V) + b * a.k_sb + kvh * a.k_sh;
+    const int nk = a.causal ? q + 1 : a.S;
+    float mx = -INFINITY;
+    for (int j = lane; j < nk; j += 64) {
+        const float* Kr = Kp + (long long)j * a.k_ss;
+        float dot = 0.f;
+        for (int d = 0; d < a.hd; d++) dot += Qr[d] * Kr[d];
+        dot *= a.scale;
+        sc[j] = dot;
+        mx = fmaxf(mx, dot);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int j = lane; j < nk; j += 64) {
+        const float e = __expf(sc[j] - mx);
+        sc[j] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    __syncthreads();
+    float* Or = static_cast<float*>(a.Out) + b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+    for (int d = lane; d < a.hd; d += 64) {
+        float acc = 0.f;
+        for (int j = 0; j < nk; j++) acc += sc[j] * Vp[(long long)j * a.k_ss + d];
+        Or[d] = acc / sum;
+    }
+    if (lane == 0) a.LSE[((long long)b * a.Hq + hq) * a.S + q] = mx + logf(sum);
+}
+
+__global__ __launch_bounds__(64) void attn_f32_bwd_dq_kernel(AttnArgs a) {
+    extern __shared__ float ds[];
+    const int q = blockIdx.x, hq = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const int kvh = hq / a.G;
+    const long long qoff = b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+    const float* Qr = static_cast<const float*>(a.Q) + qoff;
+    const float* dOr = static_cast<const float*>(a.dO) + qoff;
+    const float* Or = static_cast<const float*>(a.O) + qoff;
+    const float* Kp = static_cast<const float*>(a.K) + b * a.k_sb + kvh * a.k_sh;
+    const float* Vp = static_cast<const float*>(a.V) + b * a.k_sb + kvh * a.k_sh;
+    const long long stat = ((long long)b * a.Hq + hq) * a.S + q;
+    float dpart = 0.f;
+    for (int d = lane; d < a.hd; d += 64) dpart += dOr[d] * Or[d];
+    const float Dq = wave_sum(dpart);
+    if (lane == 0) a.D[stat] = Dq;
+    const float lse = a.LSE[stat];
+    const int nk = a.causal ? q + 1 : a.S;
+    for (int j = lane; j < nk; j += 64) {
+        const float* Kr = Kp + (long long)j * a.k_ss;
+        const float* Vr = Vp + (long long)j * a.k_ss;
+        float dot = 0.f, dp = 0.f;
+        for (int d = 0; d < a.hd; d++) {
+            dot += Qr[d] * Kr[d];
+            dp += dOr[d] * Vr[d];
+        }
+        const float p = __expf(dot * a.scale - lse);
+        ds[j] = p * (dp - Dq) * a.scale;
+    }
+    __syncthreads();
+    float* dQr = static_cast<float*>(a.dQ) + qoff;
+    for (int d = lane; d < a.hd; d += 64) {
+        float acc = 0.f;
+        for (int j = 0; j < nk; j++) acc += ds[j] * Kp[(long long)j * a.k_ss + d];
+        dQr[d] = acc;
+    }
+}
+
+// one wave per key row; walks the query heads of the group (ascending, like repeat_kv's
+// backward) and the queries that see this key.
+__global__ __launch_bounds__(64) void attn_f32_bwd_dkv_kernel(AttnArgs a) {
+    extern __shared__ float sm[];  // p[S], ds[S]
+    float* pbuf = sm;
+    float* dsbuf = sm + a.S;
+    const int j = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const long long koff = b * a.k_sb + kvh * a.k_sh + (long long)j * a.k_ss;
+    const float* Kr = static_cast<const float*>(a.K) + koff;
+    const float* Vr = static_cast<const float*>(a.V) + koff;
+    const int qs = a.causal ? j : 0;
+    // per-lane accumulators for d = lane, lane+64, ... (head_dim <= 256)
+    float accK[4] = {0.f, 0.f, 0.f, 0.f}, accV[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int hh = 0; hh < a.G; hh++) {
+        const int hq = kvh * a.G + hh;
+        const float* Qp = static_cast<const float*>(a.Q) + b * a.q_sb + hq * a.q_sh;
+        const float* dOp = static_cast<const float*>(a.dO) + b * a.q_sb + hq * a.q_sh;
+        const long long stat0 = ((long long)b * a.Hq + hq) * a.S;
+        __syncthreads();
+        for (int q = qs + lane; q < a.S; q += 64) {
+            const float* Qr = Qp + (long long)q * a.q_ss;
+            const float* dOr = dOp + (long long)q * a.q_ss;
+            float dot = 0.f, dp = 0.f;
+            for (int d = 0; d < a.hd; d++) {
+                dot += Qr[d] * Kr[d];
+                dp += dOr[d] * Vr[d];
+            }
+            const float p = __expf(dot * a.scale - a.LSE[stat0 + q]);
+            pbuf[q] = p;
+            dsbuf[q] = p * (dp - a.D[stat0 + q]) * a.scale;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int d = lane + 64 * u;
+            if (d < a.hd)
+                for (int q = qs; q < a.S; q++) {
+                    accV[u] += pbuf[q] * dOp[(long long)q * a.q_ss + d];
+                    accK[u] += dsbuf[q] * Qp[(long long)q * a.q_ss + d];
+                }
+        }
+    }
+    float* dKr = static_cast<float*>(a.dK) + koff;
+    float* dVr = static_cast<float*>(a.dV) + koff;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int d = lane + 64 * u;
+        if (d < a.hd) {
+            dKr[d] = accK[u];
+            dVr[d] = accV[u];
+        }
+    }
+}
+
+int fill_args(eisen_ctx* ctx, AttnArgs& a, int dtype, size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
+              const long long* q_strides, const long long* kv_strides, float scale, int causal, const char* who) {
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "%s: unknown dtype %d", who, dtype);
+    EISEN_REQUIRE(ctx, B > 0 && S > 0 && Hq > 0 && Hkv > 0 && hd > 0, EISEN_E_SHAPE, "%s: empty dimension", who);
+    EISEN_REQUIRE(ctx, Hq % Hkv == 0, EISEN_E_SHAPE, "%s: %zu query heads not divisible by %zu kv heads", who, Hq, Hkv);
+    EISEN_REQUIRE(ctx, B < 65536 && Hq < 65536 && S < (size_t(1) << 24) && hd <= 256, EISEN_E_SHAPE, "%s: dimension out of range", who);
+    if (dtype == EISEN_BF16)
+        EISEN_REQUIRE(ctx, hd == 32 || hd == 64 || hd == 128, EISEN_E_SHAPE, "%s: bf16 path supports head_dim 32, 64, 128 (got %zu)", who, hd);
+    a.B = (int)B; a.S = (int)S; a.Hq = (int)Hq; a.Hkv = (int)Hkv; a.G = (int)(Hq / Hkv); a.hd = (int)hd;
+    if (q_strides) { a.q_sb = q_strides[0]; a.q_ss = q_strides[1]; a.q_sh = q_strides[2]; }
+    else { a.q_sb = (long long)(S * Hq * hd); a.q_ss = (long long)(Hq * hd); a.q_sh = (long long)hd; }
+    if (kv_strides) { a.k_sb = kv_strides[0]; a.k_ss = kv_strides[1]; a.k_sh = kv_strides[2]; }
+    else { a.k_sb = (long long)(S * Hkv * hd); a.k_ss = (long long)(Hkv * hd); a.k_sh = (long long)hd; }
+    if (dtype == EISEN_BF16)
+        EISEN_REQUIRE(ctx, a.q_sb % 8 == 0 && a.q_ss % 8 == 0 && a.q_sh % 8 == 0 && a.k_sb % 8 == 0 && a.k_ss % 8 == 0 && a.k_sh % 8 == 0,
+                      EISEN_E_ALIGN, "%s: strides must be multiples of 8 elements for bf16", who);
+    a.scale = scale;
+    a.scale_log2e = scale * kLog2e;
+    a.causal = causal;
+    return 0;
+}
+
+template <int HD>
+void launch_fwd(eisen_ctx* ctx, const AttnArgs& a) {
+    const int gw = a.G % 4 == 0 ? 4 : (a.G % 2 == 0 ? 2 : 1);
+    const int qs = 4 / gw;
+    dim3 grid((unsigned)eisen_ceil_div(a.S, 32 * qs), (unsigned)(a.Hkv * (a.G / gw)), (unsigned)a.B);
+    if (gw == 4) fa_fwd_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
+    else if (gw == 2) fa_fwd_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
+    else fa_fwd_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
+}
+template <int HD>
+void launch_bwd(eisen_ctx* ctx, const AttnArgs& a) {
+    const int gw = a.G % 4 == 0 ? 4 : (a.G % 2 == 0 ? 2 : 1);
+    const int qs = 4 / gw;
+    dim3 grid((unsigned)eisen_ceil_div(a.S, 32 * qs), (unsigned)(a.Hkv * (a.G / gw)), (unsigned)a.B);
+    if (gw == 4) fa_bwd_dq_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
+    else if (gw == 2) fa_bwd_dq_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
+    else fa_bwd_dq_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
+    dim3 grid2((unsigned)eisen_ceil_div(a.S, 128), (unsigned)a.Hkv, (unsigned)a.B);
+    fa_bwd_dkv_kernel<HD><<<grid2, 256, 0, ctx->stream>>>(a);
+}
+
+}  // namespace
+
+extern "C" int eisen_hip_attention_forward(eisen_ctx* ctx, const void* q, const void* k, const void* v, void* out,
+                                           float* lse, int dtype, size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
+                                           const long long* q_strides, const long long* kv_strides, float scale,
+                                           int causal) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, q && k && v && out && lse, EISEN_E_ARG, "attention_forward: null pointer");
+    AttnArgs a{};
+    int rc = fill_args(ctx, a, dtype, B, S, Hq, Hkv, hd, q_strides, kv_strides, scale, causal, "attention_forward");
+    if (rc) return rc;
+    a.Q = q; a.K = k; a.V = v; a.Out = out; a.LSE = lse;
+    if (dtype == EISEN_BF16) {
+        EISEN_REQUIRE(ctx, eisen_aligned(q, 16) && eisen_aligned(k, 16) && eisen_aligned(v, 16) && eisen_aligned(out, 16),
+                      EISEN_E_ALIGN, "attention_forward: bf16 buffers must be 16-byte aligned");
+        if (hd == 32) launch_fwd<32>(ctx, a);
+        else if (hd == 64) launch_fwd<64>(ctx, a);
+        else launch_fwd<128>(ctx, a);
+    } else {
+        EISEN_REQUIRE(ctx, S * sizeof(float) <= 64 * 1024, EISEN_E_SHAPE, "attention_forward: f32 path supports S <= 16384");
+        dim3 grid((unsigned)S, (unsigned)Hq, (unsigned)B);
+        attn_f32_fwd_kernel<<<grid, 64, S * sizeof(float), ctx->stream>>>(a);
+    }
+    EISEN_LAUNCH_CHECK(ctx, "attention forward");
+    return 0;
+}
+
+extern "C" int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                            const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype,
+                                            size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
+                                            const long long* q_strides, const long long* kv_strides, float scale,
+                                            int causal) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, q && k && v && out && dout && lse && dq && dk && dv, EISEN_E_ARG, "attention_backward: null pointer");
+    AttnArgs a{};
+    int rc = fill_args(ctx, a, dtype, B, S, Hq, Hkv, hd, q_strides, kv_strides, scale, causal, "attention_backward");
+    if (rc) return rc;
+    a.Q = q; a.K = k; a.V = v; a.O = out; a.dO = dout; a.LSE = const_cast<float*>(lse);
+    a.dQ = dq; a.dK = dk; a.dV = dv;
+    void* ws = nullptr;
+    rc = eisen_workspace(ctx, B * Hq * S * sizeof(float), &ws);
+    if (rc) return rc;
+    a.D = static_cast<float*>(ws);
+    if (dtype == EISEN_BF16) {
+        EISEN_REQUIRE(ctx, eisen_aligned(q, 16) && eisen_aligned(k, 16) && eisen_aligned(v, 16) && eisen_aligned(out, 16) &&
+                               eisen_aligned(dout, 16) && eisen_aligned(dq, 16) && eisen_aligned(dk, 16) && eisen_aligned(dv, 16),
+                      EISEN_E_ALIGN, "attention_backward: bf16 buffers must be 16-byte aligned");
+        if (hd == 32) launch_bwd<32>(ctx, a);
+        else if (hd == 64) launch_bwd<64>(ctx, a);
+        else launch_bwd<128>(ctx, a);
+    } else {
+        EISEN_REQUIRE(ctx, 2 * S * sizeof(float) <= 64 * 1024, EISEN_E_SHAPE, "attention_backward: f32 path supports S <= 8192");
+        dim3 grid((unsigned)S, (unsigned)Hq, (unsigned)B);
+        attn_f32_bwd_dq_kernel<<<grid, 64, S * sizeof(float), ctx->stream>>>(a);
+        dim3 grid2((unsigned)S, (unsigned)Hkv, (unsigned)B);
+        attn_f32_bwd_dkv_kernel<<<grid2, 64, 2 * S * sizeof(float), ctx->stream>>>(a);
+    }
+    EISEN_LAUNCH_CHECK(ctx, "attention backward");
+    return 0;
+}

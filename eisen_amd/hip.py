@@ -236,6 +236,21 @@ class Context:
     def bmm(self, A, B, Cbuf, dtype_ab, dtype_c, trans_a, trans_b, batch, M, N, K, accumulate=0):
         self._call("eisen_hip_bmm", _ptr(A), _ptr(B), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(batch), _sz(M), _sz(N), _sz(K), _i(accumulate))
 
+    # ---- attention --------------------------------------------------------------------
+    @staticmethod
+    def _strides(v):
+        return None if v is None else (C.c_longlong * 3)(*[int(x) for x in v])
+
+    def attention_forward(self, q, k, v, out, lse, dtype, B, S, Hq, Hkv, hd, scale, causal=True, q_strides=None, kv_strides=None):
+        self._call("eisen_hip_attention_forward", _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _i(dtype), _sz(B), _sz(S), _sz(Hq),
+                   _sz(Hkv), _sz(hd), self._strides(q_strides), self._strides(kv_strides), _f(scale), _i(int(causal)))
+
+    def attention_backward(self, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, scale, causal=True, q_strides=None,
+                           kv_strides=None):
+        self._call("eisen_hip_attention_backward", _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk),
+                   _ptr(dv), _i(dtype), _sz(B), _sz(S), _sz(Hq), _sz(Hkv), _sz(hd), self._strides(q_strides), self._strides(kv_strides),
+                   _f(scale), _i(int(causal)))
+
     # ---- embedding --------------------------------------------------------------------
     def gather(self, weight, ids, out, dtype, n_ids, vocab, hidden):
         self._call("eisen_hip_gather", _ptr(weight), _ptr(ids), _ptr(out), _i(dtype), _sz(n_ids), _sz(vocab), _sz(hidden))

@@ -187,6 +187,28 @@ int eisen_hip_gemm(eisen_ctx* ctx, const void* A, const void* B, void* C, int dt
 int eisen_hip_bmm(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
                   int trans_b, size_t batch, size_t M, size_t N, size_t K, int accumulate);
 
+/* ---- attention ------------------------------------------------------------------------- */
+
+/* Causal grouped-query attention with saved log-sum-exp, and its backward.  Computes what
+ * GroupedQueryAttention::forward_with_mask builds from reshape / transpose_0213 / repeat_kv /
+ * bmm / mul(scale) / add(mask) / softmax / bmm (src/nn/attention.rs:300-375) and what that
+ * chain's backward closures accumulate (src/graph/ops/linear.rs:1452-1498, reduction.rs:504-512,
+ * gqa.rs:168-184), without materialising scores or repeated K/V.  The reference's own fused
+ * kernel is forward/inference only (flash_attention_f32, kernels/ops_f32.cu:648-692;
+ * src/graph/ops/attention.rs:7-18).
+ *   q, out, dout, dq : [B, S, Hq, hd];  k, v, dk, dv : [B, S, Hkv, hd];  lse : [B, Hq, S] f32.
+ * q_strides / kv_strides: optional {batch, seq, head} element strides (NULL = the contiguous
+ * layouts above; {Hq*S*hd, hd, S*hd} addresses the reference's [B,H,S,hd] tensors).
+ * Query head h attends KV head h / (Hq/Hkv); dk, dv are summed over the heads of each group.
+ * dq, dk, dv are overwritten.  bf16: hd in {32, 64, 128}; f32: hd <= 256, S <= 8192. */
+int eisen_hip_attention_forward(eisen_ctx* ctx, const void* q, const void* k, const void* v, void* out, float* lse,
+                                int dtype, size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
+                                const long long* q_strides, const long long* kv_strides, float scale, int causal);
+int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                 const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype, size_t B,
+                                 size_t S, size_t Hq, size_t Hkv, size_t hd, const long long* q_strides,
+                                 const long long* kv_strides, float scale, int causal);
+
 /* ---- embedding ------------------------------------------------------------------------- */
 
 /* gather_f32 (kernels/ops_f32.cu:513; Graph::gather, src/graph/ops/transform.rs:132-324).
