@@ -1,0 +1,712 @@
+// Graph / Tensor / Tape for Device::Gpu over the eisen_hip C-ABI.  See graph.hpp.
+#include "graph.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <numeric>
+
+namespace eisen {
+
+namespace {
+size_t numel_of(const std::vector<size_t>& shape) {
+    size_t n = 1;
+    for (size_t s : shape) n *= s;
+    return n;
+}
+std::string shape_str(const std::vector<size_t>& s) {
+    std::string r = "[";
+    for (size_t i = 0; i < s.size(); i++) r += (i ? "," : "") + std::to_string(s[i]);
+    return r + "]";
+}
+constexpr size_t kHostCopyLimit = size_t(1) << 22;  // elements; token-id tensors are far below
+}  // namespace
+
+std::vector<size_t> compute_strides(const std::vector<size_t>& shape) {
+    std::vector<size_t> st(shape.size(), 0);
+    size_t cur = 1;
+    for (size_t i = shape.size(); i-- > 0;) {
+        st[i] = cur;
+        cur *= shape[i];
+    }
+    return st;
+}
+std::vector<size_t> broadcasted_shape(const std::vector<size_t>& a, const std::vector<size_t>& b) {
+    const size_t ml = std::max(a.size(), b.size());
+    std::vector<size_t> out(ml);
+    for (size_t i = 0; i < ml; i++) {
+        const size_t da = i < ml - a.size() ? 1 : a[i - (ml - a.size())];
+        const size_t db = i < ml - b.size() ? 1 : b[i - (ml - b.size())];
+        out[i] = std::max(da, db);
+    }
+    return out;
+}
+std::vector<size_t> broadcasted_strides(const std::vector<size_t>& shape, const std::vector<size_t>& base,
+                                        const std::vector<size_t>& out_shape) {
+    std::vector<size_t> st(out_shape.size(), 0);
+    const size_t pad = out_shape.size() - shape.size();
+    for (size_t i = 0; i < shape.size(); i++)
+        if (shape[i] == out_shape[pad + i]) st[pad + i] = base[i];
+    return st;
+}
+
+Graph::Graph(eisen_ctx* ctx, PrecisionMode mode) : precision_mode(mode), ctx_(ctx) {
+    if (!ctx) throw Error("Graph: null device context (Device::Gpu needs eisen_hip_init)");
+}
+
+Graph::~Graph() {
+    for (auto& t : tensors) release(t);
+}
+
+void Graph::check(int rc, const char* what) const {
+    if (rc != 0) throw Error(std::string(what) + ": " + eisen_hip_last_error(ctx_) + " (code " + std::to_string(rc) + ")");
+}
+
+Tensor& Graph::at(size_t id) {
+    if (id >= tensors.size()) throw Error("tensor id " + std::to_string(id) + " out of range");
+    return tensors[id];
+}
+
+Storage Graph::device_alloc(size_t numel, int dtype, bool zero) {
+    Storage s;
+    s.numel = numel;
+    s.dtype = dtype;
+    const size_t bytes = std::max<size_t>(numel, 1) * (dtype == EISEN_BF16 ? 2 : 4);
+    check(zero ? eisen_hip_malloc_zeroed(ctx_, bytes, &s.ptr) : eisen_hip_malloc(ctx_, bytes, &s.ptr), "device allocation");
+    return s;
+}
+void Graph::device_free(Storage& s) {
+    if (s.ptr) check(eisen_hip_free(ctx_, s.ptr), "device free");
+    s = Storage();
+}
+void Graph::release(Tensor& t) {
+    if (t.data.ptr) eisen_hip_free(ctx_, t.data.ptr);
+    if (t.grad.ptr) eisen_hip_free(ctx_, t.grad.ptr);
+    if (t.shadow.ptr) eisen_hip_free(ctx_, t.shadow.ptr);
+    t.data = t.grad = t.shadow = Storage();
+}
+
+size_t Graph::push_tensor(const std::vector<size_t>& shape, int dtype, bool pooled) {
+    Tensor t;
+    t.id = tensors.size();
+    t.shape = shape;
+    t.strides = compute_strides(shape);
+    t.is_pooled = pooled;
+    t.data = device_alloc(numel_of(shape), dtype, false);
+    tensors.push_back(std::move(t));
+    return tensors.size() - 1;
+}
+
+// Graph::alloc (src/graph/mod.rs:558-564) + Tensor::new (src/tensor.rs:145-175): data uploaded,
+// gradient zero-filled.  In mixed mode the kernels read a bf16 copy; `data` stays the f32 master.
+size_t Graph::alloc(const std::vector<size_t>& shape, const float* data, size_t n) {
+    if (n != numel_of(shape)) throw Error("alloc: shape " + shape_str(shape) + " does not hold " + std::to_string(n) + " values");
+    const size_t id = push_tensor(shape, EISEN_F32, false);
+    Tensor& t = tensors[id];
+    t.is_param = true;
+    if (n) check(eisen_hip_htod(ctx_, t.data.ptr, data, n * sizeof(float)), "alloc upload");
+    t.grad = device_alloc(n, EISEN_F32, true);
+    if (n <= kHostCopyLimit) t.host_copy.assign(data, data + n);
+    if (uses_bf16_mixed_precision()) {
+        t.shadow = device_alloc(n, EISEN_BF16, false);
+        refresh_shadow(id);
+    }
+    return id;
+}
+size_t Graph::alloc(const std::vector<size_t>& shape, const std::vector<float>& data) { return alloc(shape, data.data(), data.size()); }
+
+// Graph::alloc_pooled (src/graph/mod.rs:437-556): an activation-typed buffer from the pool;
+// the gradient is allocated on first use in backward (src/graph/memory.rs:401-417).
+size_t Graph::alloc_pooled(const std::vector<size_t>& shape) { return push_tensor(shape, act_dtype(), true); }
+size_t Graph::alloc_pooled_dtype(const std::vector<size_t>& shape, int dtype) { return push_tensor(shape, dtype, true); }
+
+void Graph::refresh_shadow(size_t id) {
+    Tensor& t = at(id);
+    if (!t.shadow.valid()) return;
+    check(eisen_hip_cast(ctx_, t.data.ptr, EISEN_F32, t.shadow.ptr, EISEN_BF16, t.data.numel), "bf16 weight copy");
+}
+
+const Storage& Graph::compute_data(size_t id) {
+    Tensor& t = at(id);
+    return t.shadow.valid() ? t.shadow : t.data;
+}
+
+// Graph::load_tensor_data (src/graph/mod.rs:368-430).  bf16 storage is filled with
+// round-to-nearest-even values (the device cast), not the reference's host-side truncation.
+void Graph::load_tensor_data(size_t id, const float* host, size_t n) {
+    Tensor& t = at(id);
+    if (n != t.size()) throw Error("Shape mismatch: Tensor " + std::to_string(id) + " expects " + std::to_string(t.size()) + " elements, but got " + std::to_string(n) + ".");
+    if (n <= kHostCopyLimit) t.host_copy.assign(host, host + n);
+    else t.host_copy.clear();
+    if (t.data.dtype == EISEN_F32) {
+        check(eisen_hip_htod(ctx_, t.data.ptr, host, n * sizeof(float)), "load_tensor_data");
+        refresh_shadow(id);
+    } else {
+        Storage tmp = device_alloc(n, EISEN_F32, false);
+        check(eisen_hip_htod(ctx_, tmp.ptr, host, n * sizeof(float)), "load_tensor_data");
+        check(eisen_hip_cast(ctx_, tmp.ptr, EISEN_F32, t.data.ptr, EISEN_BF16, n), "load_tensor_data cast");
+        device_free(tmp);
+    }
+}
+
+static std::vector<float> download(Graph& g, const Storage& s) {
+    std::vector<float> out(s.numel);
+    if (!s.numel) return out;
+    if (s.dtype == EISEN_F32) {
+        g.check(eisen_hip_dtoh(g.ctx(), out.data(), s.ptr, s.numel * sizeof(float)), "sync_to_cpu");
+    } else {
+        std::vector<uint16_t> raw(s.numel);
+        g.check(eisen_hip_dtoh(g.ctx(), raw.data(), s.ptr, s.numel * 2), "sync_to_cpu");
+        for (size_t i = 0; i < s.numel; i++) {
+            const uint32_t bits = (uint32_t)raw[i] << 16;
+            std::memcpy(&out[i], &bits, 4);
+        }
+    }
+    return out;
+}
+
+// Tensor::sync_to_cpu / Graph::sync_grad_to_cpu (src/tensor.rs:177-223, src/graph/mod.rs:629-668).
+std::vector<float> Graph::sync_to_cpu(size_t id) { return download(*this, at(id).data); }
+std::vector<float> Graph::sync_grad_to_cpu(size_t id) {
+    Tensor& t = at(id);
+    materialize_grad(id);
+    if (!t.grad.valid()) return std::vector<float>(t.size(), 0.0f);  // never touched by backward: zero
+    return download(*this, t.grad);
+}
+
+void Graph::synchronize() { check(eisen_hip_stream_sync(ctx_), "synchronize"); }
+
+// Graph::reinterpret_shape (src/graph/ops/transform.rs:413-426).
+void Graph::reinterpret_shape(size_t id, const std::vector<size_t>& shape) {
+    Tensor& t = at(id);
+    if (numel_of(shape) != t.size()) throw Error("reinterpret_shape: element count mismatch");
+    t.shape = shape;
+    t.strides = compute_strides(shape);
+}
+
+// Graph::restore_save_point / clear_activations (src/graph/mod.rs:336-365, :432-435): buffers go
+// back to the size-keyed pool inside the runtime.
+void Graph::restore_save_point(size_t save_point) {
+    while (tensors.size() > save_point) {
+        release(tensors.back());
+        tensors.pop_back();
+    }
+}
+void Graph::clear_activations() {
+    tape.nodes.clear();
+    restore_save_point(num_params);
+}
+
+void Graph::record(std::vector<size_t> inputs, size_t output, std::function<void(Graph&)> fn) {
+    if (no_grad) return;  // e.g. src/graph/ops/linear.rs:288
+    tape.nodes.push_back(TapeNode{std::move(inputs), output, std::move(fn)});
+}
+
+Storage& Graph::grad_for_write(size_t id, int* accumulate) {
+    Tensor& t = at(id);
+    if (t.is_param) {
+        *accumulate = t.grad_zero_pending ? 0 : 1;
+        t.grad_zero_pending = false;
+        return t.grad;
+    }
+    if (!t.grad.valid()) {
+        t.grad = device_alloc(t.size(), t.data.dtype, false);
+        *accumulate = 0;
+    } else {
+        *accumulate = t.grad_written ? 1 : 0;
+    }
+    t.grad_written = true;
+    return t.grad;
+}
+
+const Storage& Graph::grad_for_read(size_t id) {
+    Tensor& t = at(id);
+    materialize_grad(id);
+    if (!t.grad.valid()) throw Error("backward: tensor " + std::to_string(id) + " has no gradient to read");
+    return t.grad;
+}
+
+void Graph::request_zero_grad(size_t id) {
+    Tensor& t = at(id);
+    if (t.is_param) t.grad_zero_pending = true;
+    else if (t.grad.valid()) check(eisen_hip_memset_zero(ctx_, t.grad.ptr, t.grad.numel * (t.grad.dtype == EISEN_BF16 ? 2 : 4)), "zero_grad");
+}
+
+void Graph::materialize_grad(size_t id) {
+    Tensor& t = at(id);
+    if (t.grad_zero_pending) {
+        check(eisen_hip_memset_zero(ctx_, t.grad.ptr, t.grad.numel * sizeof(float)), "zero_grad");
+        t.grad_zero_pending = false;
+    }
+}
+
+// Graph::backward (src/graph/mod.rs:670-796): seed every element of the loss gradient with 1,
+// replay the tape in reverse insertion order, keep the tape.  No per-node synchronisation:
+// everything is ordered by the one stream.
+void Graph::backward(size_t loss_id) {
+    if (no_grad) return;
+    backward_root_ = loss_id;
+    int acc = 0;
+    Storage& lg = grad_for_write(loss_id, &acc);
+    check(eisen_hip_fill(ctx_, lg.ptr, lg.dtype, 1.0f, lg.numel), "backward seed");
+    for (size_t i = tape.nodes.size(); i-- > 0;) {
+        TapeNode& node = tape.nodes[i];
+        Tensor& out = at(node.output);
+        // an output nobody differentiated through has a zero gradient: nothing to propagate
+        if (!out.is_param && !(out.grad.valid() && out.grad_written)) continue;
+        node.backward_fn(*this);
+    }
+    backward_root_ = (size_t)-1;
+}
+
+// ---- elementwise ---------------------------------------------------------------------------------
+
+// Graph::add / Graph::mul (src/graph/ops/elementwise.rs:15-183, :188-331).
+size_t Graph::elementwise_binary(size_t a, size_t b, bool is_mul) {
+    const std::vector<size_t> sa = at(a).shape, sb = at(b).shape;
+    const Storage da = compute_data(a), db = compute_data(b);
+    if (da.dtype != db.dtype) throw Error(std::string(is_mul ? "mul" : "add") + ": operands have different element types");
+    const int dtype = da.dtype;
+    const std::vector<size_t> os = broadcasted_shape(sa, sb);
+    if (os.size() > 4) throw Error("add/mul: rank above 4 is not supported");
+    const size_t n = numel_of(os);
+    const size_t out = push_tensor(os, dtype, true);
+    const bool same = sa == os && sb == os;
+    const std::vector<size_t> sta = broadcasted_strides(sa, compute_strides(sa), os), stb = broadcasted_strides(sb, compute_strides(sb), os);
+    if (same) {
+        check(is_mul ? eisen_hip_mul(ctx_, da.ptr, db.ptr, at(out).data.ptr, dtype, n) : eisen_hip_add(ctx_, da.ptr, db.ptr, at(out).data.ptr, dtype, n),
+              is_mul ? "mul" : "add");
+    } else {
+        const std::vector<size_t> osv = os.empty() ? std::vector<size_t>{1} : os;
+        std::vector<size_t> xa = sta, xb = stb;
+        if (os.empty()) { xa = {0}; xb = {0}; }
+        check(is_mul ? eisen_hip_mul_bcast(ctx_, da.ptr, db.ptr, at(out).data.ptr, dtype, (int)osv.size(), osv.data(), xa.data(), xb.data())
+                     : eisen_hip_add_bcast(ctx_, da.ptr, db.ptr, at(out).data.ptr, dtype, (int)osv.size(), osv.data(), xa.data(), xb.data()),
+              is_mul ? "mul (broadcast)" : "add (broadcast)");
+    }
+    record({a, b}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        auto one_side = [&](size_t self, size_t other, const std::vector<size_t>& self_shape, const std::vector<size_t>& self_st,
+                            const std::vector<size_t>& other_st) {
+            int acc = 0;
+            Storage& gs = g.grad_for_write(self, &acc);
+            if (gs.dtype != go.dtype) throw Error("add/mul backward: gradient element types differ (parameter operand in mixed precision)");
+            const Storage od = g.compute_data(other);
+            if (self_shape == os) {
+                if (is_mul) {
+                    // ga (+)= other * go, expressed through mul_backward with the other side disabled
+                    if (other_st == compute_strides(os)) {
+                        g.check(eisen_hip_mul_backward(g.ctx(), od.ptr, od.ptr, go.ptr, gs.ptr, nullptr, dtype, n, acc, 0), "mul backward");
+                    } else {
+                        const std::vector<size_t> full = compute_strides(os);
+                        g.check(eisen_hip_bcast_backward(g.ctx(), gs.ptr, go.ptr, od.ptr, dtype, (int)os.size(), os.data(), full.data(), other_st.data(), n, acc), "mul backward");
+                    }
+                } else {
+                    g.check(eisen_hip_accumulate(g.ctx(), gs.ptr, go.ptr, dtype, n, acc), "add backward");
+                }
+            } else {
+                const std::vector<size_t> osv = os.empty() ? std::vector<size_t>{1} : os;
+                g.check(eisen_hip_bcast_backward(g.ctx(), gs.ptr, go.ptr, is_mul ? od.ptr : nullptr, dtype, (int)osv.size(), osv.data(), self_st.data(),
+                                                 is_mul ? other_st.data() : nullptr, numel_of(self_shape), acc),
+                        "broadcast backward");
+            }
+        };
+        one_side(a, b, sa, sta, stb);  // when a == b both contributions land on the same buffer
+        one_side(b, a, sb, stb, sta);
+    });
+    return out;
+}
+size_t Graph::add(size_t a, size_t b) { return elementwise_binary(a, b, false); }
+size_t Graph::mul(size_t a, size_t b) { return elementwise_binary(a, b, true); }
+
+// Graph::silu (src/graph/ops/elementwise.rs:337-465).
+size_t Graph::silu(size_t a) {
+    const Storage da = compute_data(a);
+    const size_t out = push_tensor(at(a).shape, da.dtype, true);
+    check(eisen_hip_silu(ctx_, da.ptr, at(out).data.ptr, da.dtype, da.numel), "silu");
+    record({a}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& ga = g.grad_for_write(a, &acc);
+        g.check(eisen_hip_silu_backward(g.ctx(), g.compute_data(a).ptr, go.ptr, ga.ptr, go.dtype, go.numel, acc), "silu backward");
+    });
+    return out;
+}
+
+// silu(gate) * up in one pass each way: the gate/silu/up/mul part of
+// TransformerBlock::forward_with_mask (src/nn/transformer.rs:40-43).
+size_t Graph::swiglu(size_t gate, size_t up) {
+    const Storage dg = compute_data(gate), du = compute_data(up);
+    if (at(gate).shape != at(up).shape || dg.dtype != du.dtype) throw Error("swiglu: gate and up must have the same shape and type");
+    const size_t out = push_tensor(at(gate).shape, dg.dtype, true);
+    check(eisen_hip_swiglu(ctx_, dg.ptr, du.ptr, at(out).data.ptr, dg.dtype, dg.numel), "swiglu");
+    record({gate, up}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int ag = 0, au = 0;
+        Storage& gg = g.grad_for_write(gate, &ag);
+        Storage& gu = g.grad_for_write(up, &au);
+        g.check(eisen_hip_swiglu_backward(g.ctx(), g.compute_data(gate).ptr, g.compute_data(up).ptr, go.ptr, gg.ptr, gu.ptr, go.dtype, go.numel, ag, au),
+                "swiglu backward");
+    });
+    return out;
+}
+
+// ---- contractions --------------------------------------------------------------------------------
+
+// Graph::matmul / matmul_bf16 (src/graph/ops/linear.rs:8-297, :526-656): a [..., K] flattened to
+// [M, K], b [K, N] -> [M, N].  dA += dC B^T, dB += A^T dC.
+size_t Graph::matmul(size_t a, size_t b) {
+    const std::vector<size_t> sa = at(a).shape, sb = at(b).shape;
+    if (sb.size() != 2 || sa.empty()) throw Error("matmul: expects a [..,K] and b [K,N], got " + shape_str(sa) + " x " + shape_str(sb));
+    const size_t K = sa.back(), M = numel_of(sa) / std::max<size_t>(K, 1), N = sb[1];
+    if (sb[0] != K) throw Error("matmul: inner dimensions differ: " + shape_str(sa) + " x " + shape_str(sb));
+    const Storage da = compute_data(a), db = compute_data(b);
+    if (da.dtype != db.dtype) throw Error("matmul: operands have different element types");
+    const size_t out = push_tensor({M, N}, da.dtype, true);
+    check(eisen_hip_gemm(ctx_, da.ptr, db.ptr, at(out).data.ptr, da.dtype, da.dtype, 0, 0, M, N, K, 0), "matmul");
+    record({a, b}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& ga = g.grad_for_write(a, &acc);
+        g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc), "matmul backward dA");
+        Storage& gb = g.grad_for_write(b, &acc);
+        g.check(eisen_hip_gemm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul backward dB");
+    });
+    return out;
+}
+
+// Graph::matmul_trans_b (src/graph/ops/linear.rs:301-523; GPU arm semantics): C = A B^T with
+// b stored [N, K]; dA += dC B, dB += dC^T A.  Leading dims of a are kept.
+size_t Graph::matmul_trans_b(size_t a, size_t b) {
+    const std::vector<size_t> sa = at(a).shape, sb = at(b).shape;
+    if (sb.size() != 2 || sa.empty()) throw Error("matmul_trans_b: expects a [..,K] and b [N,K]");
+    const size_t K = sa.back(), M = numel_of(sa) / std::max<size_t>(K, 1), N = sb[0];
+    if (sb[1] != K) throw Error("matmul_trans_b: inner dimensions differ: " + shape_str(sa) + " x " + shape_str(sb) + "^T");
+    const Storage da = compute_data(a), db = compute_data(b);
+    if (da.dtype != db.dtype) throw Error("matmul_trans_b: operands have different element types");
+    std::vector<size_t> os = sa;
+    os.back() = N;
+    const size_t out = push_tensor(os, da.dtype, true);
+    check(eisen_hip_gemm(ctx_, da.ptr, db.ptr, at(out).data.ptr, da.dtype, da.dtype, 0, 1, M, N, K, 0), "matmul_trans_b");
+    record({a, b}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& ga = g.grad_for_write(a, &acc);
+        g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 0, M, K, N, acc), "matmul_trans_b backward dA");
+        Storage& gb = g.grad_for_write(b, &acc);
+        g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(a).ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, N, K, M, acc), "matmul_trans_b backward dB");
+    });
+    return out;
+}
+
+// Graph::bmm (src/graph/ops/linear.rs:1198-1511): a [B,M,K]; b [B,N,K] if trans_b else [B,K,N].
+size_t Graph::bmm(size_t a, size_t b, bool trans_b) {
+    const std::vector<size_t> sa = at(a).shape, sb = at(b).shape;
+    if (sa.size() != 3 || sb.size() != 3 || sa[0] != sb[0]) throw Error("bmm: expects [B,M,K] and [B,N,K]/[B,K,N]");
+    const size_t B = sa[0], M = sa[1], K = sa[2], N = trans_b ? sb[1] : sb[2];
+    if ((trans_b ? sb[2] : sb[1]) != K) throw Error("bmm: inner dimensions differ");
+    const Storage da = compute_data(a), db = compute_data(b);
+    if (da.dtype != db.dtype) throw Error("bmm: operands have different element types");
+    const size_t out = push_tensor({B, M, N}, da.dtype, true);
+    check(eisen_hip_bmm(ctx_, da.ptr, db.ptr, at(out).data.ptr, da.dtype, da.dtype, 0, trans_b ? 1 : 0, B, M, N, K, 0), "bmm");
+    record({a, b}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& ga = g.grad_for_write(a, &acc);
+        // dA = dC * B (trans_b: B is [N,K]) or dC * B^T (B is [K,N])
+        g.check(eisen_hip_bmm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, trans_b ? 0 : 1, B, M, K, N, acc), "bmm backward dA");
+        Storage& gb = g.grad_for_write(b, &acc);
+        if (trans_b)  // dB [N,K] = dC^T * A
+            g.check(eisen_hip_bmm(g.ctx(), go.ptr, g.compute_data(a).ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, B, N, K, M, acc), "bmm backward dB");
+        else          // dB [K,N] = A^T * dC
+            g.check(eisen_hip_bmm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, B, K, N, M, acc), "bmm backward dB");
+    });
+    return out;
+}
+
+// ---- reductions / loss ---------------------------------------------------------------------------
+
+// Graph::softmax (src/graph/ops/reduction.rs:397-523), over the last dim.
+size_t Graph::softmax(size_t a) {
+    const std::vector<size_t> sa = at(a).shape;
+    if (sa.empty()) throw Error("softmax: scalar input");
+    const size_t n = sa.back(), rows = numel_of(sa) / std::max<size_t>(n, 1);
+    const Storage da = compute_data(a);
+    const size_t out = push_tensor(sa, da.dtype, true);
+    check(eisen_hip_softmax(ctx_, da.ptr, at(out).data.ptr, da.dtype, rows, n), "softmax");
+    record({a}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& ga = g.grad_for_write(a, &acc);
+        g.check(eisen_hip_softmax_backward(g.ctx(), g.at(out).data.ptr, go.ptr, ga.ptr, go.dtype, rows, n, acc), "softmax backward");
+    });
+    return out;
+}
+
+// Graph::cross_entropy_masked (src/graph/ops/reduction.rs:724-944); Graph::cross_entropy is the
+// case without masked rows (:529-716).  The gradient of the logits is produced by the forward
+// kernel in the same pass; the recorded backward only rescales it when the loss is not the root.
+size_t Graph::cross_entropy_masked(size_t logits, const std::vector<int64_t>& targets) {
+    const std::vector<size_t> sl = at(logits).shape;
+    if (sl.size() != 2) throw Error("cross_entropy: logits must be [rows, classes], got " + shape_str(sl));
+    const size_t rows = sl[0], classes = sl[1];
+    if (targets.size() != rows) throw Error("cross_entropy: " + std::to_string(targets.size()) + " targets for " + std::to_string(rows) + " rows");
+    std::vector<int32_t> t32(rows);
+    size_t valid = 0;
+    for (size_t i = 0; i < rows; i++) {
+        if (targets[i] == (int64_t)-1) {
+            t32[i] = EISEN_IGNORE_INDEX;
+        } else {
+            if (targets[i] < 0 || (size_t)targets[i] >= classes)
+                throw Error("cross_entropy: target " + std::to_string(targets[i]) + " at row " + std::to_string(i) + " outside [0, " + std::to_string(classes) + ")");
+            t32[i] = (int32_t)targets[i];
+            valid++;
+        }
+    }
+    const size_t out = push_tensor({}, EISEN_F32, true);
+    if (valid == 0) {  // src/graph/ops/reduction.rs:737-741: zero loss, no tape node
+        check(eisen_hip_fill(ctx_, at(out).data.ptr, EISEN_F32, 0.0f, 1), "cross_entropy");
+        return out;
+    }
+    const float normalizer = 1.0f / (float)valid;
+    const Storage dl = compute_data(logits);
+    Storage tgt = device_alloc(rows, EISEN_F32, false);  // int32 payload
+    check(eisen_hip_htod(ctx_, tgt.ptr, t32.data(), rows * sizeof(int32_t)), "cross_entropy targets");
+    Storage row_loss = device_alloc(rows, EISEN_F32, false);
+    // Fast path: the logits are a fresh activation, so their gradient buffer is created here and the
+    // kernel writes straight into it.  Otherwise (a leaf that already owns a gradient, or no_grad) the
+    // gradient goes to a pooled side tensor and is added in backward.
+    Tensor& tl = at(logits);
+    const bool direct = !no_grad && !tl.is_param && !tl.grad.valid();
+    size_t side = (size_t)-1;
+    void* dlogits = nullptr;
+    if (direct) {
+        int acc = 0;
+        dlogits = grad_for_write(logits, &acc).ptr;
+    } else {
+        side = push_tensor(sl, dl.dtype, true);
+        dlogits = at(side).data.ptr;
+    }
+    check(eisen_hip_cross_entropy(ctx_, dl.ptr, (const int32_t*)tgt.ptr, dlogits, (float*)row_loss.ptr, (float*)at(out).data.ptr, nullptr, nullptr,
+                                  dl.dtype, rows, classes, normalizer, 1.0f),
+          "cross_entropy");
+    device_free(tgt);  // stream-ordered: reused only by later work
+    device_free(row_loss);
+    record({logits}, out, [=](Graph& g) {
+        const bool scale = g.backward_root() != out;  // seed 1: the stored gradient is already final
+        if (direct) {
+            if (!scale) return;
+            Storage& gl = g.at(logits).grad;
+            g.check(eisen_hip_scale_by_device_scalar(g.ctx(), gl.ptr, gl.dtype, (const float*)g.grad_for_read(out).ptr, gl.numel), "cross_entropy backward");
+            return;
+        }
+        Storage& sd = g.at(side).data;
+        if (scale) g.check(eisen_hip_scale_by_device_scalar(g.ctx(), sd.ptr, sd.dtype, (const float*)g.grad_for_read(out).ptr, sd.numel), "cross_entropy backward");
+        int acc = 0;
+        Storage& gl = g.grad_for_write(logits, &acc);
+        if (gl.dtype == sd.dtype) {
+            g.check(eisen_hip_accumulate(g.ctx(), gl.ptr, sd.ptr, sd.dtype, sd.numel, acc), "cross_entropy backward");
+        } else {  // f32 leaf gradient, bf16 logits
+            Storage tmp = g.device_alloc(sd.numel, gl.dtype, false);
+            g.check(eisen_hip_cast(g.ctx(), sd.ptr, sd.dtype, tmp.ptr, gl.dtype, sd.numel), "cross_entropy backward");
+            g.check(eisen_hip_accumulate(g.ctx(), gl.ptr, tmp.ptr, gl.dtype, sd.numel, acc), "cross_entropy backward");
+            g.device_free(tmp);
+        }
+    });
+    return out;
+}
+size_t Graph::cross_entropy(size_t logits, const std::vector<int64_t>& targets) {
+    for (int64_t t : targets)
+        if (t == (int64_t)-1) throw Error("cross_entropy: IGNORE_INDEX target; use cross_entropy_masked");
+    return cross_entropy_masked(logits, targets);
+}
+
+// ---- layout --------------------------------------------------------------------------------------
+
+// Graph::transpose_0213 (src/graph/ops/transform.rs:7-127).
+size_t Graph::transpose_0213(size_t a) {
+    const std::vector<size_t> sa = at(a).shape;
+    if (sa.size() != 4) throw Error("transpose_0213 requires a 4-D tensor");
+    const size_t b = sa[0], s = sa[1], h = sa[2], d = sa[3];
+    const Storage da = compute_data(a);
+    const size_t out = push_tensor({b, h, s, d}, da.dtype, true);
+    check(eisen_hip_transpose_0213(ctx_, da.ptr, at(out).data.ptr, da.dtype, b, s, h, d, 0), "transpose_0213");
+    record({a}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& ga = g.grad_for_write(a, &acc);
+        g.check(eisen_hip_transpose_0213(g.ctx(), go.ptr, ga.ptr, go.dtype, b, h, s, d, acc), "transpose_0213 backward");
+    });
+    return out;
+}
+
+// Graph::gather (src/graph/ops/transform.rs:132-324).  Indices are a tensor of f32 ids loaded from
+// the host (`as usize` truncation, :294); their host copy drives the deterministic backward.
+size_t Graph::gather(size_t weights, size_t indices) {
+    const std::vector<size_t> sw = at(weights).shape;
+    if (sw.size() != 2) throw Error("gather: weights must be [vocab, hidden]");
+    const size_t vocab = sw[0], hidden = sw[1];
+    Tensor& ti = at(indices);
+    const size_t n = ti.size();
+    if (ti.host_copy.size() != n) {
+        std::vector<float> host = sync_to_cpu(indices);  // ids that never came from the host: read them back
+        at(indices).host_copy = host;
+    }
+    std::vector<int32_t> ids(n);
+    const std::vector<float>& hc = at(indices).host_copy;
+    for (size_t i = 0; i < n; i++) {
+        const float f = hc[i];
+        if (!(f >= 0.0f) || (size_t)f >= vocab) throw Error("gather: index " + std::to_string(f) + " at position " + std::to_string(i) + " outside [0, " + std::to_string(vocab) + ")");
+        ids[i] = (int32_t)f;
+    }
+    const Storage dw = compute_data(weights);
+    std::vector<size_t> os = at(indices).shape;
+    os.push_back(hidden);
+    const size_t out = push_tensor(os, dw.dtype, true);
+    Storage dids = device_alloc(n, EISEN_F32, false);  // int32 payload
+    check(eisen_hip_htod(ctx_, dids.ptr, ids.data(), n * sizeof(int32_t)), "gather ids");
+    check(eisen_hip_gather(ctx_, dw.ptr, (const int32_t*)dids.ptr, at(out).data.ptr, dw.dtype, n, vocab, hidden), "gather");
+    device_free(dids);
+    record({weights, indices}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        g.materialize_grad(weights);  // the scatter touches only the rows that occur
+        Tensor& w = g.at(weights);
+        if (!w.is_param) {
+            int acc = 0;
+            Storage& gw0 = g.grad_for_write(weights, &acc);
+            if (!acc) g.check(eisen_hip_memset_zero(g.ctx(), gw0.ptr, gw0.numel * (gw0.dtype == EISEN_BF16 ? 2 : 4)), "gather backward");
+        }
+        if (w.grad.dtype != EISEN_F32) throw Error("gather backward: the embedding gradient must be f32");
+        g.check(eisen_hip_gather_backward(g.ctx(), ids.data(), go.ptr, (float*)w.grad.ptr, go.dtype, n, vocab, hidden), "gather backward");
+    });
+    return out;
+}
+
+// Graph::reshape (src/graph/ops/transform.rs:329-406): a copy with a new shape.
+size_t Graph::reshape(size_t a, const std::vector<size_t>& shape) {
+    if (numel_of(shape) != at(a).size()) throw Error("reshape: element count mismatch");
+    const Storage da = compute_data(a);
+    const size_t out = push_tensor(shape, da.dtype, true);
+    check(eisen_hip_dtod(ctx_, at(out).data.ptr, da.ptr, da.numel * (da.dtype == EISEN_BF16 ? 2 : 4)), "reshape");
+    record({a}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& ga = g.grad_for_write(a, &acc);
+        if (ga.dtype != go.dtype) throw Error("reshape backward: gradient element types differ");
+        g.check(eisen_hip_accumulate(g.ctx(), ga.ptr, go.ptr, go.dtype, go.numel, acc), "reshape backward");
+    });
+    return out;
+}
+
+// Graph::rope (src/graph/ops/transform.rs:467-610): a [batch, seq, hidden].
+size_t Graph::rope(size_t a, size_t head_dim) {
+    const std::vector<size_t> sa = at(a).shape;
+    if (sa.size() != 3) throw Error("rope: expects [batch, seq, hidden]");
+    const Storage da = compute_data(a);
+    const size_t out = push_tensor(sa, da.dtype, true);
+    check(eisen_hip_rope(ctx_, da.ptr, at(out).data.ptr, da.dtype, sa[0], sa[1], sa[2], head_dim), "rope");
+    record({a}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& ga = g.grad_for_write(a, &acc);
+        g.check(eisen_hip_rope_backward(g.ctx(), go.ptr, ga.ptr, go.dtype, sa[0], sa[1], sa[2], head_dim, acc), "rope backward");
+    });
+    return out;
+}
+
+// Graph::rms_norm (src/graph/ops/normalization.rs:8-184): the gain is an f32 parameter.
+size_t Graph::rms_norm(size_t x, size_t w, float eps) {
+    const std::vector<size_t> sx = at(x).shape;
+    if (sx.empty()) throw Error("rms_norm: scalar input");
+    const size_t dim = sx.back(), rows = numel_of(sx) / std::max<size_t>(dim, 1);
+    if (at(w).size() != dim || at(w).data.dtype != EISEN_F32) throw Error("rms_norm: weight must be an f32 vector of the last dimension");
+    const Storage dx = compute_data(x);
+    const size_t out = push_tensor(sx, dx.dtype, true);
+    const size_t rr = push_tensor({rows}, EISEN_F32, true);  // reciprocal RMS per row, kept for backward
+    check(eisen_hip_rms_norm(ctx_, dx.ptr, (const float*)at(w).data.ptr, at(out).data.ptr, (float*)at(rr).data.ptr, dx.dtype, rows, dim, eps), "rms_norm");
+    record({x, w}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& gx = g.grad_for_write(x, &acc);
+        g.materialize_grad(w);
+        Tensor& tw = g.at(w);
+        if (!tw.grad.valid() || tw.grad.dtype != EISEN_F32) throw Error("rms_norm backward: the gain needs an f32 gradient buffer");
+        g.check(eisen_hip_rms_norm_backward(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr, (const float*)g.at(rr).data.ptr, go.ptr, gx.ptr,
+                                            (float*)tw.grad.ptr, go.dtype, rows, dim, acc),
+                "rms_norm backward");
+    });
+    return out;
+}
+
+// Graph::repeat_kv (src/graph/ops/gqa.rs:13-194).
+size_t Graph::repeat_kv(size_t x, size_t repeats) {
+    const std::vector<size_t> sx = at(x).shape;
+    if (sx.size() != 4) throw Error("repeat_kv requires [Batch, KVHeads, SeqLen, HeadDim]");
+    if (repeats == 1) return x;
+    const Storage dx = compute_data(x);
+    const size_t out = push_tensor({sx[0], sx[1] * repeats, sx[2], sx[3]}, dx.dtype, true);
+    check(eisen_hip_repeat_kv(ctx_, dx.ptr, at(out).data.ptr, dx.dtype, sx[0], sx[1], sx[2], sx[3], repeats), "repeat_kv");
+    record({x}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& gx = g.grad_for_write(x, &acc);
+        g.check(eisen_hip_repeat_kv_backward(g.ctx(), go.ptr, gx.ptr, go.dtype, sx[0], sx[1], sx[2], sx[3], repeats, acc), "repeat_kv backward");
+    });
+    return out;
+}
+
+// ---- attention -----------------------------------------------------------------------------------
+
+size_t Graph::attention_impl(size_t q, size_t k, size_t v, size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd, const long long* qs,
+                             const long long* ks, float scale, bool causal, const std::vector<size_t>& out_shape) {
+    Graph& g = *this;
+    const Storage dq = g.compute_data(q), dk = g.compute_data(k), dv = g.compute_data(v);
+    if (dq.dtype != dk.dtype || dq.dtype != dv.dtype) throw Error("attention: q, k, v must share an element type");
+    const size_t out = g.alloc_pooled_dtype(out_shape, dq.dtype);
+    const size_t lse = g.alloc_pooled_dtype({B, Hq, S}, EISEN_F32);  // log-sum-exp per query row, kept for backward
+    std::vector<long long> qsv, ksv;
+    if (qs) qsv.assign(qs, qs + 3);
+    if (ks) ksv.assign(ks, ks + 3);
+    g.check(eisen_hip_attention_forward(g.ctx(), dq.ptr, dk.ptr, dv.ptr, g.at(out).data.ptr, (float*)g.at(lse).data.ptr, dq.dtype, B, S, Hq, Hkv, hd,
+                                        qs ? qsv.data() : nullptr, ks ? ksv.data() : nullptr, scale, causal ? 1 : 0),
+            "attention forward");
+    record({q, k, v}, out, [=](Graph& gg) {
+        const Storage& go = gg.grad_for_read(out);
+        int aq = 0, ak = 0, av = 0;
+        // the kernels overwrite: route through temporaries when a gradient is already there
+        Storage& gq = gg.grad_for_write(q, &aq);
+        Storage& gk = gg.grad_for_write(k, &ak);
+        Storage& gv = gg.grad_for_write(v, &av);
+        if (aq || ak || av) throw Error("attention backward: q, k, v must not have other consumers");
+        gg.check(eisen_hip_attention_backward(gg.ctx(), gg.compute_data(q).ptr, gg.compute_data(k).ptr, gg.compute_data(v).ptr, gg.at(out).data.ptr, go.ptr,
+                                              (const float*)gg.at(lse).data.ptr, gq.ptr, gk.ptr, gv.ptr, go.dtype, B, S, Hq, Hkv, hd,
+                                              qsv.empty() ? nullptr : qsv.data(), ksv.empty() ? nullptr : ksv.data(), scale, causal ? 1 : 0),
+                 "attention backward");
+    });
+    return out;
+}
+
+size_t Graph::attention_gqa(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal) {
+    const std::vector<size_t> sq = at(q).shape, sk = at(k).shape;
+    if (sq.size() != 3 || sk.size() != 3 || at(v).shape != sk) throw Error("attention_gqa: expects q [B,S,Hq*hd], k/v [B,S,Hkv*hd]");
+    if (heads == 0 || kv_heads == 0 || sq[2] % heads || heads % kv_heads) throw Error("attention_gqa: bad head counts");
+    const size_t hd = sq[2] / heads;
+    if (sk[2] != kv_heads * hd || sk[0] != sq[0] || sk[1] != sq[1]) throw Error("attention_gqa: k/v shape does not match q");
+    return attention_impl(q, k, v, sq[0], sq[1], heads, kv_heads, hd, nullptr, nullptr, scale, causal, sq);
+}
+
+size_t Graph::flash_attention(size_t q, size_t k, size_t v, float scale, bool causal) {
+    const std::vector<size_t> sq = at(q).shape, sk = at(k).shape, sv = at(v).shape;
+    if (sq.size() != 3) throw Error("flash_attention expects q=[B,M,D]");
+    if (sk.size() != 3) throw Error("flash_attention expects k=[B,N,D]");
+    if (sv.size() != 3) throw Error("flash_attention expects v=[B,N,D]");
+    if (sk[0] != sq[0] || sv[0] != sq[0]) throw Error("flash_attention batch mismatch");
+    if (sk[2] != sq[2] || sv[2] != sq[2]) throw Error("flash_attention head dim mismatch");
+    if (sv[1] != sk[1]) throw Error("flash_attention sequence mismatch k/v");
+    if (sq[2] > 256) throw Error("flash_attention kernel currently supports head_dim <= 256");
+    if (sk[1] != sq[1]) throw Error("flash_attention: this backend needs M == N (self-attention)");
+    const long long st[3] = {(long long)(sq[1] * sq[2]), (long long)sq[2], 0};
+    return attention_impl(q, k, v, sq[0], sq[1], 1, 1, sq[2], st, st, scale, causal, sq);
+}
+
+}  // namespace eisen

@@ -1,0 +1,159 @@
+// Host side of the Device::Gpu backend: Graph / Tensor / Tape with the reference's operator
+// interface (src/graph/mod.rs, src/graph/ops/*.rs, src/tensor.rs, src/tape.rs), written against
+// the public C-ABI of include/eisen_hip.h only -- every device action below is one eisen_hip_* call.
+//
+// Differences from the reference that a caller can observe are limited to what its GPU arm
+// could not do: attention and SwiGLU have fused ops with gradients, activation gradients are
+// bf16 in mixed mode, parameters keep f32 master weights next to a bf16 copy, and nothing
+// synchronises the stream unless the caller reads a value back.
+#pragma once
+#include <cstdint>
+#include <functional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "eisen_hip.h"
+
+namespace eisen {
+
+// src/graph/mod.rs:48-53
+enum class PrecisionMode { Fp32 = 0, Bf16Mixed = 1 };
+
+struct Error : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+// src/tensor.rs:35-44 `Storage`: one device allocation and its element type.
+struct Storage {
+    void* ptr = nullptr;
+    size_t numel = 0;
+    int dtype = EISEN_F32;
+    bool valid() const { return ptr != nullptr; }
+};
+
+// src/tensor.rs:132-142 `Tensor` (public fields are API: shape/strides/data/grad/name/is_pooled).
+struct Tensor {
+    size_t id = 0;
+    std::vector<size_t> shape, strides;
+    Storage data;            // activations: f32 or bf16; parameters: f32 master
+    Storage grad;            // parameters: f32, allocated with the tensor; activations: lazily, activation dtype
+    Storage shadow;          // parameters in Bf16Mixed: bf16 copy of `data` the kernels read
+    std::string name;
+    bool is_pooled = false;
+    bool is_param = false;        // allocated through alloc()/alloc_param_bf16(): owns an f32 grad
+    bool grad_written = false;    // this backward pass already stored into grad (next store accumulates)
+    bool grad_zero_pending = false;  // zero_grad() was requested; materialised on first use
+    std::vector<float> host_copy;    // kept for small host-loaded tensors (token ids)
+    size_t size() const {
+        size_t n = 1;
+        for (size_t s : shape) n *= s;
+        return n;
+    }
+};
+
+class Graph;
+
+// src/tape.rs:3-7
+struct TapeNode {
+    std::vector<size_t> inputs;
+    size_t output;
+    std::function<void(Graph&)> backward_fn;
+};
+struct Tape {
+    std::vector<TapeNode> nodes;
+};
+
+class Graph {
+   public:
+    std::vector<Tensor> tensors;
+    Tape tape;
+    size_t num_params = 0;
+    bool no_grad = false;
+    PrecisionMode precision_mode;
+
+    Graph(eisen_ctx* ctx, PrecisionMode mode);
+    ~Graph();
+    Graph(const Graph&) = delete;
+    Graph& operator=(const Graph&) = delete;
+
+    eisen_ctx* ctx() const { return ctx_; }
+    int act_dtype() const { return precision_mode == PrecisionMode::Bf16Mixed ? EISEN_BF16 : EISEN_F32; }
+    bool uses_bf16_mixed_precision() const { return precision_mode == PrecisionMode::Bf16Mixed; }
+
+    // ---- runtime (src/graph/mod.rs:317-598) ------------------------------------------------
+    void name_tensor(size_t id, const std::string& name) { at(id).name = name; }
+    void mark_params() { num_params = tensors.size(); }
+    size_t mark_save_point() const { return tensors.size(); }
+    void restore_save_point(size_t save_point);
+    void clear_activations();
+    size_t alloc(const std::vector<size_t>& shape, const std::vector<float>& data);
+    size_t alloc(const std::vector<size_t>& shape, const float* data, size_t n);
+    size_t alloc_pooled(const std::vector<size_t>& shape);
+    size_t alloc_pooled_dtype(const std::vector<size_t>& shape, int dtype);   // pooled buffer of an explicit element type
+    size_t alloc_param_bf16(const std::vector<size_t>& shape, const std::vector<float>& data) { return alloc(shape, data); }
+    void load_tensor_data(size_t id, const float* host, size_t n);
+    std::vector<float> sync_to_cpu(size_t id);
+    std::vector<float> sync_grad_to_cpu(size_t id);
+    void reinterpret_shape(size_t id, const std::vector<size_t>& shape);
+    void synchronize();
+
+    // ---- ops (src/graph/ops/*.rs); all return the output tensor id ------------------------------
+    size_t add(size_t a, size_t b);
+    size_t mul(size_t a, size_t b);
+    size_t silu(size_t a);
+    size_t swiglu(size_t gate, size_t up);                      // fused silu(gate) * up
+    size_t matmul(size_t a, size_t b);
+    size_t matmul_bf16(size_t a, size_t b) { return matmul(a, b); }
+    size_t matmul_trans_b(size_t a, size_t b);
+    size_t bmm(size_t a, size_t b, bool trans_b);
+    size_t softmax(size_t a);
+    size_t cross_entropy(size_t logits, const std::vector<int64_t>& targets);
+    size_t cross_entropy_masked(size_t logits, const std::vector<int64_t>& targets);
+    size_t transpose_0213(size_t a);
+    size_t gather(size_t weights, size_t indices);
+    size_t reshape(size_t a, const std::vector<size_t>& shape);
+    size_t rope(size_t a, size_t head_dim);
+    size_t rms_norm(size_t x, size_t w, float eps);
+    size_t repeat_kv(size_t x, size_t repeats);
+    // Reference signature (src/graph/ops/attention.rs:7-14): q [B,M,D], k/v [B,N,D], M == N here.
+    // Unlike the reference it also records a backward.
+    size_t flash_attention(size_t q, size_t k, size_t v, float scale, bool causal);
+    // q [B,S,Hq*hd], k/v [B,S,Hkv*hd] straight from the projections -> [B,S,Hq*hd].
+    size_t attention_gqa(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal);
+
+    // src/graph/mod.rs:670-796
+    void backward(size_t loss_id);
+
+    // ---- helpers for optimisers and backward closures -----------------------------------------
+    Tensor& at(size_t id);
+    // Gradient buffer of `id` for a store; *accumulate tells the kernel whether to add.
+    Storage& grad_for_write(size_t id, int* accumulate);
+    // Gradient as an input (must have been written).
+    const Storage& grad_for_read(size_t id);
+    void materialize_grad(size_t id);      // apply a pending zero_grad
+    void request_zero_grad(size_t id);     // AdamW::zero_grad, lazily
+    const Storage& compute_data(size_t id);   // what kernels read: bf16 shadow for mixed-mode params
+    void refresh_shadow(size_t id);           // re-cast the master weight into the bf16 copy
+    void check(int rc, const char* what) const;
+    size_t backward_root() const { return backward_root_; }
+
+   private:
+    eisen_ctx* ctx_;
+    size_t backward_root_ = (size_t)-1;
+    size_t push_tensor(const std::vector<size_t>& shape, int dtype, bool pooled);
+    Storage device_alloc(size_t numel, int dtype, bool zero);
+    void device_free(Storage& s);
+    void release(Tensor& t);
+    void record(std::vector<size_t> inputs, size_t output, std::function<void(Graph&)> fn);
+    size_t elementwise_binary(size_t a, size_t b, bool is_mul);
+    size_t attention_impl(size_t q, size_t k, size_t v, size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd, const long long* qs,
+                          const long long* ks, float scale, bool causal, const std::vector<size_t>& out_shape);
+};
+
+std::vector<size_t> compute_strides(const std::vector<size_t>& shape);                      // src/tensor.rs:225-233
+std::vector<size_t> broadcasted_shape(const std::vector<size_t>& a, const std::vector<size_t>& b);  // :235-244
+std::vector<size_t> broadcasted_strides(const std::vector<size_t>& shape, const std::vector<size_t>& base,
+                                        const std::vector<size_t>& out_shape);              // :246-260
+
+}  // namespace eisen

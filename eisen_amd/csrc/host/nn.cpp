@@ -1,0 +1,356 @@
+#include "nn.hpp"
+
+#include <cmath>
+#include <cstring>
+
+namespace eisen {
+
+namespace {
+// f32::powi -> compiler-rt __powisf2 (square and multiply), as AdamW::step uses it (src/nn/optim.rs:337-338).
+float powi_f32(float a, int b) {
+    const bool recip = b < 0;
+    float r = 1.0f;
+    while (true) {
+        if (b & 1) r *= a;
+        b /= 2;
+        if (b == 0) break;
+        a *= a;
+    }
+    return recip ? 1.0f / r : r;
+}
+}  // namespace
+
+// Linear::new (src/nn/linear.rs:10-50): the same seed-42 LCG for every layer.
+Linear::Linear(Graph& g, size_t in_features, size_t out_features, bool use_bias) {
+    const size_t n = in_features * out_features;
+    std::vector<float> w(n);
+    const float stdv = 0.02f;
+    uint32_t seed = 42;
+    const float umax = (float)UINT32_MAX;
+    for (size_t i = 0; i < n; i++) {
+        const float u1 = std::fmin((float)seed / umax + 1e-7f, 1.0f - 1e-7f);
+        seed = seed * 1664525u + 1013904223u;
+        const float u2 = std::fmin(std::fmax((float)seed / umax, 1e-7f), 1.0f - 1e-7f);
+        seed = seed * 1664525u + 1013904223u;
+        const float mag = std::sqrt(-2.0f * std::log(u1));
+        w[i] = mag * std::cos(2.0f * 3.14159274101257324f * u2) * stdv;
+    }
+    weight_id = g.alloc({in_features, out_features}, w);
+    has_bias = use_bias;
+    if (use_bias) bias_id = g.alloc({out_features}, std::vector<float>(out_features, 0.0f));
+}
+
+// Linear::forward (src/nn/linear.rs:53-95): matmul over flattened rows, 3-D shape restored.
+size_t Linear::forward(Graph& g, size_t x_id) const {
+    const std::vector<size_t> xs = g.at(x_id).shape;
+    size_t out = g.matmul(x_id, weight_id);
+    if (has_bias) out = g.add(out, bias_id);
+    if (xs.size() == 3) g.reinterpret_shape(out, {xs[0], xs[1], g.at(weight_id).shape[1]});
+    return out;
+}
+std::vector<size_t> Linear::params() const {
+    std::vector<size_t> p{weight_id};
+    if (has_bias) p.push_back(bias_id);
+    return p;
+}
+
+// Embedding::new (src/nn/embedding.rs:9-31)
+Embedding::Embedding(Graph& g, size_t vocab_size, size_t hidden_dim) {
+    const size_t n = vocab_size * hidden_dim;
+    std::vector<float> w(n);
+    uint32_t seed = 84;
+    const float umax = (float)UINT32_MAX;
+    for (size_t i = 0; i < n; i++) {
+        seed = seed * 1664525u + 1013904223u;
+        w[i] = ((float)seed / umax * 2.0f - 1.0f) * 0.02f;
+    }
+    weight_id = g.alloc({vocab_size, hidden_dim}, w);
+}
+
+RMSNorm::RMSNorm(Graph& g, size_t dim, float eps_) : eps(eps_) { weight_id = g.alloc({dim}, std::vector<float>(dim, 1.0f)); }
+
+GroupedQueryAttention::GroupedQueryAttention(Graph& g, size_t hidden, size_t heads, size_t kv_heads) {
+    if (hidden % heads) throw Error("hidden_dim must be cleanly divisible by num_heads");
+    if (heads % kv_heads) throw Error("num_heads must be divisible by num_kv_heads");
+    num_heads = heads;
+    num_kv_heads = kv_heads;
+    head_dim = hidden / heads;
+    hidden_dim = hidden;
+    const size_t kv_dim = kv_heads * head_dim;
+    q_proj = Linear(g, hidden, hidden, false);
+    k_proj = Linear(g, hidden, kv_dim, false);
+    v_proj = Linear(g, hidden, kv_dim, false);
+    out_proj = Linear(g, hidden, hidden, false);
+}
+
+// GroupedQueryAttention::forward_with_mask (src/nn/attention.rs:289-388).
+size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool causal) const {
+    const std::vector<size_t> xs = g.at(x_id).shape;
+    if (xs.size() != 3) throw Error("GQA requires [Batch, Seq, Dim]");
+    const size_t batch = xs[0], seq = xs[1];
+    const size_t q = q_proj.forward(g, x_id), k = k_proj.forward(g, x_id), v = v_proj.forward(g, x_id);
+    const size_t q_rope = g.rope(q, head_dim), k_rope = g.rope(k, head_dim);
+    const float scale = 1.0f / std::sqrt((float)head_dim);
+    if (fused) {
+        // one op for steps 3-11: head split, GQA repeat, scores, scale, mask, softmax, P V, merge
+        const size_t ctx = g.attention_gqa(q_rope, k_rope, v, num_heads, num_kv_heads, scale, causal);
+        return out_proj.forward(g, ctx);
+    }
+    const size_t q4 = g.reshape(q_rope, {batch, seq, num_heads, head_dim});
+    const size_t k4 = g.reshape(k_rope, {batch, seq, num_kv_heads, head_dim});
+    const size_t v4 = g.reshape(v, {batch, seq, num_kv_heads, head_dim});
+    const size_t qt = g.transpose_0213(q4), kt = g.transpose_0213(k4), vt = g.transpose_0213(v4);
+    const size_t repeats = num_heads / num_kv_heads;
+    const size_t kr = g.repeat_kv(kt, repeats), vr = g.repeat_kv(vt, repeats);
+    const size_t bh = batch * num_heads;
+    g.reinterpret_shape(qt, {bh, seq, head_dim});
+    g.reinterpret_shape(kr, {bh, seq, head_dim});
+    g.reinterpret_shape(vr, {bh, seq, head_dim});
+    size_t ctx;
+    if (g.no_grad) {
+        ctx = g.flash_attention(qt, kr, vr, scale, causal);
+    } else {
+        const size_t scores = g.bmm(qt, kr, true);
+        // the reference uploads a full [bh, seq, seq] tensor of `scale`; a broadcast scalar is the same product
+        const size_t scale_id = g.alloc_pooled({1});
+        g.load_tensor_data(scale_id, &scale, 1);
+        size_t scaled = g.mul(scores, scale_id);
+        if (causal) {
+            std::vector<float> mask(seq * seq, 0.0f);
+            for (size_t r = 0; r < seq; r++)
+                for (size_t c = r + 1; c < seq; c++) mask[r * seq + c] = -1e20f;
+            const size_t mask_id = g.alloc_pooled({1, seq, seq});
+            g.load_tensor_data(mask_id, mask.data(), mask.size());
+            scaled = g.add(scaled, mask_id);
+        }
+        ctx = g.bmm(g.softmax(scaled), vr, false);
+    }
+    g.reinterpret_shape(ctx, {batch, num_heads, seq, head_dim});
+    const size_t ctx_t = g.transpose_0213(ctx);
+    const size_t ctx_flat = g.reshape(ctx_t, {batch, seq, hidden_dim});
+    return out_proj.forward(g, ctx_flat);
+}
+std::vector<size_t> GroupedQueryAttention::params() const {
+    return {q_proj.weight_id, k_proj.weight_id, v_proj.weight_id, out_proj.weight_id};
+}
+
+// TransformerBlock::new (src/nn/transformer.rs:19-28): allocation order norm1, attn, norm2, gate, ffn1, ffn2.
+TransformerBlock::TransformerBlock(Graph& g, size_t hidden, size_t heads, size_t kv_heads, size_t ffn_dim) {
+    norm1 = RMSNorm(g, hidden, 1e-5f);
+    attn = GroupedQueryAttention(g, hidden, heads, kv_heads);
+    norm2 = RMSNorm(g, hidden, 1e-5f);
+    ffn_gate = Linear(g, hidden, ffn_dim, false);
+    ffn1 = Linear(g, hidden, ffn_dim, false);
+    ffn2 = Linear(g, ffn_dim, hidden, false);
+}
+
+// TransformerBlock::forward_with_mask (src/nn/transformer.rs:31-49).
+size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) const {
+    const size_t norm1_out = norm1.forward(g, x_id);
+    const size_t attn_out = attn.forward_with_mask(g, norm1_out, causal);
+    const size_t res1 = g.add(x_id, attn_out);
+    const size_t norm2_out = norm2.forward(g, res1);
+    const size_t gate_out = ffn_gate.forward(g, norm2_out);
+    size_t gated;
+    if (attn.fused) {
+        const size_t up = ffn1.forward(g, norm2_out);
+        gated = g.swiglu(gate_out, up);
+    } else {
+        const size_t gate = g.silu(gate_out);
+        const size_t up = ffn1.forward(g, norm2_out);
+        gated = g.mul(gate, up);
+    }
+    const size_t ffn2_out = ffn2.forward(g, gated);
+    return g.add(res1, ffn2_out);
+}
+// params order (src/nn/transformer.rs:57-66): norm1, attn, norm2, ffn1, ffn2, ffn_gate
+std::vector<size_t> TransformerBlock::params() const {
+    std::vector<size_t> p{norm1.weight_id};
+    for (size_t id : attn.params()) p.push_back(id);
+    p.push_back(norm2.weight_id);
+    p.push_back(ffn1.weight_id);
+    p.push_back(ffn2.weight_id);
+    p.push_back(ffn_gate.weight_id);
+    return p;
+}
+
+// TransformerLM::new (src/nn/transformer.rs:78-117); nothing is demoted to the host here.
+TransformerLM::TransformerLM(Graph& g, size_t vocab, size_t hidden, size_t heads, size_t kv_heads, size_t ffn_dim, size_t layers, bool tie)
+    : tie_weights(tie), vocab_size(vocab) {
+    token_emb = Embedding(g, vocab, hidden);
+    blocks.reserve(layers);
+    for (size_t l = 0; l < layers; l++) blocks.emplace_back(g, hidden, heads, kv_heads, ffn_dim);
+    norm_f = RMSNorm(g, hidden, 1e-5f);
+    if (tie) {
+        lm_head.weight_id = token_emb.weight_id;
+        lm_head.has_bias = false;
+    } else {
+        lm_head = Linear(g, hidden, vocab, false);
+    }
+}
+
+std::vector<std::pair<std::string, size_t>> TransformerLM::named_params() const {
+    std::vector<std::pair<std::string, size_t>> out;
+    out.emplace_back("model.embed_tokens.weight", token_emb.weight_id);
+    for (size_t i = 0; i < blocks.size(); i++) {
+        const TransformerBlock& b = blocks[i];
+        const std::string p = "model.layers." + std::to_string(i) + ".";
+        out.emplace_back(p + "input_layernorm.weight", b.norm1.weight_id);
+        out.emplace_back(p + "self_attn.q_proj.weight", b.attn.q_proj.weight_id);
+        out.emplace_back(p + "self_attn.k_proj.weight", b.attn.k_proj.weight_id);
+        out.emplace_back(p + "self_attn.v_proj.weight", b.attn.v_proj.weight_id);
+        out.emplace_back(p + "self_attn.o_proj.weight", b.attn.out_proj.weight_id);
+        out.emplace_back(p + "post_attention_layernorm.weight", b.norm2.weight_id);
+        out.emplace_back(p + "mlp.gate_proj.weight", b.ffn_gate.weight_id);
+        out.emplace_back(p + "mlp.up_proj.weight", b.ffn1.weight_id);
+        out.emplace_back(p + "mlp.down_proj.weight", b.ffn2.weight_id);
+    }
+    out.emplace_back("model.norm.weight", norm_f.weight_id);
+    if (!tie_weights) out.emplace_back("lm_head.weight", lm_head.weight_id);
+    return out;
+}
+void TransformerLM::tag_parameters(Graph& g) const {
+    for (auto& kv : named_params()) g.name_tensor(kv.second, kv.first);
+}
+void TransformerLM::set_fused(bool fused) {
+    for (auto& b : blocks) b.attn.fused = fused;
+}
+
+// TransformerLM::forward (src/nn/transformer.rs:184-196).
+size_t TransformerLM::forward(Graph& g, size_t x_id) const {
+    size_t h = token_emb.forward(g, x_id);
+    for (const TransformerBlock& b : blocks) h = b.forward_with_mask(g, h, true);
+    h = norm_f.forward(g, h);
+    if (tie_weights) return g.matmul_trans_b(h, lm_head.weight_id);
+    return lm_head.forward(g, h);
+}
+std::vector<size_t> TransformerLM::params() const {
+    std::vector<size_t> p = token_emb.params();
+    for (const TransformerBlock& b : blocks)
+        for (size_t id : b.params()) p.push_back(id);
+    p.push_back(norm_f.weight_id);
+    if (!tie_weights) p.push_back(lm_head.weight_id);
+    return p;
+}
+
+// ---- AdamW (src/nn/optim.rs) -----------------------------------------------------------------------
+
+AdamW::AdamW(Graph& g, std::vector<size_t> params_, float lr_) : params(std::move(params_)), lr(lr_), g_(g) {
+    void* p = nullptr;
+    g_.check(eisen_hip_malloc_zeroed(g_.ctx(), 2 * sizeof(float), &p), "AdamW");
+    norm_dev_ = (float*)p;
+}
+AdamW::~AdamW() {
+    for (auto& s : m_)
+        if (s.ptr) eisen_hip_free(g_.ctx(), s.ptr);
+    for (auto& s : v_)
+        if (s.ptr) eisen_hip_free(g_.ctx(), s.ptr);
+    if (norm_dev_) eisen_hip_free(g_.ctx(), norm_dev_);
+}
+
+// AdamW::init_moments (src/nn/optim.rs:70-112): f32 first and second moments, zero.
+void AdamW::init_moments() {
+    if (!m_.empty()) return;
+    for (size_t id : params) {
+        const size_t n = g_.at(id).size();
+        Storage m, v;
+        m.numel = v.numel = n;
+        g_.check(eisen_hip_malloc_zeroed(g_.ctx(), std::max<size_t>(n, 1) * sizeof(float), &m.ptr), "AdamW moments");
+        g_.check(eisen_hip_malloc_zeroed(g_.ctx(), std::max<size_t>(n, 1) * sizeof(float), &v.ptr), "AdamW moments");
+        m_.push_back(m);
+        v_.push_back(v);
+    }
+}
+
+std::vector<eisen_param_slot> AdamW::slots() {
+    init_moments();
+    std::vector<eisen_param_slot> out;
+    for (size_t i = 0; i < params.size(); i++) {
+        Tensor& t = g_.at(params[i]);
+        if (!t.is_param || t.data.dtype != EISEN_F32) throw Error("AdamW: tensor " + std::to_string(params[i]) + " is not an f32 parameter");
+        eisen_param_slot s;
+        s.w = (float*)t.data.ptr;
+        s.g = (const float*)t.grad.ptr;
+        s.m = (float*)m_[i].ptr;
+        s.v = (float*)v_[i].ptr;
+        s.w_bf16 = t.shadow.ptr;
+        s.n = t.size();
+        if (s.n) out.push_back(s);
+    }
+    return out;
+}
+
+// AdamW::zero_grad (src/nn/optim.rs:207-245).  Deferred: the first gradient store of the next
+// backward overwrites instead of adding, so the buffers are not swept twice.
+void AdamW::zero_grad() {
+    for (size_t id : params) g_.request_zero_grad(id);
+}
+
+// AdamW::clip_grad_norm (src/nn/optim.rs:250-321): norm and coefficient are computed on the device
+// (f64 accumulation), gradients scaled in place when the coefficient is below 1.
+std::pair<float, float> AdamW::clip_grad_norm(float max_norm) {
+    for (size_t id : params) g_.materialize_grad(id);
+    std::vector<eisen_param_slot> s = slots();
+    g_.check(eisen_hip_grad_norm(g_.ctx(), s.data(), s.size(), max_norm, norm_dev_), "clip_grad_norm");
+    float host[2] = {0.f, 1.f};
+    g_.check(eisen_hip_dtoh(g_.ctx(), host, norm_dev_, sizeof(host)), "clip_grad_norm");
+    if (host[1] < 1.0f)
+        for (auto& slot : s) g_.check(eisen_hip_scale_by_device_scalar(g_.ctx(), (void*)slot.g, EISEN_F32, norm_dev_ + 1, slot.n), "clip_grad_norm scale");
+    norm_valid_ = true;
+    return {host[0], host[1]};
+}
+
+float AdamW::last_grad_norm() {
+    if (!norm_valid_) return 0.0f;
+    float host[2];
+    g_.check(eisen_hip_dtoh(g_.ctx(), host, norm_dev_, sizeof(host)), "last_grad_norm");
+    return host[0];
+}
+float AdamW::last_grad_scale() {
+    if (!norm_valid_) return 1.0f;
+    float host[2];
+    g_.check(eisen_hip_dtoh(g_.ctx(), host, norm_dev_, sizeof(host)), "last_grad_scale");
+    return host[1];
+}
+
+// AdamW::step (src/nn/optim.rs:334-562): optional clip (maybe_clip_gradients, :114-200), t += 1,
+// bias corrections by f32 powi, then one fused launch over every parameter.  With a clip norm
+// configured the coefficient stays on the device and is applied inside the update kernel.
+void AdamW::step() {
+    for (size_t id : params) g_.materialize_grad(id);
+    std::vector<eisen_param_slot> s = slots();
+    const float* scale_dev = nullptr;
+    if (grad_clip_norm_ > 0.0f) {
+        g_.check(eisen_hip_grad_norm(g_.ctx(), s.data(), s.size(), grad_clip_norm_, norm_dev_), "AdamW clip");
+        scale_dev = norm_dev_ + 1;
+        norm_valid_ = true;
+    }
+    t_ += 1;
+    const float bc1 = 1.0f / (1.0f - powi_f32(beta1, (int)t_));
+    const float bc2 = 1.0f / (1.0f - powi_f32(beta2, (int)t_));
+    g_.check(eisen_hip_adamw_step(g_.ctx(), s.data(), s.size(), lr, beta1, beta2, eps, weight_decay, bc1, bc2, scale_dev), "AdamW step");
+}
+
+// CosineScheduler::get_lr (src/nn/scheduler.rs:45-55)
+float CosineScheduler::get_lr(size_t step) const {
+    if (step < warmup_steps) return lr_max * (float)(step + 1) / (float)warmup_steps;
+    const size_t decay = std::max<size_t>(total_steps - warmup_steps, 1);
+    float progress = (float)(step - warmup_steps) / (float)decay;
+    progress = std::fmin(std::fmax(progress, 0.0f), 1.0f);
+    return lr_min + 0.5f * (lr_max - lr_min) * (1.0f + std::cos(3.14159274101257324f * progress));
+}
+
+void lm_micro_step(Graph& g, const TransformerLM& lm, const float* ids, const int64_t* targets, size_t mb, size_t seq, float* loss_out) {
+    const size_t x_id = g.alloc_pooled({mb, seq});
+    g.name_tensor(x_id, "input");
+    g.load_tensor_data(x_id, ids, mb * seq);
+    const size_t logits = lm.forward(g, x_id);
+    g.reinterpret_shape(logits, {mb * seq, lm.vocab_size});  // train_llm.rs:440 reshapes (a copy); the view is equivalent
+    const std::vector<int64_t> t(targets, targets + mb * seq);
+    const size_t loss = g.cross_entropy_masked(logits, t);
+    if (loss_out) *loss_out = g.sync_to_cpu(loss)[0];
+    g.backward(loss);
+    g.clear_activations();
+}
+
+}  // namespace eisen

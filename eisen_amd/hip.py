@@ -70,9 +70,14 @@ class Context:
         if rc != 0:
             raise EisenHipError("eisen_hip_init", rc, "no usable HIP device" if rc > 0 else "bad device index")
         self.h = h
+        self._children = []     # weak references to Graph objects created on this context
 
     def close(self):
         if getattr(self, "h", None):
+            for ref in getattr(self, "_children", []):
+                child = ref()
+                if child is not None:
+                    child.close()
             self.lib.eisen_hip_destroy(self.h)
             self.h = None
 

@@ -1,0 +1,118 @@
+/*
+ * eisen_graph.h -- C-ABI of the host-side Graph / nn / AdamW layer in libeisen_hip.so.
+ *
+ * The reference's host layer is Rust (`Graph`, `Tensor`, the `Module` trait, `AdamW`;
+ * src/graph/mod.rs and the files under src/nn/).  Where a Rust toolchain is present that layer binds
+ * include/eisen_hip.h directly; this header exposes the C++ mirror of it that ships in the
+ * library, with the same operations, argument meaning and error behaviour, so tests, the
+ * benchmark and non-Rust hosts can drive a full training step.
+ *
+ * Every function returns 0 on success and non-zero on failure (the reference panics; a host
+ * may turn non-zero into a panic).  `eisen_graph_last_error` returns the message.  Tensor ids
+ * are the reference's `usize` ids: indices into `Graph.tensors`.  Shapes are size_t arrays.
+ */
+#ifndef EISEN_GRAPH_H
+#define EISEN_GRAPH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "eisen_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct eisen_graph eisen_graph;
+typedef struct eisen_lm eisen_lm;
+typedef struct eisen_adamw eisen_adamw;
+
+enum { EISEN_PRECISION_FP32 = 0, EISEN_PRECISION_BF16_MIXED = 1 }; /* PrecisionMode, src/graph/mod.rs:48-53 */
+#define EISEN_MAX_RANK 8
+
+/* Graph::new(Device::Gpu(ctx, stream)) (src/graph/mod.rs:152-307). */
+int eisen_graph_new(eisen_ctx* ctx, int precision, eisen_graph** out);
+int eisen_graph_free(eisen_graph* g);
+const char* eisen_graph_last_error(eisen_graph* g);
+
+/* Graph::alloc / alloc_pooled / load_tensor_data / mark_params / mark_save_point /
+ * restore_save_point / clear_activations / reinterpret_shape / no_grad
+ * (src/graph/mod.rs:328-598, src/graph/ops/transform.rs:413-426). */
+int eisen_graph_alloc(eisen_graph* g, const size_t* shape, int rank, const float* data, size_t* id_out);
+int eisen_graph_alloc_pooled(eisen_graph* g, const size_t* shape, int rank, size_t* id_out);
+int eisen_graph_load_tensor_data(eisen_graph* g, size_t id, const float* host, size_t n);
+int eisen_graph_mark_params(eisen_graph* g);
+int eisen_graph_mark_save_point(eisen_graph* g, size_t* save_point_out);
+int eisen_graph_restore_save_point(eisen_graph* g, size_t save_point);
+int eisen_graph_clear_activations(eisen_graph* g);
+int eisen_graph_reinterpret_shape(eisen_graph* g, size_t id, const size_t* shape, int rank);
+int eisen_graph_set_no_grad(eisen_graph* g, int no_grad);
+int eisen_graph_num_tensors(eisen_graph* g, size_t* out);
+int eisen_graph_num_params(eisen_graph* g, size_t* out);
+int eisen_graph_tape_len(eisen_graph* g, size_t* out);
+int eisen_graph_tensor_shape(eisen_graph* g, size_t id, size_t* shape_out, int* rank_out);
+/* Tensor::sync_to_cpu / Graph::sync_grad_to_cpu (src/tensor.rs:177-223, src/graph/mod.rs:629-668):
+ * n must equal the element count; bf16 storage is widened to f32. */
+int eisen_graph_sync_to_cpu(eisen_graph* g, size_t id, float* out, size_t n);
+int eisen_graph_sync_grad_to_cpu(eisen_graph* g, size_t id, float* out, size_t n);
+int eisen_graph_synchronize(eisen_graph* g);
+
+/* Ops: one per `impl Graph` method under src/graph/ops/ (file:line at each definition in
+ * eisen_amd/csrc/host/graph.cpp).  Each writes the output tensor id. */
+int eisen_graph_add(eisen_graph* g, size_t a, size_t b, size_t* out);
+int eisen_graph_mul(eisen_graph* g, size_t a, size_t b, size_t* out);
+int eisen_graph_silu(eisen_graph* g, size_t a, size_t* out);
+int eisen_graph_swiglu(eisen_graph* g, size_t gate, size_t up, size_t* out);
+int eisen_graph_matmul(eisen_graph* g, size_t a, size_t b, size_t* out);
+int eisen_graph_matmul_trans_b(eisen_graph* g, size_t a, size_t b, size_t* out);
+int eisen_graph_bmm(eisen_graph* g, size_t a, size_t b, int trans_b, size_t* out);
+int eisen_graph_softmax(eisen_graph* g, size_t a, size_t* out);
+/* targets: int64, -1 = IGNORE_INDEX (usize::MAX, src/data/fim.rs:173) for the masked form. */
+int eisen_graph_cross_entropy(eisen_graph* g, size_t logits, const int64_t* targets, size_t n_targets, size_t* out);
+int eisen_graph_cross_entropy_masked(eisen_graph* g, size_t logits, const int64_t* targets, size_t n_targets, size_t* out);
+int eisen_graph_transpose_0213(eisen_graph* g, size_t a, size_t* out);
+int eisen_graph_gather(eisen_graph* g, size_t weights, size_t indices, size_t* out);
+int eisen_graph_reshape(eisen_graph* g, size_t a, const size_t* shape, int rank, size_t* out);
+int eisen_graph_rope(eisen_graph* g, size_t a, size_t head_dim, size_t* out);
+int eisen_graph_rms_norm(eisen_graph* g, size_t x, size_t w, float eps, size_t* out);
+int eisen_graph_repeat_kv(eisen_graph* g, size_t x, size_t repeats, size_t* out);
+int eisen_graph_flash_attention(eisen_graph* g, size_t q, size_t k, size_t v, float scale, int causal, size_t* out);
+int eisen_graph_attention_gqa(eisen_graph* g, size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, int causal,
+                              size_t* out);
+/* Graph::backward (src/graph/mod.rs:670-796). */
+int eisen_graph_backward(eisen_graph* g, size_t loss_id);
+
+/* TransformerLM (src/nn/transformer.rs:70-211).  Parameters are created in the reference's
+ * order with the reference's initialisers; load other weights with eisen_graph_load_tensor_data. */
+int eisen_lm_new(eisen_graph* g, size_t vocab, size_t hidden, size_t heads, size_t kv_heads, size_t ffn, size_t layers, int tie_weights,
+                 eisen_lm** out);
+int eisen_lm_free(eisen_lm* lm);
+/* Module::params order (src/nn/transformer.rs:57-66, :198-210). */
+int eisen_lm_params(eisen_lm* lm, size_t* ids_out, size_t capacity, size_t* count_out);
+int eisen_lm_forward(eisen_graph* g, eisen_lm* lm, size_t x_id, size_t* logits_out);
+/* 1: fused attention + SwiGLU ops (default); 0: the reference's materialised op chain. */
+int eisen_lm_set_fused(eisen_lm* lm, int fused);
+/* One micro-step of examples/train_llm.rs:433-458 (upload ids, forward, cross entropy, backward,
+ * clear_activations).  ids: f32 token ids [mb*seq]; targets int64 [mb*seq].  loss_out may be
+ * NULL, in which case nothing synchronises. */
+int eisen_lm_micro_step(eisen_graph* g, eisen_lm* lm, const float* ids, const int64_t* targets, size_t micro_batch, size_t seq_len,
+                        float* loss_out);
+
+/* AdamW (src/nn/optim.rs). */
+int eisen_adamw_new(eisen_graph* g, const size_t* params, size_t n_params, float lr, eisen_adamw** out);
+int eisen_adamw_free(eisen_adamw* opt);
+int eisen_adamw_config(eisen_adamw* opt, float lr, float beta1, float beta2, float eps, float weight_decay, float grad_clip_norm);
+int eisen_adamw_init_moments(eisen_adamw* opt);
+int eisen_adamw_zero_grad(eisen_adamw* opt);
+int eisen_adamw_clip_grad_norm(eisen_adamw* opt, float max_norm, float* norm_out, float* coef_out);
+int eisen_adamw_step(eisen_adamw* opt);
+int eisen_adamw_last_grad_norm(eisen_adamw* opt, float* norm_out, float* scale_out);
+/* Moments of the i-th parameter, copied to the host (tests). */
+int eisen_adamw_moments_to_cpu(eisen_adamw* opt, size_t i, float* m_out, float* v_out, size_t n);
+/* CosineScheduler::get_lr (src/nn/scheduler.rs:45-55). */
+float eisen_cosine_lr(float lr_max, float lr_min, size_t warmup_steps, size_t total_steps, size_t step);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EISEN_GRAPH_H */
