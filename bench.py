@@ -1,0 +1,290 @@
+#!/usr/bin/env python3
+"""Benchmark of the training step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c3|c2]
+
+Default workload c5 = BASELINE config 5: the "~1.1B" Llama-style model (vocab 32000, d 2048,
+16 layers, 32 query / 8 KV heads, head_dim 64, SiLU-gated MLP 5632, untied lm_head), seq 1024,
+micro-batch 4, gradient accumulation 8 (32,768 tokens per optimiser step), bf16 activations and
+matmuls, f32 master weights and AdamW state, synthetic Zipf(1.1) token ids, N(0, 0.02) weights.
+One "step" = zero_grad, 8 x (upload ids, forward, fused cross entropy, backward), gradient-norm
+clip, fused AdamW -- the loop of examples/train_llm.rs:386-477.
+
+Prints one JSON line.  `value` is tokens/s over K timed steps (inputs resident in host memory,
+weights and optimiser state resident in HBM).  `roofline` describes the kernel that takes the
+largest share of the step, timed with HIP events on the library's stream in one extra,
+instrumented step.  `cpu_baseline` times the CPU oracle (a single-threaded restatement of the
+reference's Device::Cpu path) on a bounded sample of the same architecture.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from tests import gen  # noqa: E402  (seeded synthetic inputs shared with the tests)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+CONFIGS = {
+    "c5": dict(vocab=32000, hidden=2048, heads=32, kv_heads=8, ffn=5632, layers=16, tie=False, seq=1024, mb=4, accum=8,
+               label="config5 ~1.1B Llama-style (852,559,872 params untied), bf16 mixed, seq 1024, micro-batch 4, accum 8"),
+    "c4": dict(vocab=8192, hidden=256, heads=8, kv_heads=2, ffn=1024, layers=6, tie=True, seq=256, mb=32, accum=1,
+               label="config4 ~14M Llama-style (7,802,112 params tied), bf16 mixed, seq 256, micro-batch 32"),
+}
+
+
+def flops_per_token(c):
+    """6*P_mm + 6*L*S*d: matmul parameters incl. lm_head, causal attention fwd+bwd without recompute."""
+    d, f, L, V = c["hidden"], c["ffn"], c["layers"], c["vocab"]
+    dkv = c["kv_heads"] * (d // c["heads"])
+    p_mm = L * (2 * d * d + 2 * d * dkv + 3 * d * f) + d * V
+    return 6 * p_mm + 6 * L * c["seq"] * d
+
+
+def arch(c):
+    return {k: c[k] for k in ("vocab", "hidden", "heads", "kv_heads", "ffn", "layers", "tie")}
+
+
+def pick_dominant(prof):
+    name = max(prof, key=lambda k: prof[k]["ms"])
+    e = prof[name]
+    per_launch_ms = e["ms"] / e["launches"]
+    if e["unit"] == "flop":
+        achieved = e["work"] / e["launches"] / (per_launch_ms * 1e-3) / 1e12
+        return name, dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                          frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=None)
+    achieved = e["work"] / e["launches"] / (per_launch_ms * 1e-3) / 1e9
+    return name, dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None)
+
+
+def kernel_table(prof):
+    rows = []
+    for name, e in sorted(prof.items(), key=lambda kv: -kv[1]["ms"]):
+        rate = e["work"] / (e["ms"] * 1e-3) if e["ms"] > 0 else 0.0
+        rows.append(dict(kernel=name, ms=round(e["ms"], 3), launches=e["launches"], avg_us=round(1e3 * e["ms"] / e["launches"], 2),
+                         rate=round(rate / (1e12 if e["unit"] == "flop" else 1e9), 2), rate_unit="TFLOP/s" if e["unit"] == "flop" else "GB/s"))
+    return rows
+
+
+# ---------------------------------------------------------------------------------------------
+# CPU baseline: the oracle (port of the reference's single-threaded CPU arms) on a bounded sample
+# ---------------------------------------------------------------------------------------------
+
+def cpu_baseline_lm(c, budget_tokens):
+    """Times fwd+bwd of a 1-layer and a 2-layer model of the same width/vocab on `budget_tokens` tokens,
+    separates the per-layer from the embedding/lm_head/CE cost, and extrapolates to the full depth."""
+    from oracle import cpu_ref as R
+    R.set_threads(1)
+    times = {}
+    for layers in (1, 2):
+        cfg = dict(arch(c), layers=layers)
+        g = R.Graph()
+        lm = R.TransformerLM(g, **cfg)
+        for pid, (_, w) in enumerate(gen.lm_weights(5, **cfg)):
+            g.load_tensor_data(pid, w)
+        g.mark_params()
+        x, y = gen.lm_batch(9, 1, budget_tokens, c["vocab"], "zipf")
+        lm.micro_step(x, y)                      # untimed: first touch of the gradient pages
+        t0 = time.perf_counter()
+        lm.micro_step(x, y)
+        times[layers] = time.perf_counter() - t0
+        del lm, g
+    per_layer = max(times[2] - times[1], 1e-9)
+    head = max(times[1] - per_layer, 0.0)
+    per_token = (c["layers"] * per_layer + head) / budget_tokens
+    return dict(value=round(1.0 / per_token, 3), unit="tokens/s", cores=1, kind="port",
+                sample=(f"oracle fwd+bwd of 1- and 2-layer models of this width/vocab on {budget_tokens} tokens (seq {budget_tokens}, so the "
+                        f"S^2 attention share is understated), {times[1]:.1f}s + {times[2]:.1f}s, extrapolated to {c['layers']} layers; AdamW excluded"))
+
+
+# ---------------------------------------------------------------------------------------------
+# workloads
+# ---------------------------------------------------------------------------------------------
+
+def bench_lm(name, steps, warmup, cpu_tokens):
+    from eisen_amd import graph as G
+    from eisen_amd import hip
+    c = CONFIGS[name]
+    ctx = hip.Context(0)
+    g = G.Graph(ctx, G.BF16_MIXED)
+    lm = G.TransformerLM(g, **arch(c))
+    rng = np.random.default_rng(1234)
+    for pid in range(g.num_tensors()):
+        shape = g.shape(pid)
+        if len(shape) == 2:   # matrices N(0, 0.02); norm gains stay 1.0
+            g.load_tensor_data(pid, rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02))
+    g.mark_params()
+    opt = G.AdamW(g, lm.params(), 1e-3)
+    opt.config(1e-3, 0.9, 0.95, 1e-8, 0.1, 1.0)      # train_llm.rs:266-270 + grad clip 1.0
+    opt.init_moments()
+    n_batches = (steps + warmup + 1) * c["accum"]
+    batches = [gen.lm_batch(100 + i, c["mb"], c["seq"], c["vocab"], "zipf") for i in range(n_batches)]
+    batches = [(x.astype(np.float32), y) for x, y in batches]
+    it = iter(batches)
+
+    def one_step(want_loss=False):
+        opt.zero_grad()
+        loss = None
+        for _ in range(c["accum"]):
+            x, y = next(it)
+            loss = lm.micro_step(x, y, want_loss=want_loss)
+        opt.step()
+        return loss
+
+    for _ in range(warmup):
+        one_step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one_step()
+    ctx.sync()
+    elapsed = time.perf_counter() - t0
+    # one more, instrumented step for the per-kernel numbers (not part of `value`)
+    ctx.profile_start()
+    last_loss = one_step(want_loss=True)
+    prof = ctx.profile_stop()
+    tokens_per_step = c["accum"] * c["mb"] * c["seq"]
+    value = steps * tokens_per_step / elapsed
+    dom, roofline = pick_dominant(prof)
+    roofline["kernel"] = dom
+    step_flops = flops_per_token(c) * tokens_per_step
+    out = dict(metric="train tokens/sec (fwd+bwd+AdamW)", value=round(value, 1), unit="tokens/s", n_gpus=1, steps=steps, warmup=warmup,
+               ms_per_step=round(1e3 * elapsed / steps, 3), higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16",
+               data="synthetic",
+               config=dict(workload=c["label"], tokens_per_step=tokens_per_step, parallelism="single GPU",
+                           step_model_tflops=round(step_flops / 1e12, 2),
+                           mfma_frac_of_step=round(step_flops / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 4), last_loss=round(float(last_loss), 4)),
+               roofline=roofline, kernels=kernel_table(prof))
+    ctx.close()
+    out["cpu_baseline"] = cpu_baseline_lm(c, cpu_tokens)
+    return out
+
+
+def bench_c3(steps, warmup):
+    """Config 3: causal GQA flash attention forward + backward, B8 S1024 Hq16 Hkv4 hd64 bf16, layout [B,H,S,hd]."""
+    from eisen_amd import hip
+    from oracle import cpu_ref as R
+    B, S, Hq, Hkv, hd = 8, 1024, 16, 4, 64
+    ctx = hip.Context(0)
+    sd = 1.0 / 8
+    q, do = gen.normal(600, (B, Hq, S, hd), sd), gen.normal(601, (B, Hq, S, hd), sd)
+    k, v = gen.normal(602, (B, Hkv, S, hd), sd), gen.normal(603, (B, Hkv, S, hd), sd)
+    dq_, dk_, dv_, ddo = (ctx.upload(t, hip.BF16) for t in (q, k, v, do))
+    out, lse = ctx.malloc(q.size * 2), ctx.malloc(B * Hq * S * 4)
+    gq, gk, gv = ctx.malloc(q.size * 2), ctx.malloc(k.size * 2), ctx.malloc(k.size * 2)
+    qs, ks = (Hq * S * hd, hd, S * hd), (Hkv * S * hd, hd, S * hd)
+
+    def step():
+        ctx.attention_forward(dq_, dk_, dv_, out, lse, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+        ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+
+    for _ in range(warmup):
+        step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    ctx.sync()
+    elapsed = time.perf_counter() - t0
+    ctx.profile_start()
+    for _ in range(steps):
+        step()
+    prof = ctx.profile_stop()
+    bwd_ms = (prof["attn_bwd_dq_bf16"]["ms"] + prof["attn_bwd_dkv_bf16"]["ms"]) / steps
+    bwd_flops = 4 * 2 * hd * (S * (S + 1) / 2) * B * Hq          # 34.39 GFLOP: four GEMMs, causal pairs, no recompute
+    achieved = bwd_flops / (bwd_ms * 1e-3) / 1e12
+    tokens = B * S
+    ctx.close()
+    # CPU: the unfused chain on one batch element and one KV group (4 query heads), scaled by B*Hkv
+    R.set_threads(1)
+    t1 = time.perf_counter()
+    R.attention_chain(np.ascontiguousarray(q[:1, :4].transpose(0, 2, 1, 3)), np.ascontiguousarray(k[:1, :1].transpose(0, 2, 1, 3)),
+                       np.ascontiguousarray(v[:1, :1].transpose(0, 2, 1, 3)), np.ascontiguousarray(do[:1, :4].transpose(0, 2, 1, 3)), np.float32(0.125))
+    cpu_s = (time.perf_counter() - t1) * B * Hkv
+    return dict(metric="flash-attention fwd+bwd tokens/sec (config 3)", value=round(steps * tokens / elapsed, 1), unit="tokens/s", n_gpus=1,
+                steps=steps, warmup=warmup, ms_per_step=round(1e3 * elapsed / steps, 4), higher_is_better=True, scaling="weak",
+                vs_baseline=None, dtype="bf16", data="synthetic",
+                config=dict(workload="config3 causal GQA flash attention fwd+bwd, B8 S1024 Hq16 Hkv4 hd64, [B,H,S,hd]"),
+                roofline=dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                              frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=None, kernel="attn_bwd (dq + dkv kernels)"),
+                kernels=kernel_table(prof),
+                cpu_baseline=dict(value=round(tokens / cpu_s, 2), unit="tokens/s", cores=1, kind="port",
+                                  sample="oracle unfused attention chain fwd+bwd on 1 of 32 (batch, KV group) slices, scaled x32"))
+
+
+def bench_c2(steps, warmup):
+    """Config 2: fused softmax-cross-entropy forward+backward, bf16 [8192 x 32000]."""
+    from eisen_amd import hip
+    from oracle import cpu_ref as R
+    rows, V = 8192, 32000
+    ctx = hip.Context(0)
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((rows, V), dtype=np.float32) * np.float32(2.0)
+    t = rng.integers(0, V, rows)
+    dx, dt = ctx.upload(x, hip.BF16), ctx.upload(t.astype(np.int32))
+    dl, rl, lo = ctx.malloc(rows * V * 2), ctx.malloc(rows * 4), ctx.malloc(4)
+
+    def step():
+        ctx.cross_entropy(dx, dt, dl, rl, lo, hip.BF16, rows, V, 1.0 / rows)
+
+    for _ in range(warmup):
+        step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    ctx.sync()
+    elapsed = time.perf_counter() - t0
+    ctx.profile_start()
+    for _ in range(steps):
+        step()
+    prof = ctx.profile_stop()
+    dom, roofline = pick_dominant(prof)
+    roofline["kernel"] = dom
+    ctx.close()
+    R.set_threads(1)
+    sample = 64
+    xs = hip.round_bf16(x[:sample])
+    t1 = time.perf_counter()
+    R.cross_entropy(xs, t[:sample])
+    cpu_rows_s = sample / (time.perf_counter() - t1)
+    return dict(metric="fused softmax-cross-entropy fwd+bwd rows/sec (config 2)", value=round(steps * rows / elapsed, 1), unit="rows/s", n_gpus=1,
+                steps=steps, warmup=warmup, ms_per_step=round(1e3 * elapsed / steps, 4), higher_is_better=True, scaling="weak", vs_baseline=None,
+                dtype="bf16", data="synthetic", config=dict(workload="config2 fused softmax-CE fwd+bwd, bf16 logits [8192 x 32000]"),
+                roofline=roofline, kernels=kernel_table(prof),
+                cpu_baseline=dict(value=round(cpu_rows_s, 2), unit="rows/s", cores=1, kind="port", sample=f"oracle CE fwd+bwd on {sample} of 8192 rows"))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default="c5", choices=["c5", "c4", "c3", "c2"])
+    ap.add_argument("--cpu-tokens", type=int, default=None, help="tokens in the CPU-baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if args.workload in ("c5", "c4"):
+        steps = args.steps if args.steps is not None else (3 if args.workload == "c5" else 20)
+        warmup = args.warmup if args.warmup is not None else (1 if args.workload == "c5" else 3)
+        cpu_tokens = args.cpu_tokens or (16 if args.workload == "c5" else 256)
+        out = bench_lm(args.workload, steps, warmup, cpu_tokens)
+    elif args.workload == "c3":
+        out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3)
+    else:
+        out = bench_c2(args.steps or 20, args.warmup if args.warmup is not None else 3)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

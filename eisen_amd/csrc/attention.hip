@@ -518,8 +518,15 @@ int fill_args(eisen_ctx* ctx, AttnArgs& a, int dtype, size_t B, size_t S, size_t
     return 0;
 }
 
+// Algorithmic flops of one attention GEMM over the visible (query, key) pairs.
+static double attn_pair_flops(const AttnArgs& a) {
+    const double pairs = a.causal ? (double)a.S * ((double)a.S + 1.0) / 2.0 : (double)a.S * (double)a.S;
+    return 2.0 * (double)a.hd * pairs * (double)a.B * (double)a.Hq;
+}
+
 template <int HD>
 void launch_fwd(eisen_ctx* ctx, const AttnArgs& a) {
+    EisenProfScope prof(ctx, "attn_fwd_bf16", 2.0 * attn_pair_flops(a), true);
     const int gw = a.G % 4 == 0 ? 4 : (a.G % 2 == 0 ? 2 : 1);
     const int qs = 4 / gw;
     dim3 grid((unsigned)eisen_ceil_div(a.S, 32 * qs), (unsigned)(a.Hkv * (a.G / gw)), (unsigned)a.B);
@@ -532,11 +539,17 @@ void launch_bwd(eisen_ctx* ctx, const AttnArgs& a) {
     const int gw = a.G % 4 == 0 ? 4 : (a.G % 2 == 0 ? 2 : 1);
     const int qs = 4 / gw;
     dim3 grid((unsigned)eisen_ceil_div(a.S, 32 * qs), (unsigned)(a.Hkv * (a.G / gw)), (unsigned)a.B);
-    if (gw == 4) fa_bwd_dq_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
-    else if (gw == 2) fa_bwd_dq_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
-    else fa_bwd_dq_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
+    {   // dQ = scale dS K: one of the four backward GEMMs (S and dP are recomputed here as well)
+        EisenProfScope prof(ctx, "attn_bwd_dq_bf16", 1.0 * attn_pair_flops(a), true);
+        if (gw == 4) fa_bwd_dq_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
+        else if (gw == 2) fa_bwd_dq_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
+        else fa_bwd_dq_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
+    }
     dim3 grid2((unsigned)eisen_ceil_div(a.S, 128), (unsigned)a.Hkv, (unsigned)a.B);
-    fa_bwd_dkv_kernel<HD><<<grid2, 256, 0, ctx->stream>>>(a);
+    {   // dP, dV, dK: three of the four backward GEMMs
+        EisenProfScope prof(ctx, "attn_bwd_dkv_bf16", 3.0 * attn_pair_flops(a), true);
+        fa_bwd_dkv_kernel<HD><<<grid2, 256, 0, ctx->stream>>>(a);
+    }
 }
 
 }  // namespace

@@ -243,6 +243,9 @@ extern "C" int eisen_hip_cross_entropy(eisen_ctx* ctx, const void* logits, const
     EISEN_REQUIRE(ctx, rows > 0 && rows < (size_t(1) << 31), EISEN_E_SHAPE, "cross_entropy: rows %zu out of range", rows);
     EISEN_REQUIRE(ctx, classes > 0 && classes < (size_t(1) << 30), EISEN_E_SHAPE, "cross_entropy: classes %zu out of range", classes);
     const float scale = normalizer * grad_scale;
+    // algorithmic bytes: logits read once, dlogits written once, targets read, row losses written
+    EisenProfScope prof(ctx, dtype == EISEN_BF16 ? "ce_fused_bf16" : "ce_fused_f32",
+                        2.0 * (double)rows * (double)classes * (double)eisen_dtype_size(dtype) + 8.0 * (double)rows);
     int rc = dtype == EISEN_F32
                  ? ce_dispatch<float>(ctx, logits, targets, dlogits, row_loss, argmax_out, target_logit_out, rows, classes, scale)
                  : ce_dispatch<bf16_t>(ctx, logits, targets, dlogits, row_loss, argmax_out, target_logit_out, rows, classes, scale);

@@ -8,9 +8,10 @@
 // bf16 path: MFMA v_mfma_f32_32x32x16_bf16, f32 accumulate.  A workgroup of 4 waves owns a
 // BM x BN tile of C; each wave owns a (BM/2) x (BN/2) quadrant made of 32x32 MFMA tiles.  K is walked in slabs of
 // 32 through double-buffered LDS (one barrier per slab) with the next slab's global loads in
-// flight during the current slab's MFMAs.  LDS always holds both operands K-contiguous, which
-// is the order the MFMA operand registers want (8 consecutive k per lane, one ds_read_b128);
-// an operand whose memory order is the other way round is transposed on its way into LDS.
+// flight during the current slab's MFMAs.  The MFMA operand registers want 8 consecutive k per
+// lane: a k-contiguous operand gets them with one ds_read_b128, an operand stored the other
+// way round with two ds_read_b64_tr_b16 (LDS transpose reads), so dX, dW and the forward GEMM
+// all stream their operands through LDS as plain 16-byte copies.
 //
 // f32 path and odd shapes: a plain LDS-tiled FMA kernel (64x64 tile, 4x4 per thread).
 #include "device_utils.cuh"
@@ -34,18 +35,70 @@ struct GemmArgs {
 
 // ---- MFMA kernel -------------------------------------------------------------------------
 // A_KC: A is stored [M][K] (k contiguous); otherwise [K][M].  B_KC: B is stored [N][K];
-// otherwise [K][N].
+// otherwise [K][N].  Either way a slab travels global -> registers -> LDS as straight 16-byte
+// copies in its memory order:
+//   k-contiguous operand : LDS tile [rows][BK + 8];  MFMA operand = one ds_read_b128
+//   other order          : LDS tile [BK][rows + 16]; MFMA operand = two ds_read_b64_tr_b16, the
+//                          LDS transpose read that hands a lane 4 consecutive k of one column
+// so no operand is ever transposed element by element.
+typedef bf16x4 __attribute__((address_space(3))) * lds_bf16x4_ptr;
+
+template <int ROWS, bool KC>
+struct OperandTile {
+    static constexpr int PITCH = KC ? BK + 8 : ROWS + 16;
+    static constexpr int ELEMS = KC ? ROWS * PITCH : BK * PITCH;
+    static constexpr int CHUNKS = ROWS * BK / 8 / kGemmThreads;  // 16-byte chunks per thread per slab
+
+    // global coordinates (row = m or n, k) of chunk `c` of thread `tid`
+    static __device__ __forceinline__ void chunk_coords(int c, int tid, int& row, int& k) {
+        const int chunk = c * kGemmThreads + tid;
+        if (KC) {
+            row = chunk / (BK / 8);
+            k = (chunk % (BK / 8)) * 8;
+        } else {
+            k = chunk / (ROWS / 8);
+            row = (chunk % (ROWS / 8)) * 8;
+        }
+    }
+    static __device__ __forceinline__ bf16x8 load(const bf16_t* base, int ld, int row0, int k0, int row_limit, int k_limit, int c, int tid) {
+        int row, k;
+        chunk_coords(c, tid, row, k);
+        row += row0;
+        k += k0;
+        const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (row >= row_limit || k >= k_limit) return zero8;
+        return *reinterpret_cast<const bf16x8*>(KC ? base + (long long)row * ld + k : base + (long long)k * ld + row);
+    }
+    static __device__ __forceinline__ void store(bf16_t* tile, bf16x8 v, int c, int tid) {
+        int row, k;
+        chunk_coords(c, tid, row, k);
+        *reinterpret_cast<bf16x8*>(KC ? tile + row * PITCH + k : tile + k * PITCH + row) = v;
+    }
+    // MFMA operand of the 32 rows starting at `row0` for contraction offsets ks..ks+15:
+    // lane l holds row row0 + l%32 and k = ks + 8*(l/32) + 0..7.
+    static __device__ __forceinline__ bf16x8 fragment(const bf16_t* tile, int row0, int ks, int lane) {
+        if (KC) return *reinterpret_cast<const bf16x8*>(tile + (row0 + (lane & 31)) * PITCH + ks + 8 * (lane >> 5));
+        const int L = lane & 15, half = (lane >> 4) & 1;
+        const bf16_t* p = tile + (ks + 8 * (lane >> 5) + (L >> 2)) * PITCH + row0 + 16 * half + 4 * (L & 3);
+        const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p));
+        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p + 4 * PITCH));
+        bf16x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    }
+};
+
 template <int BM, int BN, bool A_KC, bool B_KC, typename TC>
 __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
     constexpr int WM = BM / 2, WN = BN / 2;          // wave quadrant
     constexpr int TM = WM / 32, TN = WN / 32;        // 32x32 tiles per wave
-    constexpr int A_CHUNKS = BM * BK / 8 / kGemmThreads;  // 16-byte chunks per thread per slab
-    constexpr int B_CHUNKS = BN * BK / 8 / kGemmThreads;
-    __shared__ __attribute__((aligned(16))) bf16_t lds[2][(BM + BN) * LDS_PITCH];
+    using TA = OperandTile<BM, A_KC>;
+    using TB = OperandTile<BN, B_KC>;
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2][TA::ELEMS + TB::ELEMS];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    // neighbouring workgroups share an A row-block: walk N fastest inside a strip of M
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const bf16_t* A = static_cast<const bf16_t*>(g.A) + (long long)blockIdx.z * g.sA;
     const bf16_t* B = static_cast<const bf16_t*>(g.B) + (long long)blockIdx.z * g.sB;
@@ -59,64 +112,18 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-    bf16x8 ra[A_CHUNKS], rb[B_CHUNKS];
-    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-
+    bf16x8 ra[TA::CHUNKS], rb[TB::CHUNKS];
     auto load_global = [&](int k0) {
 #pragma unroll
-        for (int c = 0; c < A_CHUNKS; c++) {
-            const int chunk = c * kGemmThreads + tid;
-            if (A_KC) {
-                const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
-                const int m = m0 + row, k = k0 + kc * 8;
-                ra[c] = (m < g.M && k < g.K) ? *reinterpret_cast<const bf16x8*>(A + (long long)m * g.lda + k) : zero8;
-            } else {
-                const int kk = chunk / (BM / 8), mc = chunk % (BM / 8);
-                const int m = m0 + mc * 8, k = k0 + kk;
-                ra[c] = (m < g.M && k < g.K) ? *reinterpret_cast<const bf16x8*>(A + (long long)k * g.lda + m) : zero8;
-            }
-        }
+        for (int c = 0; c < TA::CHUNKS; c++) ra[c] = TA::load(A, g.lda, m0, k0, g.M, g.K, c, tid);
 #pragma unroll
-        for (int c = 0; c < B_CHUNKS; c++) {
-            const int chunk = c * kGemmThreads + tid;
-            if (B_KC) {
-                const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
-                const int n = n0 + row, k = k0 + kc * 8;
-                rb[c] = (n < g.N && k < g.K) ? *reinterpret_cast<const bf16x8*>(B + (long long)n * g.ldb + k) : zero8;
-            } else {
-                const int kk = chunk / (BN / 8), nc = chunk % (BN / 8);
-                const int n = n0 + nc * 8, k = k0 + kk;
-                rb[c] = (n < g.N && k < g.K) ? *reinterpret_cast<const bf16x8*>(B + (long long)k * g.ldb + n) : zero8;
-            }
-        }
+        for (int c = 0; c < TB::CHUNKS; c++) rb[c] = TB::load(B, g.ldb, n0, k0, g.N, g.K, c, tid);
     };
     auto store_lds = [&](int buf) {
-        bf16_t* As = lds[buf];
-        bf16_t* Bs = lds[buf] + BM * LDS_PITCH;
 #pragma unroll
-        for (int c = 0; c < A_CHUNKS; c++) {
-            const int chunk = c * kGemmThreads + tid;
-            if (A_KC) {
-                const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
-                *reinterpret_cast<bf16x8*>(As + row * LDS_PITCH + kc * 8) = ra[c];
-            } else {
-                const int kk = chunk / (BM / 8), mc = chunk % (BM / 8);
+        for (int c = 0; c < TA::CHUNKS; c++) TA::store(lds[buf], ra[c], c, tid);
 #pragma unroll
-                for (int j = 0; j < 8; j++) As[(mc * 8 + j) * LDS_PITCH + kk] = ra[c][j];
-            }
-        }
-#pragma unroll
-        for (int c = 0; c < B_CHUNKS; c++) {
-            const int chunk = c * kGemmThreads + tid;
-            if (B_KC) {
-                const int row = chunk / (BK / 8), kc = chunk % (BK / 8);
-                *reinterpret_cast<bf16x8*>(Bs + row * LDS_PITCH + kc * 8) = rb[c];
-            } else {
-                const int kk = chunk / (BN / 8), nc = chunk % (BN / 8);
-#pragma unroll
-                for (int j = 0; j < 8; j++) Bs[(nc * 8 + j) * LDS_PITCH + kk] = rb[c][j];
-            }
-        }
+        for (int c = 0; c < TB::CHUNKS; c++) TB::store(lds[buf] + TA::ELEMS, rb[c], c, tid);
     };
 
     const int nk = (g.K + BK - 1) / BK;
@@ -126,15 +133,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
     for (int kt = 0; kt < nk; kt++) {
         const int buf = kt & 1;
         if (kt + 1 < nk) load_global((kt + 1) * BK);
-        const bf16_t* As = lds[buf] + (wm * WM + (lane & 31)) * LDS_PITCH + (lane >> 5) * 8;
-        const bf16_t* Bs = lds[buf] + BM * LDS_PITCH + (wn * WN + (lane & 31)) * LDS_PITCH + (lane >> 5) * 8;
+        const bf16_t* As = lds[buf];
+        const bf16_t* Bs = lds[buf] + TA::ELEMS;
 #pragma unroll
         for (int ks = 0; ks < BK; ks += 16) {
             bf16x8 a[TM], b[TN];
 #pragma unroll
-            for (int i = 0; i < TM; i++) a[i] = *reinterpret_cast<const bf16x8*>(As + i * 32 * LDS_PITCH + ks);
+            for (int i = 0; i < TM; i++) a[i] = TA::fragment(As, wm * WM + i * 32, ks, lane);
 #pragma unroll
-            for (int j = 0; j < TN; j++) b[j] = *reinterpret_cast<const bf16x8*>(Bs + j * 32 * LDS_PITCH + ks);
+            for (int j = 0; j < TN; j++) b[j] = TB::fragment(Bs, wn * WN + j * 32, ks, lane);
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -262,6 +269,10 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         return 0;
     }
     const bool a_kc = !trans_a, b_kc = trans_b != 0;
+    char pname[48];
+    snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
+             dtype_c == EISEN_BF16 ? "bf16out" : "f32out");
+    EisenProfScope prof(ctx, pname, 2.0 * (double)M * (double)N * (double)K * (double)batch, true);
     bool mfma_ok = dtype_ab == EISEN_BF16 && eisen_aligned(A, 16) && eisen_aligned(B, 16) && g.lda % 8 == 0 && g.ldb % 8 == 0 &&
                    sA % 8 == 0 && sB % 8 == 0;
     // the contiguous dimension of each operand must be a whole number of 8-element chunks

@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -15,6 +16,21 @@
 struct eisen_rope_table {
     size_t seq = 0, head_dim = 0;
     float* cos_sin = nullptr;  // [seq][head_dim/2][2] f32 on the device
+};
+
+// Optional per-kernel timing: every instrumented launch is bracketed by two events on the stream.
+struct eisen_prof_rec {
+    int key;
+    hipEvent_t start, stop;
+    double work;  // algorithmic flops or bytes of the launch
+};
+struct eisen_prof {
+    bool enabled = false;
+    std::vector<std::string> names;
+    std::vector<int> is_flops;
+    std::vector<hipEvent_t> pool;
+    size_t pool_used = 0;
+    std::vector<eisen_prof_rec> recs;
 };
 
 struct eisen_ctx {
@@ -27,14 +43,35 @@ struct eisen_ctx {
     std::unordered_map<size_t, std::vector<void*>> free_lists;
     std::unordered_map<void*, size_t> live;
     size_t in_use_bytes = 0, cached_bytes = 0;
-    // pinned staging for asynchronous uploads
-    void* stage = nullptr;
-    size_t stage_bytes = 0;
+    // pinned staging ring for asynchronous uploads: a slot is reused only after its copy's event fired
+    struct StageSlot {
+        void* ptr = nullptr;
+        size_t bytes = 0;
+        hipEvent_t done = nullptr;
+        bool in_flight = false;
+    };
+    static constexpr int kStageSlots = 16;
+    StageSlot stage[kStageSlots];
+    int stage_next = 0;
     // grow-only device workspace for two-stage reductions and tables
     void* ws = nullptr;
     size_t ws_bytes = 0;
     std::vector<eisen_rope_table> rope_tables;
+    eisen_prof prof;
     char last_error[512] = {0};
+};
+
+// Brackets the launches issued during its lifetime when profiling is on; free when it is off.
+int eisen_prof_begin(eisen_ctx* ctx, const char* name, double work, bool is_flops);
+void eisen_prof_end(eisen_ctx* ctx, int rec);
+struct EisenProfScope {
+    eisen_ctx* ctx;
+    int rec;
+    EisenProfScope(eisen_ctx* c, const char* name, double work, bool is_flops = false)
+        : ctx(c), rec(c->prof.enabled ? eisen_prof_begin(c, name, work, is_flops) : -1) {}
+    ~EisenProfScope() {
+        if (rec >= 0) eisen_prof_end(ctx, rec);
+    }
 };
 
 struct eisen_module {
@@ -47,8 +84,8 @@ struct eisen_function {
 int eisen_set_error(eisen_ctx* ctx, int code, const char* fmt, ...);
 // Returns a device workspace of at least `bytes` (grow-only, stream-ordered reuse).
 int eisen_workspace(eisen_ctx* ctx, size_t bytes, void** out);
-// Pinned staging buffer of at least `bytes`; waits for earlier uploads that still read it.
-int eisen_staging(eisen_ctx* ctx, size_t bytes, void** out);
+// Next pinned staging slot, grown to at least `bytes`; waits only if that slot's last copy is still in flight.
+int eisen_staging(eisen_ctx* ctx, size_t bytes, eisen_ctx::StageSlot** out);
 
 #define EISEN_HIP_TRY(ctx, expr)                                                              \
     do {                                                                                      \

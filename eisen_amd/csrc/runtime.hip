@@ -66,7 +66,11 @@ extern "C" int eisen_hip_destroy(eisen_ctx* ctx) {
     for (auto& t : ctx->rope_tables) (void)hipFreeAsync(t.cos_sin, ctx->stream);
     if (ctx->ws) (void)hipFreeAsync(ctx->ws, ctx->stream);
     (void)hipStreamSynchronize(ctx->stream);
-    if (ctx->stage) (void)hipHostFree(ctx->stage);
+    for (auto& sl : ctx->stage) {
+        if (sl.ptr) (void)hipHostFree(sl.ptr);
+        if (sl.done) (void)hipEventDestroy(sl.done);
+    }
+    for (hipEvent_t e : ctx->prof.pool) (void)hipEventDestroy(e);
     (void)hipEventDestroy(ctx->ev_start);
     (void)hipEventDestroy(ctx->ev_stop);
     (void)hipStreamDestroy(ctx->stream);
@@ -164,18 +168,23 @@ int eisen_workspace(eisen_ctx* ctx, size_t bytes, void** out) {
     return 0;
 }
 
-int eisen_staging(eisen_ctx* ctx, size_t bytes, void** out) {
-    // an earlier asynchronous upload may still be reading the staging buffer
-    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    if (bytes > ctx->stage_bytes) {
-        if (ctx->stage) EISEN_HIP_TRY(ctx, hipHostFree(ctx->stage));
-        ctx->stage = nullptr;
-        ctx->stage_bytes = 0;
-        size_t want = (bytes + (size_t(1) << 16) - 1) & ~((size_t(1) << 16) - 1);
-        EISEN_HIP_TRY(ctx, hipHostMalloc(&ctx->stage, want, hipHostMallocDefault));
-        ctx->stage_bytes = want;
+int eisen_staging(eisen_ctx* ctx, size_t bytes, eisen_ctx::StageSlot** out) {
+    eisen_ctx::StageSlot& s = ctx->stage[ctx->stage_next];
+    ctx->stage_next = (ctx->stage_next + 1) % eisen_ctx::kStageSlots;
+    if (!s.done) EISEN_HIP_TRY(ctx, hipEventCreateWithFlags(&s.done, hipEventDisableTiming));
+    if (s.in_flight) {
+        EISEN_HIP_TRY(ctx, hipEventSynchronize(s.done));
+        s.in_flight = false;
     }
-    *out = ctx->stage;
+    if (bytes > s.bytes) {
+        if (s.ptr) EISEN_HIP_TRY(ctx, hipHostFree(s.ptr));
+        s.ptr = nullptr;
+        s.bytes = 0;
+        size_t want = (bytes + (size_t(1) << 16) - 1) & ~((size_t(1) << 16) - 1);
+        EISEN_HIP_TRY(ctx, hipHostMalloc(&s.ptr, want, hipHostMallocDefault));
+        s.bytes = want;
+    }
+    *out = &s;
     return 0;
 }
 
@@ -187,13 +196,13 @@ extern "C" int eisen_hip_htod(eisen_ctx* ctx, void* dst, const void* src, size_t
     if (bytes == 0) return 0;
     if (bytes <= kStageLimit) {
         // small uploads (token ids, targets, tables) go through pinned staging and stay asynchronous
-        void* st = nullptr;
-        if (bytes > ctx->stage_bytes || true) {
-            int rc = eisen_staging(ctx, bytes, &st);
-            if (rc) return rc;
-        }
-        memcpy(st, src, bytes);
-        EISEN_HIP_TRY(ctx, hipMemcpyAsync(dst, st, bytes, hipMemcpyHostToDevice, ctx->stream));
+        eisen_ctx::StageSlot* st = nullptr;
+        int rc = eisen_staging(ctx, bytes, &st);
+        if (rc) return rc;
+        memcpy(st->ptr, src, bytes);
+        EISEN_HIP_TRY(ctx, hipMemcpyAsync(dst, st->ptr, bytes, hipMemcpyHostToDevice, ctx->stream));
+        EISEN_HIP_TRY(ctx, hipEventRecord(st->done, ctx->stream));
+        st->in_flight = true;
         return 0;
     }
     EISEN_HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
@@ -286,5 +295,69 @@ extern "C" int eisen_hip_timer_stop(eisen_ctx* ctx, float* ms_out) {
     EISEN_HIP_TRY(ctx, hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop));
     ctx->timer_running = false;
     if (ms_out) *ms_out = ms;
+    return 0;
+}
+
+// ---- per-kernel timing ----------------------------------------------------------------------------
+
+int eisen_prof_begin(eisen_ctx* ctx, const char* name, double work, bool is_flops) {
+    eisen_prof& p = ctx->prof;
+    int key = -1;
+    for (size_t i = 0; i < p.names.size(); i++)
+        if (p.names[i] == name) key = (int)i;
+    if (key < 0) {
+        p.names.push_back(name);
+        p.is_flops.push_back(is_flops ? 1 : 0);
+        key = (int)p.names.size() - 1;
+    }
+    while (p.pool.size() < p.pool_used + 2) {
+        hipEvent_t e;
+        if (hipEventCreate(&e) != hipSuccess) return -1;
+        p.pool.push_back(e);
+    }
+    eisen_prof_rec r{key, p.pool[p.pool_used], p.pool[p.pool_used + 1], work};
+    p.pool_used += 2;
+    if (hipEventRecord(r.start, ctx->stream) != hipSuccess) return -1;
+    p.recs.push_back(r);
+    return (int)p.recs.size() - 1;
+}
+void eisen_prof_end(eisen_ctx* ctx, int rec) { (void)hipEventRecord(ctx->prof.recs[rec].stop, ctx->stream); }
+
+extern "C" int eisen_hip_profile_start(eisen_ctx* ctx) {
+    EISEN_CHECK_CTX(ctx);
+    ctx->prof.enabled = true;
+    ctx->prof.recs.clear();
+    ctx->prof.pool_used = 0;
+    return 0;
+}
+
+extern "C" int eisen_hip_profile_stop(eisen_ctx* ctx, eisen_prof_entry* out, size_t capacity, size_t* count_out) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, count_out != nullptr, EISEN_E_ARG, "eisen_hip_profile_stop: null count_out");
+    eisen_prof& p = ctx->prof;
+    p.enabled = false;
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    std::vector<eisen_prof_entry> acc(p.names.size());
+    for (size_t i = 0; i < p.names.size(); i++) {
+        std::memset(&acc[i], 0, sizeof(eisen_prof_entry));
+        std::strncpy(acc[i].name, p.names[i].c_str(), sizeof(acc[i].name) - 1);
+        acc[i].work_is_flops = p.is_flops[i];
+    }
+    for (const eisen_prof_rec& r : p.recs) {
+        float ms = 0.f;
+        EISEN_HIP_TRY(ctx, hipEventElapsedTime(&ms, r.start, r.stop));
+        acc[r.key].ms += ms;
+        acc[r.key].work += r.work;
+        acc[r.key].launches += 1;
+    }
+    size_t n = 0;
+    for (const eisen_prof_entry& e : acc)
+        if (e.launches) {
+            if (out && n < capacity) out[n] = e;
+            n++;
+        }
+    *count_out = n;
+    p.recs.clear();
+    p.pool_used = 0;
     return 0;
 }

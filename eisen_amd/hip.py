@@ -39,6 +39,10 @@ class ParamSlot(C.Structure):
     _fields_ = [("w", _vp), ("g", _vp), ("m", _vp), ("v", _vp), ("w_bf16", _vp), ("n", _sz)]
 
 
+class ProfEntry(C.Structure):
+    _fields_ = [("name", C.c_char * 48), ("ms", C.c_double), ("work", C.c_double), ("launches", C.c_ulonglong), ("work_is_flops", C.c_int)]
+
+
 class Buffer:
     """A device allocation from the context's pool."""
 
@@ -150,6 +154,20 @@ class Context:
         ms = _f()
         self._call("eisen_hip_timer_stop", C.byref(ms))
         return ms.value
+
+    def profile_start(self):
+        """Bracket every instrumented kernel launch with HIP events on the context's stream."""
+        self._call("eisen_hip_profile_start")
+
+    def profile_stop(self):
+        """-> {kernel family: dict(ms, launches, work, unit)}; synchronises."""
+        arr = (ProfEntry * 64)()
+        n = _sz()
+        self._call("eisen_hip_profile_stop", arr, _sz(64), C.byref(n))
+        out = {}
+        for e in arr[:min(n.value, 64)]:
+            out[e.name.decode()] = dict(ms=e.ms, launches=int(e.launches), work=e.work, unit="flop" if e.work_is_flops else "byte")
+        return out
 
     # ---- by-name launch ---------------------------------------------------------------
     def module_load(self, path=HSACO_PATH):

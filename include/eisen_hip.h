@@ -95,6 +95,20 @@ int eisen_hip_launch(eisen_ctx* ctx, eisen_function* fn, const unsigned grid[3],
 int eisen_hip_timer_start(eisen_ctx* ctx);
 int eisen_hip_timer_stop(eisen_ctx* ctx, float* ms_out);
 
+/* Per-kernel timing for roofline reports: between start and stop every instrumented launch is
+ * bracketed by two HIP events on the context's stream.  stop() synchronises and returns one
+ * entry per kernel family that ran: total milliseconds, launches, and the algorithmic work
+ * (flops for the MFMA kernels, bytes for the HBM-bound ones) those launches were asked for. */
+typedef struct {
+    char name[48];
+    double ms;
+    double work;
+    unsigned long long launches;
+    int work_is_flops;
+} eisen_prof_entry;
+int eisen_hip_profile_start(eisen_ctx* ctx);
+int eisen_hip_profile_stop(eisen_ctx* ctx, eisen_prof_entry* out, size_t capacity, size_t* count_out);
+
 /* ---- elementwise ---------------------------------------------------------------------- */
 
 /* fill_f32 / scale_f32 (kernels/ops_f32.cu:101,107; callers src/graph/mod.rs:683-693,

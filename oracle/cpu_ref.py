@@ -491,6 +491,30 @@ class Graph:
         return _lib.ref_gqa_forward(self.h, heads, kv_heads, head_dim, wq, wk, wv, wo, x, int(causal))
 
 
+def attention_chain(q, k, v, do, scale, causal=True):
+    """q, do: [B,S,Hq,hd]; k, v: [B,S,Hkv,hd].  The reference's training chain
+    (src/nn/attention.rs:319-378): transpose_0213, repeat_kv, bmm(q,k^T), mul(scale), add(mask),
+    softmax, bmm(p,v), transpose back.  Returns O, dQ, dK, dV in the input layouts."""
+    B, S, Hq, hd = q.shape
+    Hkv = k.shape[2]
+    g = Graph()
+    qi, ki, vi = g.alloc(q.shape, q), g.alloc(k.shape, k), g.alloc(v.shape, v)
+    qt, kt, vt = g.transpose_0213(qi), g.transpose_0213(ki), g.transpose_0213(vi)
+    kr, vr = g.repeat_kv(kt, Hq // Hkv), g.repeat_kv(vt, Hq // Hkv)
+    for t in (qt, kr, vr):
+        g.reinterpret_shape(t, (B * Hq, S, hd))
+    sc = g.bmm(qt, kr, True)
+    sc = g.mul_const(sc, g.alloc((B * Hq, S, S), np.full((B * Hq, S, S), scale, np.float32)))
+    if causal:
+        sc = g.add(sc, g.alloc((1, S, S), np.triu(np.full((S, S), -1e20, np.float32), 1)))
+    ctx_ = g.bmm(g.softmax(sc), vr, False)
+    g.reinterpret_shape(ctx_, (B, Hq, S, hd))
+    o = g.transpose_0213(ctx_)
+    seed = g.alloc(do.shape, do)
+    g.backward(g.sum(g.sum(g.sum(g.sum(g.mul(o, seed), 3), 2), 1), 0))
+    return g.data(o), g.grad(qi), g.grad(ki), g.grad(vi)
+
+
 class TransformerLM:
     """Mirror of src/nn/transformer.rs TransformerLM over the C oracle."""
 
