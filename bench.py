@@ -130,7 +130,12 @@ def bench_lm(name, steps, warmup, cpu_tokens):
     batches = [(x.astype(np.float32), y) for x, y in batches]
     it = iter(batches)
 
+    step_no = [0]
+
     def one_step(want_loss=False):
+        # linear warm-up of the reference's CosineScheduler (src/nn/scheduler.rs:45-55; train_llm.rs:391-392)
+        opt.config(g.cosine_lr(3e-4, 3e-5, 100, 10000, step_no[0]), 0.9, 0.95, 1e-8, 0.1, 1.0)
+        step_no[0] += 1
         opt.zero_grad()
         loss = None
         for _ in range(c["accum"]):

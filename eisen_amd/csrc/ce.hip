@@ -1,8 +1,8 @@
 // Fused softmax-cross-entropy forward+backward: one read of the logits, one write of dLogits.
 //
 // One workgroup owns one row.  The row is loaded once with 16-byte packets and stays in
-// registers (VPT packets per lane) across the three phases: row max (+ first argmax), sum of
-// exponentials, gradient write.  Reductions are wave64 shuffles plus one LDS exchange
+// registers (VPT packets per lane, widened to f32) across the three phases: row max (+ first
+// argmax when asked for), exponentials (computed once, kept) and their sum, gradient write.  Reductions are wave64 shuffles plus one LDS exchange
 // between the block's waves.  Per-row losses go to a buffer; a second one-block kernel sums
 // them in a fixed order, so the loss carries no float atomics and is reproducible.
 //
@@ -33,13 +33,14 @@ __device__ __forceinline__ ArgMax wave_argmax(ArgMax a) {
     return a;
 }
 
-template <typename T, int THREADS, int VPT>
+template <typename T, int THREADS, int VPT, bool WANT_ARGMAX>
 __global__ __launch_bounds__(THREADS) void ce_fused_kernel(const T* __restrict__ logits, const int32_t* __restrict__ targets,
                                                            T* __restrict__ dlogits, float* __restrict__ row_loss,
                                                            int32_t* __restrict__ argmax_out, float* __restrict__ target_logit_out,
                                                            int classes, float scale) {
     constexpr int N = Pack<T>::N;
     constexpr int W = THREADS / kWave;
+    constexpr float kLog2e = 1.4426950408889634f;
     __shared__ float s_f[W];
     __shared__ int s_i[W];
     const size_t row = blockIdx.x;
@@ -68,69 +69,87 @@ __global__ __launch_bounds__(THREADS) void ce_fused_kernel(const T* __restrict__
         return;
     }
 
-    Pack<T> x[VPT];
+    // phase 1: the row comes in once (VPT packets per lane, all loads in flight together) and is
+    // widened to f32 registers; running maximum (and, when asked for, its first index)
+    float x[VPT][N];
     ArgMax am{-INFINITY, 0x7fffffff};
 #pragma unroll
     for (int v = 0; v < VPT; v++) {
         const int c = (v * THREADS + threadIdx.x) * N;
         if (c < classes) {
-            x[v] = load_pack(xr + c);
+            const Pack<T> pk = load_pack(xr + c);
 #pragma unroll
             for (int j = 0; j < N; j++) {
-                const float f = x[v].get(j);
-                if (f > am.v) {  // ascending c within the lane: strict > keeps the first
-                    am.v = f;
-                    am.i = c + j;
+                x[v][j] = pk.get(j);
+                if (WANT_ARGMAX) {
+                    if (x[v][j] > am.v) {  // ascending c within the lane: strict > keeps the first
+                        am.v = x[v][j];
+                        am.i = c + j;
+                    }
+                } else {
+                    am.v = fmaxf(am.v, x[v][j]);
                 }
             }
         }
     }
-    am = wave_argmax(am);
-    if (W > 1) {
-        if (lane == 0) {
-            s_f[wid] = am.v;
-            s_i[wid] = am.i;
-        }
-        __syncthreads();
-        am = ArgMax{s_f[0], s_i[0]};
+    if (WANT_ARGMAX) {
+        am = wave_argmax(am);
+        if (W > 1) {
+            if (lane == 0) {
+                s_f[wid] = am.v;
+                s_i[wid] = am.i;
+            }
+            __syncthreads();
+            am = ArgMax{s_f[0], s_i[0]};
 #pragma unroll
-        for (int k = 1; k < W; k++) am = argmax_combine(am, ArgMax{s_f[k], s_i[k]});
-        __syncthreads();
+            for (int k = 1; k < W; k++) am = argmax_combine(am, ArgMax{s_f[k], s_i[k]});
+            __syncthreads();
+        }
+    } else {
+        am.v = block_max<THREADS>(am.v, s_f);
     }
     const float mx = am.v;
 
+    // phase 2: e = 2^(x*log2e - max*log2e), kept in the same registers; row sum
+    const float bias = -mx * kLog2e;
     float sum = 0.f;
 #pragma unroll
     for (int v = 0; v < VPT; v++) {
         const int c = (v * THREADS + threadIdx.x) * N;
         if (c < classes) {
 #pragma unroll
-            for (int j = 0; j < N; j++) sum += __expf(x[v].get(j) - mx);
+            for (int j = 0; j < N; j++) {
+                if (c + j == target && target_logit_out) target_logit_out[row] = x[v][j];
+                x[v][j] = exp2f(fmaf(x[v][j], kLog2e, bias));
+                sum += x[v][j];
+            }
         }
     }
     sum = block_sum<THREADS>(sum, s_f);
     const float inv = 1.0f / sum;
+    const float gscale = inv * scale;
 
+    // phase 3: dlogit = (e/sum - onehot) * scale, one multiply per element; the lane that holds the
+    // target fixes its element up and writes the row loss
 #pragma unroll
     for (int v = 0; v < VPT; v++) {
         const int c = (v * THREADS + threadIdx.x) * N;
         if (c < classes) {
             Pack<T> g;
+            const bool has_target = target >= c && target < c + N;
 #pragma unroll
             for (int j = 0; j < N; j++) {
-                const float xv = x[v].get(j);
-                float p = __expf(xv - mx) * inv;
-                if (c + j == target) {
-                    row_loss[row] = -logf(p + 1e-8f);
-                    if (target_logit_out) target_logit_out[row] = xv;
-                    p -= 1.0f;
+                float gv = x[v][j] * gscale;
+                if (has_target && c + j == target) {
+                    row_loss[row] = -logf(x[v][j] * inv + 1e-8f);
+                    gv -= scale;
                 }
-                g.set(j, p * scale);
+                g.set(j, gv);
             }
             store_pack(gr + c, g);
         }
     }
-    if (threadIdx.x == 0 && argmax_out) argmax_out[row] = am.i;
+    if (WANT_ARGMAX && threadIdx.x == 0 && argmax_out) argmax_out[row] = am.i;
 }
 
 // Generic row kernel for class counts that do not fit the register-resident variants or
@@ -207,8 +226,12 @@ __global__ __launch_bounds__(1024) void ce_loss_reduce_kernel(const float* __res
 template <typename T, int THREADS, int VPT>
 void launch_fused(eisen_ctx* ctx, const void* logits, const int32_t* targets, void* dlogits, float* row_loss,
                   int32_t* argmax_out, float* target_logit_out, size_t rows, size_t classes, float scale) {
-    ce_fused_kernel<T, THREADS, VPT><<<dim3((unsigned)rows), dim3(THREADS), 0, ctx->stream>>>(
-        (const T*)logits, targets, (T*)dlogits, row_loss, argmax_out, target_logit_out, (int)classes, scale);
+    if (argmax_out)
+        ce_fused_kernel<T, THREADS, VPT, true><<<dim3((unsigned)rows), dim3(THREADS), 0, ctx->stream>>>(
+            (const T*)logits, targets, (T*)dlogits, row_loss, argmax_out, target_logit_out, (int)classes, scale);
+    else
+        ce_fused_kernel<T, THREADS, VPT, false><<<dim3((unsigned)rows), dim3(THREADS), 0, ctx->stream>>>(
+            (const T*)logits, targets, (T*)dlogits, row_loss, argmax_out, target_logit_out, (int)classes, scale);
 }
 
 template <typename T>

@@ -8,6 +8,8 @@ namespace {
 
 constexpr int kRowThreads = 256;  // 4 waves = 4 rows per block
 constexpr int kRowWaves = kRowThreads / kWave;
+constexpr int kBwdThreads = 512;  // backward: 8 waves per block share one partial-dw row
+constexpr int kBwdWaves = kBwdThreads / kWave;
 
 // y = x * rrms * w,  rrms = 1/sqrt(mean(x^2) + eps)   (src/graph/ops/normalization.rs:141-151)
 template <typename T, bool VEC>
@@ -39,7 +41,13 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_fwd_kernel(const T* __re
             const Pack<T> p = load_pack(xr + c);  // second read of a row this wave just streamed: L2/TCP hit
             Pack<T> o;
 #pragma unroll
-            for (int j = 0; j < N; j++) o.set(j, p.get(j) * rrms * w[c + j]);
+            for (int j = 0; j < N; j += 4) {
+                const float4 g4 = *reinterpret_cast<const float4*>(w + c + j);
+                o.set(j, p.get(j) * rrms * g4.x);
+                o.set(j + 1, p.get(j + 1) * rrms * g4.y);
+                o.set(j + 2, p.get(j + 2) * rrms * g4.z);
+                o.set(j + 3, p.get(j + 3) * rrms * g4.w);
+            }
             store_pack(orow + c, o);
         } else {
             orow[c] = from_f32<T>(to_f32(xr[c]) * rrms * w[c]);
@@ -52,37 +60,59 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_fwd_kernel(const T* __re
 // and keeps its dw partial in registers; partials meet in LDS and leave as one row of
 // `partial` per block.  A second kernel sums the block rows in fixed order.
 template <typename T, int MAXP>
-__global__ __launch_bounds__(kRowThreads) void rms_norm_bwd_kernel(const T* __restrict__ x, const float* __restrict__ w,
+__global__ __launch_bounds__(kBwdThreads) void rms_norm_bwd_kernel(const T* __restrict__ x, const float* __restrict__ w,
                                                                    const float* __restrict__ rrms_in,
                                                                    const T* __restrict__ go, T* __restrict__ gx,
                                                                    float* __restrict__ partial, size_t rows, int dim,
                                                                    int accumulate_x) {
     constexpr int N = Pack<T>::N;
-    extern __shared__ float lds[];  // [kRowWaves][dim]
+    extern __shared__ float lds[];  // [kBwdWaves][dim]
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
-    const size_t wave_global = (size_t)blockIdx.x * kRowWaves + wid;
-    const size_t wave_stride = (size_t)gridDim.x * kRowWaves;
+    const size_t wave_global = (size_t)blockIdx.x * kBwdWaves + wid;
+    const size_t wave_stride = (size_t)gridDim.x * kBwdWaves;
     float dw[MAXP][N];
 #pragma unroll
     for (int p = 0; p < MAXP; p++)
 #pragma unroll
         for (int j = 0; j < N; j++) dw[p][j] = 0.f;
 
+    // a lane owns the same columns in every row: its gains live in registers
+    float wv[MAXP][N];
+#pragma unroll
+    for (int p = 0; p < MAXP; p++) {
+        const int c = (p * kWave + lane) * N;
+#pragma unroll
+        for (int j = 0; j < N; j += 4) {
+            const float4 t = c < dim ? *reinterpret_cast<const float4*>(w + c + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            wv[p][j] = t.x; wv[p][j + 1] = t.y; wv[p][j + 2] = t.z; wv[p][j + 3] = t.w;
+        }
+    }
+    // the next row's packets are requested before the current row is reduced, so a wave always has
+    // two rows of loads in flight
+    Pack<T> xp[MAXP], gp[MAXP], xn[MAXP], gn[MAXP];
+    auto fetch = [&](size_t row, Pack<T>* xd, Pack<T>* gd) {
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) {
+            const int c = (p * kWave + lane) * N;
+            if (c < dim) {
+                xd[p] = load_pack(x + row * dim + c);
+                gd[p] = load_pack(go + row * dim + c);
+            }
+        }
+    };
+    if (wave_global < rows) fetch(wave_global, xp, gp);
     for (size_t row = wave_global; row < rows; row += wave_stride) {
-        const T* xr = x + row * dim;
-        const T* gr = go + row * dim;
         T* gxr = gx + row * dim;
         const float rrms = rrms_in[row];
-        Pack<T> xp[MAXP], gp[MAXP];
+        const size_t next = row + wave_stride;
+        if (next < rows) fetch(next, xn, gn);
         float gdxw = 0.f;
 #pragma unroll
         for (int p = 0; p < MAXP; p++) {
             const int c = (p * kWave + lane) * N;
             if (c < dim) {
-                xp[p] = load_pack(xr + c);
-                gp[p] = load_pack(gr + c);
 #pragma unroll
-                for (int j = 0; j < N; j++) gdxw += gp[p].get(j) * xp[p].get(j) * w[c + j];
+                for (int j = 0; j < N; j++) gdxw += gp[p].get(j) * xp[p].get(j) * wv[p][j];
             }
         }
         gdxw = wave_sum(gdxw);
@@ -96,12 +126,17 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_bwd_kernel(const T* __re
 #pragma unroll
                 for (int j = 0; j < N; j++) {
                     const float xv = xp[p].get(j), gv = gp[p].get(j);
-                    const float dx = rrms * (gv * w[c + j]) - xv * rrc_d * gdxw;
+                    const float dx = rrms * (gv * wv[p][j]) - xv * rrc_d * gdxw;
                     o.set(j, accumulate_x ? o.get(j) + dx : dx);
                     dw[p][j] += gv * xv * rrms;
                 }
                 store_pack(gxr + c, o);
             }
+        }
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) {
+            xp[p] = xn[p];
+            gp[p] = gn[p];
         }
     }
     // combine the block's waves in a fixed order
@@ -113,20 +148,32 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_bwd_kernel(const T* __re
             for (int j = 0; j < N; j++) lds[wid * dim + c + j] = dw[p][j];
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < dim; c += kRowThreads) {
+    for (int c = threadIdx.x; c < dim; c += kBwdThreads) {
         float s = 0.f;
 #pragma unroll
-        for (int k = 0; k < kRowWaves; k++) s += lds[k * dim + c];
+        for (int k = 0; k < kBwdWaves; k++) s += lds[k * dim + c];
         partial[(size_t)blockIdx.x * dim + c] = s;
     }
 }
 
-__global__ void rms_norm_dw_reduce_kernel(const float* __restrict__ partial, float* __restrict__ gw, int nblocks, int dim) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= dim) return;
+// Second stage: gw[c] += sum over the block rows of `partial`, in a fixed order.  A workgroup owns
+// 32 columns; its 8 row groups each add every 8th partial row, then meet in LDS (group 0..7 in order).
+__global__ __launch_bounds__(256) void rms_norm_dw_reduce_kernel(const float* __restrict__ partial, float* __restrict__ gw, int nblocks, int dim) {
+    __shared__ float sh[8][32];
+    const int cl = threadIdx.x & 31, rg = threadIdx.x >> 5;
+    const int c = blockIdx.x * 32 + cl;
     float s = 0.f;
-    for (int b = 0; b < nblocks; b++) s += partial[(size_t)b * dim + c];
-    gw[c] += s;
+    if (c < dim)
+#pragma unroll 8
+        for (int b = rg; b < nblocks; b += 8) s += partial[(size_t)b * dim + c];
+    sh[rg][cl] = s;
+    __syncthreads();
+    if (rg == 0 && c < dim) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) t += sh[k][cl];
+        gw[c] += t;
+    }
 }
 
 // Scalar fallback for rows that are not packet-aligned: one wave per row, same arithmetic.
@@ -202,7 +249,7 @@ __global__ __launch_bounds__(kRowThreads) void softmax_bwd_kernel(const T* __res
 template <typename T>
 int rms_norm_fwd(eisen_ctx* ctx, const void* x, const float* w, void* out, float* rrms, size_t rows, size_t dim, float eps) {
     const unsigned blocks = (unsigned)eisen_ceil_div(rows, kRowWaves);
-    const bool vec = dim % Pack<T>::N == 0 && eisen_aligned(x, 16) && eisen_aligned(out, 16);
+    const bool vec = dim % Pack<T>::N == 0 && eisen_aligned(x, 16) && eisen_aligned(out, 16) && eisen_aligned(w, 16);
     if (vec)
         rms_norm_fwd_kernel<T, true><<<blocks, kRowThreads, 0, ctx->stream>>>((const T*)x, w, (T*)out, rrms, rows, (int)dim, eps);
     else
@@ -215,15 +262,15 @@ template <typename T, int MAXP>
 int rms_norm_bwd_vec(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* gw,
                      size_t rows, size_t dim, int accumulate_x) {
     // enough waves to cover the chip a few times over, few enough that the partial rows stay small
-    unsigned blocks = (unsigned)std::min<size_t>(eisen_ceil_div(rows, kRowWaves), 512);
+    unsigned blocks = (unsigned)std::min<size_t>(eisen_ceil_div(rows, kBwdWaves), 256);
     void* ws = nullptr;
     int rc = eisen_workspace(ctx, (size_t)blocks * dim * sizeof(float), &ws);
     if (rc) return rc;
-    const size_t lds = (size_t)kRowWaves * dim * sizeof(float);
-    rms_norm_bwd_kernel<T, MAXP><<<blocks, kRowThreads, lds, ctx->stream>>>((const T*)x, w, rrms, (const T*)go, (T*)gx,
+    const size_t lds = (size_t)kBwdWaves * dim * sizeof(float);
+    rms_norm_bwd_kernel<T, MAXP><<<blocks, kBwdThreads, lds, ctx->stream>>>((const T*)x, w, rrms, (const T*)go, (T*)gx,
                                                                             (float*)ws, rows, (int)dim, accumulate_x);
     EISEN_LAUNCH_CHECK(ctx, "rms_norm_bwd_kernel");
-    rms_norm_dw_reduce_kernel<<<(unsigned)eisen_ceil_div(dim, 256), 256, 0, ctx->stream>>>((const float*)ws, gw, (int)blocks, (int)dim);
+    rms_norm_dw_reduce_kernel<<<(unsigned)eisen_ceil_div(dim, 32), 256, 0, ctx->stream>>>((const float*)ws, gw, (int)blocks, (int)dim);
     EISEN_LAUNCH_CHECK(ctx, "rms_norm_dw_reduce_kernel");
     return 0;
 }
@@ -232,8 +279,8 @@ template <typename T>
 int rms_norm_bwd(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* gw,
                  size_t rows, size_t dim, int accumulate_x) {
     constexpr int N = Pack<T>::N;
-    const bool vec = dim % N == 0 && eisen_aligned(x, 16) && eisen_aligned(go, 16) && eisen_aligned(gx, 16) &&
-                     dim <= (size_t)kWave * N * 8 && (size_t)kRowWaves * dim * sizeof(float) <= 64 * 1024;
+    const bool vec = dim % N == 0 && eisen_aligned(x, 16) && eisen_aligned(go, 16) && eisen_aligned(gx, 16) && eisen_aligned(w, 16) &&
+                     dim <= (size_t)kWave * N * 8 && (size_t)kBwdWaves * dim * sizeof(float) <= 64 * 1024;
     if (vec) {
         const size_t packs = eisen_ceil_div(dim, (size_t)kWave * N);
         if (packs <= 1) return rms_norm_bwd_vec<T, 1>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
