@@ -32,6 +32,14 @@ from tests import gen  # noqa: E402  (seeded synthetic inputs shared with the te
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM-side bytes per launch (average over the launches of the config-5 step), from the FETCH_SIZE / WRITE_SIZE
+# runs summarised in profiles/c5_step_hbm_traffic_pmc.md (fetch x 1.997, write x 1.000 after calibration on
+# the library's copy kernel).  Keys are the profile names the library reports.
+MEASURED_TRAFFIC = {
+    "gemm_tn_bf16_f32out_128x128x32": 374.5e6,
+    "ce_fused_bf16": 524.6e6,
+}
+
 CONFIGS = {
     "c5": dict(vocab=32000, hidden=2048, heads=32, kv_heads=8, ffn=5632, layers=16, tie=False, seq=1024, mb=4, accum=8,
                label="config5 ~1.1B Llama-style (852,559,872 params untied), bf16 mixed, seq 1024, micro-batch 4, accum 8"),
@@ -59,10 +67,10 @@ def pick_dominant(prof):
     if e["unit"] == "flop":
         achieved = e["work"] / e["launches"] / (per_launch_ms * 1e-3) / 1e12
         return name, dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                          frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=None)
+                          frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(name))
     achieved = e["work"] / e["launches"] / (per_launch_ms * 1e-3) / 1e9
     return name, dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None)
+                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(name))
 
 
 def kernel_table(prof):
