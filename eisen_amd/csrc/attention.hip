@@ -65,26 +65,41 @@ __device__ __forceinline__ bf16x8 lds_tr_operand(const bf16_t* tile, int pitch, 
     return concat4(lds_read_tr(p), lds_read_tr(p + 8 * pitch));
 }
 
-// Cooperative copy of `rows` x HD bf16 (16-byte chunks) from a strided global tensor into LDS.
-template <int HD, int THREADS>
-__device__ __forceinline__ void load_tile(bf16_t* dst, const bf16_t* src, long long row_stride, int first_row, int rows,
-                                          int limit_rows) {
-    constexpr int PITCH = HD + 8, CPR = HD / 8;
-    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int c = threadIdx.x; c < rows * CPR; c += THREADS) {
-        const int r = c / CPR, cc = c % CPR;
-        const int gr = first_row + r;
-        const bf16x8 v = gr < limit_rows ? *reinterpret_cast<const bf16x8*>(src + (long long)gr * row_stride + cc * 8) : zero8;
-        *reinterpret_cast<bf16x8*>(dst + r * PITCH + cc * 8) = v;
+// 2^x as the bare hardware instruction: results below 2^-126 flush to zero, which is what a softmax
+// weight that small should be; the library exp2f spends four more instructions per value on them.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// A ROWS x HD bf16 tile on its way from a strided global tensor into LDS, held in registers in
+// between so the global loads of tile i+1 are in flight while tile i is being used.
+template <int HD, int ROWS, int THREADS>
+struct TilePrefetch {
+    static constexpr int PITCH = HD + 8, CPR = HD / 8, TOTAL = ROWS * CPR;
+    static constexpr int CH = (TOTAL + THREADS - 1) / THREADS;
+    bf16x8 r[CH];
+    __device__ __forceinline__ void fetch(const bf16_t* src, long long row_stride, int first_row, int limit_rows) {
+        const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int c = i * THREADS + threadIdx.x;
+            const int row = c / CPR, cc = c % CPR, gr = first_row + row;
+            r[i] = (c < TOTAL && gr < limit_rows) ? *reinterpret_cast<const bf16x8*>(src + (long long)gr * row_stride + cc * 8) : zero8;
+        }
     }
-}
+    __device__ __forceinline__ void commit(bf16_t* dst) const {
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const int c = i * THREADS + threadIdx.x;
+            if (c < TOTAL) *reinterpret_cast<bf16x8*>(dst + (c / CPR) * PITCH + (c % CPR) * 8) = r[i];
+        }
+    }
+};
 
 // ---- forward -------------------------------------------------------------------------------
 template <int HD, int GW>
 __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
     constexpr int QS = 4 / GW, BKV = 64, PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * PITCH];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[BKV * PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t Ksb[2][BKV * PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t Vsb[2][BKV * PITCH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, c = lane & 31;
     const int hsub = wave % GW, qsub = wave / GW;
     const int qblk = gridDim.x - 1 - blockIdx.x;  // long rows first
@@ -112,11 +127,19 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
     const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
     const int my_qmax = q0 < a.S ? q0 + 31 : -1;
 
+    TilePrefetch<HD, BKV, 256> pk, pv;
+    pk.fetch(Kp, a.k_ss, 0, a.S);
+    pv.fetch(Vp, a.k_ss, 0, a.S);
     for (int kt = 0; kt < n_kt; kt++) {
-        __syncthreads();
-        load_tile<HD, 256>(Ks, Kp, a.k_ss, kt * BKV, BKV, a.S);
-        load_tile<HD, 256>(Vs, Vp, a.k_ss, kt * BKV, BKV, a.S);
-        __syncthreads();
+        const bf16_t* Ks = Ksb[kt & 1];
+        const bf16_t* Vs = Vsb[kt & 1];
+        pk.commit(Ksb[kt & 1]);
+        pv.commit(Vsb[kt & 1]);
+        __syncthreads();  // one barrier per tile: the other buffer is only rewritten after the next barrier
+        if (kt + 1 < n_kt) {
+            pk.fetch(Kp, a.k_ss, (kt + 1) * BKV, a.S);
+            pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
+        }
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
             const int k0 = kt * BKV + sub * 32;
@@ -129,23 +152,26 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                 const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
             }
-            float mx = -INFINITY;
+            // only tiles that touch the diagonal or the end of the sequence need the mask
+            const bool need_mask = (a.causal && k0 + 31 > q0) || k0 + 32 > a.S;
+            float mx = -INFINITY;  // of the raw scores; the (positive) scale is folded into the exponent's fma
+            if (need_mask) {
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int key = k0 + acc_row(v, g);
-                float val = s[v] * a.scale_log2e;
-                if ((a.causal && key > q) || key >= a.S) val = -INFINITY;
-                s[v] = val;
-                mx = fmaxf(mx, val);
+                for (int v = 0; v < 16; v++) {
+                    const int key = k0 + acc_row(v, g);
+                    if ((a.causal && key > q) || key >= a.S) s[v] = -INFINITY;
+                }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+#pragma unroll
+            for (int v = 0; v < 16; v++) mx = fmaxf(mx, s[v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2e;
             const float m_new = fmaxf(m, mx);
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = exp2f(m - m_use);
+            const float alpha = fast_exp2(m - m_use);
             float rowsum = 0.f;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                s[v] = exp2f(s[v] - m_use);
+                s[v] = fast_exp2(fmaf(s[v], a.scale_log2e, -m_use));
                 rowsum += s[v];
             }
             rowsum += __shfl_xor(rowsum, 32, 64);
@@ -188,8 +214,8 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
 template <int HD, int GW>
 __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
     constexpr int QS = 4 / GW, BKV = 64, PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * PITCH];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[BKV * PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t Ksb[2][BKV * PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t Vsb[2][BKV * PITCH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, c = lane & 31;
     const int hsub = wave % GW, qsub = wave / GW;
     const int qblk = gridDim.x - 1 - blockIdx.x;
@@ -228,11 +254,19 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
     const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
     const int my_qmax = q0 < a.S ? q0 + 31 : -1;
 
+    TilePrefetch<HD, BKV, 256> pk, pv;
+    pk.fetch(Kp, a.k_ss, 0, a.S);
+    pv.fetch(Vp, a.k_ss, 0, a.S);
     for (int kt = 0; kt < n_kt; kt++) {
+        const bf16_t* Ks = Ksb[kt & 1];
+        const bf16_t* Vs = Vsb[kt & 1];
+        pk.commit(Ksb[kt & 1]);
+        pv.commit(Vsb[kt & 1]);
         __syncthreads();
-        load_tile<HD, 256>(Ks, Kp, a.k_ss, kt * BKV, BKV, a.S);
-        load_tile<HD, 256>(Vs, Vp, a.k_ss, kt * BKV, BKV, a.S);
-        __syncthreads();
+        if (kt + 1 < n_kt) {
+            pk.fetch(Kp, a.k_ss, (kt + 1) * BKV, a.S);
+            pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
+        }
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
             const int k0 = kt * BKV + sub * 32;
@@ -248,12 +282,21 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                 dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[st], dp, 0, 0, 0);
             }
             bf16x8 dsf[2];
+            const bool need_mask = (a.causal && k0 + 31 > q0) || k0 + 32 > a.S;
+            if (need_mask) {
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int key = k0 + acc_row(v, g);
-                const bool masked = (a.causal && key > q) || key >= a.S;
-                const float p = masked ? 0.f : exp2f(s[v] * a.scale_log2e - lse2);
-                dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - Dq));
+                for (int v = 0; v < 16; v++) {
+                    const int key = k0 + acc_row(v, g);
+                    const bool masked = (a.causal && key > q) || key >= a.S;
+                    const float p = masked ? 0.f : fast_exp2(s[v] * a.scale_log2e - lse2);
+                    dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - Dq));
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const float p = fast_exp2(s[v] * a.scale_log2e - lse2);
+                    dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - Dq));
+                }
             }
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
@@ -279,68 +322,116 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
 }
 
 // ---- backward: dK, dV (key-stationary, summed over the query heads of the group) -------------
+// One block owns the keys of two 32-key blocks of one KV head, a heavy one and its light mirror image
+// under the causal mask, so every block of the grid has the same amount of work.  Its four waves
+// each take every fourth (query head of the group, 32-query tile) item, with a private LDS tile and
+// no block barrier inside the item loop; their partial dK/dV are summed through LDS once per key block.
 template <int HD>
 __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
-    constexpr int PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
-    __shared__ __attribute__((aligned(16))) bf16_t Qs[32 * PITCH];
-    __shared__ __attribute__((aligned(16))) bf16_t dOs[32 * PITCH];
-    __shared__ float lse_s[32], d_s[32];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, c = lane & 31;
-    const int kb = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-    const int k0w = kb * 128 + wave * 32, key = k0w + c;
-    const bool valid_k = key < a.S;
-    const long long koff = b * a.k_sb + kvh * a.k_sh + (long long)key * a.k_ss;
-    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    bf16x8 kf[KSTEPS], vf[KSTEPS];
-#pragma unroll
-    for (int st = 0; st < KSTEPS; st++) {
-        const int d = st * 16 + 8 * g;
-        kf[st] = valid_k ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.K) + koff + d) : zero8;
-        vf[st] = valid_k ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.V) + koff + d) : zero8;
-    }
-    f32x16 dk[DT], dv[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) { dk[dt][v] = 0.f; dv[dt][v] = 0.f; }
-
+    constexpr int PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32, TILE = 32 * PITCH;
+    constexpr int CPR = HD / 8, CH = 32 * CPR / 64;  // 16-byte chunks per row / per lane of a tile
+    __shared__ __attribute__((aligned(16))) bf16_t tiles[4][2][TILE];  // per wave: Q tile, dO tile
+    __shared__ __attribute__((aligned(16))) float stats[4][64];        // per wave: LSE*log2(e) | D
+    static_assert(2 * TILE * sizeof(bf16_t) >= 32 * HD * sizeof(float), "reduction scratch reuses the tiles");
+    const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kvh = blockIdx.y, b = blockIdx.z;
     const int n_qt = (a.S + 31) / 32;
-    const int qt_start = a.causal ? kb * 4 : 0;  // first query tile that can see this block's first key
-    for (int hh = 0; hh < a.G; hh++) {
-        const int hq = kvh * a.G + hh;
-        const bf16_t* Qp = static_cast<const bf16_t*>(a.Q) + b * a.q_sb + hq * a.q_sh;
-        const bf16_t* dOp = static_cast<const bf16_t*>(a.dO) + b * a.q_sb + hq * a.q_sh;
-        const long long stat0 = ((long long)b * a.Hq + hq) * a.S;
-        for (int qt = qt_start; qt < n_qt; qt++) {
-            const int q0 = qt * 32;
-            __syncthreads();
-            load_tile<HD, 256>(Qs, Qp, a.q_ss, q0, 32, a.S);
-            load_tile<HD, 256>(dOs, dOp, a.q_ss, q0, 32, a.S);
-            if (threadIdx.x < 32) {
-                const int qq = q0 + threadIdx.x;
-                lse_s[threadIdx.x] = qq < a.S ? a.LSE[stat0 + qq] * kLog2e : INFINITY;
-                d_s[threadIdx.x] = qq < a.S ? a.D[stat0 + qq] : 0.f;
+    bf16_t* Qs = tiles[wave][0];
+    bf16_t* dOs = tiles[wave][1];
+    float* st = stats[wave];
+    float* red = reinterpret_cast<float*>(tiles[wave][0]);
+    const bf16_t* Qg = static_cast<const bf16_t*>(a.Q) + b * a.q_sb;
+    const bf16_t* dOg = static_cast<const bf16_t*>(a.dO) + b * a.q_sb;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    for (int pass = 0; pass < 2; pass++) {
+        const int kb = pass == 0 ? (int)blockIdx.x : n_qt - 1 - (int)blockIdx.x;
+        if (pass == 1 && kb <= (int)blockIdx.x) break;  // odd block count: the middle block has no mirror
+        const int k0 = kb * 32, key = k0 + c;
+        const bool valid_k = key < a.S;
+        const long long koff = b * a.k_sb + kvh * a.k_sh + (long long)key * a.k_ss;
+        bf16x8 kf[KSTEPS], vf[KSTEPS];
+#pragma unroll
+        for (int st_ = 0; st_ < KSTEPS; st_++) {
+            const int d = st_ * 16 + 8 * g;
+            kf[st_] = valid_k ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.K) + koff + d) : zero8;
+            vf[st_] = valid_k ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.V) + koff + d) : zero8;
+        }
+        f32x16 dk[DT], dv[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) { dk[dt][v] = 0.f; dv[dt][v] = 0.f; }
+
+        const int qt_start = a.causal ? kb : 0;  // the diagonal tile is the first one that sees these keys
+        const int per_head = n_qt - qt_start;
+        const int n_items = a.G * per_head;      // (query head of the group, query tile), head-major
+
+        bf16x8 rq[CH], rdo[CH];
+        float rstat = 0.f;
+        auto fetch = [&](int item) {
+            const int hq = kvh * a.G + item / per_head, q0 = (qt_start + item % per_head) * 32;
+            const bf16_t* qp = Qg + hq * a.q_sh;
+            const bf16_t* dop = dOg + hq * a.q_sh;
+#pragma unroll
+            for (int i = 0; i < CH; i++) {
+                const int ch = i * 64 + lane, row = q0 + ch / CPR;
+                const long long off = (long long)row * a.q_ss + (ch % CPR) * 8;
+                rq[i] = row < a.S ? *reinterpret_cast<const bf16x8*>(qp + off) : zero8;
+                rdo[i] = row < a.S ? *reinterpret_cast<const bf16x8*>(dop + off) : zero8;
             }
-            __syncthreads();
-            if (k0w >= a.S || (a.causal && q0 + 31 < k0w)) continue;  // wave-uniform
+            const int qq = q0 + c;
+            const long long si = ((long long)b * a.Hq + hq) * a.S + qq;
+            // a query past the end gets LSE = +inf, so its probabilities come out as exactly zero
+            if (g == 0) rstat = qq < a.S ? a.LSE[si] * kLog2e : INFINITY;
+            else rstat = qq < a.S ? a.D[si] : 0.f;
+        };
+        if (wave < n_items) fetch(wave);
+        for (int item = wave; item < n_items; item += 4) {
+            // The tile is private to the wave and LDS serves a wave's requests in order, so the stores
+            // below cannot overtake the previous item's reads; the fences keep the compiler from
+            // moving accesses of other lanes' data across them.
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+            for (int i = 0; i < CH; i++) {
+                const int ch = i * 64 + lane;
+                *reinterpret_cast<bf16x8*>(Qs + (ch / CPR) * PITCH + (ch % CPR) * 8) = rq[i];
+                *reinterpret_cast<bf16x8*>(dOs + (ch / CPR) * PITCH + (ch % CPR) * 8) = rdo[i];
+            }
+            st[lane] = rstat;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (item + 4 < n_items) fetch(item + 4);
+
             f32x16 s, dp;
 #pragma unroll
             for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
 #pragma unroll
-            for (int st = 0; st < KSTEPS; st++) {
-                const bf16x8 qa = *reinterpret_cast<const bf16x8*>(Qs + c * PITCH + st * 16 + 8 * g);
-                const bf16x8 da = *reinterpret_cast<const bf16x8*>(dOs + c * PITCH + st * 16 + 8 * g);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[st], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[st], dp, 0, 0, 0);
+            for (int st_ = 0; st_ < KSTEPS; st_++) {
+                const bf16x8 qa = *reinterpret_cast<const bf16x8*>(Qs + c * PITCH + st_ * 16 + 8 * g);
+                const bf16x8 da = *reinterpret_cast<const bf16x8*>(dOs + c * PITCH + st_ * 16 + 8 * g);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[st_], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[st_], dp, 0, 0, 0);
             }
             bf16x8 pf[2], dsf[2];
+            // only the diagonal tile is cut by the causal mask; rows and keys past the end need no
+            // mask (zero probability through LSE = +inf, respectively never stored)
+            const bool diag = a.causal && (item % per_head) == 0;
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int qi = acc_row(v, g), qq = q0 + qi;
-                const bool masked = (a.causal && key > qq) || qq >= a.S || !valid_k;
-                const float p = masked ? 0.f : exp2f(s[v] * a.scale_log2e - lse_s[qi]);
-                pf[v >> 3][v & 7] = (bf16_t)p;
-                dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - d_s[qi]));
+            for (int vg = 0; vg < 4; vg++) {
+                const float4 l4 = *reinterpret_cast<const float4*>(st + 8 * vg + 4 * g);
+                const float4 d4 = *reinterpret_cast<const float4*>(st + 32 + 8 * vg + 4 * g);
+                const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dvv[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int v = vg * 4 + e;
+                    float p = fast_exp2(fmaf(s[v], a.scale_log2e, -lv[e]));
+                    if (diag && c > 8 * vg + 4 * g + e) p = 0.f;  // key k0+c is after query q0+row
+                    pf[v >> 3][v & 7] = (bf16_t)p;
+                    dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - dvv[e]));
+                }
             }
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
@@ -352,19 +443,41 @@ __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
                     dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[t], qtr, dk[dt], 0, 0, 0);
                 }
         }
-    }
-    bf16_t* dKp = static_cast<bf16_t*>(a.dK) + b * a.k_sb + kvh * a.k_sh;
-    bf16_t* dVp = static_cast<bf16_t*>(a.dV) + b * a.k_sb + kvh * a.k_sh;
+
+        // Sum the four waves' partial results, dK then dV, through the (now idle) tile memory.
+        bf16_t* outs[2] = {static_cast<bf16_t*>(a.dK) + b * a.k_sb + kvh * a.k_sh,
+                           static_cast<bf16_t*>(a.dV) + b * a.k_sb + kvh * a.k_sh};
 #pragma unroll
-    for (int dt = 0; dt < DT; dt++)
+        for (int which = 0; which < 2; which++) {
+            __syncthreads();  // every wave is done with its tile / with the previous reduction
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int kr = k0w + acc_row(v, g);
-            if (kr < a.S) {
-                dKp[(long long)kr * a.k_ss + dt * 32 + c] = (bf16_t)(dk[dt][v] * a.scale);
-                dVp[(long long)kr * a.k_ss + dt * 32 + c] = (bf16_t)dv[dt][v];
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    red[acc_row(v, g) * HD + dt * 32 + c] = which == 0 ? dk[dt][v] * a.scale : dv[dt][v];
+            __syncthreads();
+            // 32 x HD outputs, 8 consecutive ones per thread step
+            for (int e0 = threadIdx.x * 8; e0 < 32 * HD; e0 += 256 * 8) {
+                float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const float* src = reinterpret_cast<const float*>(tiles[w][0]) + e0;
+                    const float4 x0 = *reinterpret_cast<const float4*>(src);
+                    const float4 x1 = *reinterpret_cast<const float4*>(src + 4);
+                    acc8[0] += x0.x; acc8[1] += x0.y; acc8[2] += x0.z; acc8[3] += x0.w;
+                    acc8[4] += x1.x; acc8[5] += x1.y; acc8[6] += x1.z; acc8[7] += x1.w;
+                }
+                const int kr = k0 + e0 / HD;
+                if (kr < a.S) {
+                    bf16x8 o8;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) o8[e] = (bf16_t)acc8[e];
+                    *reinterpret_cast<bf16x8*>(outs[which] + (long long)kr * a.k_ss + e0 % HD) = o8;
+                }
             }
         }
+        __syncthreads();  // the reduction's reads are over before the next pass refills the tiles
+    }
 }
 
 // ---- f32 path: one wave per row, any head_dim ---------------------------------------------------
@@ -545,7 +658,8 @@ void launch_bwd(eisen_ctx* ctx, const AttnArgs& a) {
         else if (gw == 2) fa_bwd_dq_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
         else fa_bwd_dq_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
     }
-    dim3 grid2((unsigned)eisen_ceil_div(a.S, 128), (unsigned)a.Hkv, (unsigned)a.B);
+    const int n_kb = eisen_ceil_div(a.S, 32);  // 32-key blocks, handled in heavy/light pairs
+    dim3 grid2((unsigned)((n_kb + 1) / 2), (unsigned)a.Hkv, (unsigned)a.B);
     {   // dP, dV, dK: three of the four backward GEMMs
         EisenProfScope prof(ctx, "attn_bwd_dkv_bf16", 3.0 * attn_pair_flops(a), true);
         fa_bwd_dkv_kernel<HD><<<grid2, 256, 0, ctx->stream>>>(a);
