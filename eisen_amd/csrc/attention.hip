@@ -36,6 +36,7 @@ struct AttnArgs {
     long long k_sb, k_ss, k_sh;
     float scale, scale_log2e;
     int causal;
+    int paired;  // query-stationary kernels: a block runs a long query block and its short mirror image
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -63,6 +64,14 @@ __device__ __forceinline__ bf16x8 lds_tr_operand(const bf16_t* tile, int pitch, 
     const int g = lane >> 5, L = lane & 15, half = (lane >> 4) & 1;
     const bf16_t* p = tile + (row0 + 16 * t + 4 * g + (L >> 2)) * pitch + col0 + 16 * half + 4 * (L & 3);
     return concat4(lds_read_tr(p), lds_read_tr(p + 8 * pitch));
+}
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  This
+// renumbering gives XCD j the contiguous id range [j*total/8, (j+1)*total/8), in dispatch order, so
+// workgroups that are neighbours in the renumbered order (and share operands) also share an L2.
+__device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
+    const int per = total / 8;
+    return linear < per * 8 ? (linear % 8) * per + linear / 8 : linear;
 }
 
 // 2^x as the bare hardware instruction: results below 2^-126 flush to zero, which is what a softmax
@@ -95,118 +104,161 @@ struct TilePrefetch {
 };
 
 // ---- forward -------------------------------------------------------------------------------
+// Grid of the two query-stationary kernels: one block per (pair of query blocks, GW query heads of a
+// KV head, batch), pair index fastest.  A block runs query block `pair` and then its mirror image
+// n-1-pair, so that under the causal mask every block sees the same number of key tiles; blocks that
+// read the same K/V (one batch and KV head) are kept on one XCD.
+struct QBlock {
+    int pair, n_qblk, kvh, hgrp, b;
+};
+template <int GW>
+__device__ __forceinline__ QBlock decode_qblock(const AttnArgs& a) {
+    constexpr int QS = 4 / GW;
+    QBlock r;
+    r.n_qblk = (a.S + 32 * QS - 1) / (32 * QS);
+    const int n_pairs = a.paired ? (r.n_qblk + 1) / 2 : r.n_qblk, groups = a.G / GW;
+    const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    r.pair = bid % n_pairs;
+    const int y = (bid / n_pairs) % (a.Hkv * groups);
+    r.kvh = y / groups;
+    r.hgrp = y % groups;
+    r.b = bid / (n_pairs * a.Hkv * groups);
+    return r;
+}
+
 template <int HD, int GW>
 __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
     constexpr int QS = 4 / GW, BKV = 64, PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
     __shared__ __attribute__((aligned(16))) bf16_t Ksb[2][BKV * PITCH];
     __shared__ __attribute__((aligned(16))) bf16_t Vsb[2][BKV * PITCH];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, c = lane & 31;
+    const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hsub = wave % GW, qsub = wave / GW;
-    const int qblk = gridDim.x - 1 - blockIdx.x;  // long rows first
-    const int groups = a.G / GW;
-    const int kvh = blockIdx.y / groups, hq = kvh * a.G + (blockIdx.y % groups) * GW + hsub, b = blockIdx.z;
-    const int q0 = (qblk * QS + qsub) * 32, q = q0 + c;
-    const bool valid_q = q < a.S;
+    const QBlock blk = decode_qblock<GW>(a);
+    const int kvh = blk.kvh, hq = kvh * a.G + blk.hgrp * GW + hsub, b = blk.b;
     const bf16_t* Qp = static_cast<const bf16_t*>(a.Q) + b * a.q_sb + hq * a.q_sh;
     const bf16_t* Kp = static_cast<const bf16_t*>(a.K) + b * a.k_sb + kvh * a.k_sh;
     const bf16_t* Vp = static_cast<const bf16_t*>(a.V) + b * a.k_sb + kvh * a.k_sh;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    bf16x8 qf[KSTEPS];
+    for (int pass = 0; pass < 2; pass++) {
+        const int qblk = pass == 0 ? blk.n_qblk - 1 - blk.pair : blk.pair;  // the long one first
+        if (pass == 1 && (!a.paired || qblk >= blk.n_qblk - 1 - blk.pair)) break;  // the middle block has no mirror
+        if (pass == 1) __syncthreads();                                     // LDS tiles of the first pass are done with
+        const int q0 = (qblk * QS + qsub) * 32, q = q0 + c;
+        const bool valid_q = q < a.S;
+        bf16x8 qf[KSTEPS];
 #pragma unroll
-    for (int st = 0; st < KSTEPS; st++)
-        qf[st] = valid_q ? *reinterpret_cast<const bf16x8*>(Qp + (long long)q * a.q_ss + st * 16 + 8 * g) : zero8;
-    f32x16 o[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) o[dt][v] = 0.f;
-    float m = -INFINITY, l = 0.f;
-
-    const int block_qmax = min(a.S - 1, (qblk * QS + QS - 1) * 32 + 31);
-    const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
-    const int my_qmax = q0 < a.S ? q0 + 31 : -1;
-
-    TilePrefetch<HD, BKV, 256> pk, pv;
-    pk.fetch(Kp, a.k_ss, 0, a.S);
-    pv.fetch(Vp, a.k_ss, 0, a.S);
-    for (int kt = 0; kt < n_kt; kt++) {
-        const bf16_t* Ks = Ksb[kt & 1];
-        const bf16_t* Vs = Vsb[kt & 1];
-        pk.commit(Ksb[kt & 1]);
-        pv.commit(Vsb[kt & 1]);
-        __syncthreads();  // one barrier per tile: the other buffer is only rewritten after the next barrier
-        if (kt + 1 < n_kt) {
-            pk.fetch(Kp, a.k_ss, (kt + 1) * BKV, a.S);
-            pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
-        }
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++) {
-            const int k0 = kt * BKV + sub * 32;
-            if (k0 >= a.S || my_qmax < 0 || (a.causal && k0 > my_qmax)) continue;  // wave-uniform
-            f32x16 s;
-#pragma unroll
-            for (int v = 0; v < 16; v++) s[v] = 0.f;
-#pragma unroll
-            for (int st = 0; st < KSTEPS; st++) {
-                const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
-            }
-            // only tiles that touch the diagonal or the end of the sequence need the mask
-            const bool need_mask = (a.causal && k0 + 31 > q0) || k0 + 32 > a.S;
-            float mx = -INFINITY;  // of the raw scores; the (positive) scale is folded into the exponent's fma
-            if (need_mask) {
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int key = k0 + acc_row(v, g);
-                    if ((a.causal && key > q) || key >= a.S) s[v] = -INFINITY;
-                }
-            }
-#pragma unroll
-            for (int v = 0; v < 16; v++) mx = fmaxf(mx, s[v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2e;
-            const float m_new = fmaxf(m, mx);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = fast_exp2(m - m_use);
-            float rowsum = 0.f;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                s[v] = fast_exp2(fmaf(s[v], a.scale_log2e, -m_use));
-                rowsum += s[v];
-            }
-            rowsum += __shfl_xor(rowsum, 32, 64);
-            l = l * alpha + rowsum;
-            m = m_new;
-            bf16x8 pf[2];
-#pragma unroll
-            for (int t = 0; t < 2; t++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) pf[t][e] = (bf16_t)s[8 * t + e];
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
-#pragma unroll
-                for (int v = 0; v < 16; v++) o[dt][v] *= alpha;
-#pragma unroll
-                for (int t = 0; t < 2; t++) {
-                    const bf16x8 vt = lds_tr_operand(Vs, PITCH, sub * 32, dt * 32, t, lane);
-                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt, pf[t], o[dt], 0, 0, 0);
-                }
-            }
-        }
-    }
-    if (valid_q) {
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
-        bf16_t* Op = static_cast<bf16_t*>(a.Out) + b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+        for (int st = 0; st < KSTEPS; st++)
+            qf[st] = valid_q ? *reinterpret_cast<const bf16x8*>(Qp + (long long)q * a.q_ss + st * 16 + 8 * g) : zero8;
+        f32x16 o[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-            for (int vg = 0; vg < 4; vg++) {
-                bf16x4 w;
-#pragma unroll
-                for (int e = 0; e < 4; e++) w[e] = (bf16_t)(o[dt][vg * 4 + e] * inv);
-                *reinterpret_cast<bf16x4*>(Op + dt * 32 + 8 * vg + 4 * g) = w;
+            for (int v = 0; v < 16; v++) o[dt][v] = 0.f;
+        // m is the reference point of the exponentials, not always the running maximum: it is only
+        // moved when a row's maximum has grown by more than 2^8 since, which keeps every exponential
+        // far inside the f32 and bf16 ranges and makes the rescaling of O rare.
+        float m = -INFINITY, l = 0.f;
+
+        const int block_qmax = min(a.S - 1, (qblk * QS + QS - 1) * 32 + 31);
+        const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
+        const int my_qmax = q0 < a.S ? q0 + 31 : -1;
+
+        TilePrefetch<HD, BKV, 256> pk, pv;
+        pk.fetch(Kp, a.k_ss, 0, a.S);
+        pv.fetch(Vp, a.k_ss, 0, a.S);
+        for (int kt = 0; kt < n_kt; kt++) {
+            const bf16_t* Ks = Ksb[kt & 1];
+            const bf16_t* Vs = Vsb[kt & 1];
+            pk.commit(Ksb[kt & 1]);
+            pv.commit(Vsb[kt & 1]);
+            __syncthreads();  // one barrier per tile: the other buffer is only rewritten after the next barrier
+            if (kt + 1 < n_kt) {
+                pk.fetch(Kp, a.k_ss, (kt + 1) * BKV, a.S);
+                pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
             }
-        if (g == 0) a.LSE[((long long)b * a.Hq + hq) * a.S + q] = (m + log2f(l)) * kLn2;
+            const int k0 = kt * BKV;
+            if (my_qmax < 0 || (a.causal && k0 > my_qmax)) continue;              // wave-uniform
+            const bool two = k0 + 32 < a.S && !(a.causal && k0 + 32 > my_qmax);  // the second 32 keys are visible
+            f32x16 s[2];
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) s[sub][v] = sub == 0 ? 0.f : (two ? 0.f : -INFINITY);
+                if (sub == 0 || two) {
+#pragma unroll
+                    for (int st = 0; st < KSTEPS; st++) {
+                        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
+                        s[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s[sub], 0, 0, 0);
+                    }
+                }
+            }
+            // only tiles that touch the diagonal or the end of the sequence need the mask
+            if ((a.causal && k0 + 63 > q0) || k0 + 64 > a.S) {
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const int key = k0 + sub * 32 + acc_row(v, g);
+                        if ((a.causal && key > q) || key >= a.S) s[sub][v] = -INFINITY;
+                    }
+            }
+            float mx = -INFINITY;  // of the raw scores; the (positive) scale is folded into the exponent's fma
+#pragma unroll
+            for (int v = 0; v < 16; v++) mx = fmaxf(mx, fmaxf(s[0][v], s[1][v]));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2e;
+            const bool grow = mx > m + 8.0f;
+            if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+                const float alpha = grow ? fast_exp2(m - mx) : 1.0f;
+                m = grow ? mx : m;
+                l *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) o[dt][v] *= alpha;
+            }
+            const float m_use = m == -INFINITY ? 0.f : m;
+            float rowsum = 0.f;
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    s[sub][v] = fast_exp2(fmaf(s[sub][v], a.scale_log2e, -m_use));
+                    rowsum += s[sub][v];
+                }
+            l += rowsum + __shfl_xor(rowsum, 32, 64);
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+                if (sub == 1 && !two) break;
+                bf16x8 pf[2];
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) pf[t][e] = (bf16_t)s[sub][8 * t + e];
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const bf16x8 vt = lds_tr_operand(Vs, PITCH, sub * 32, dt * 32, t, lane);
+                        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt, pf[t], o[dt], 0, 0, 0);
+                    }
+            }
+        }
+        if (valid_q) {
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            bf16_t* Op = static_cast<bf16_t*>(a.Out) + b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int vg = 0; vg < 4; vg++) {
+                    bf16x4 w;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) w[e] = (bf16_t)(o[dt][vg * 4 + e] * inv);
+                    *reinterpret_cast<bf16x4*>(Op + dt * 32 + 8 * vg + 4 * g) = w;
+                }
+            if (g == 0) a.LSE[((long long)b * a.Hq + hq) * a.S + q] = (m + log2f(l)) * kLn2;
+        }
     }
 }
 
@@ -216,108 +268,107 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
     constexpr int QS = 4 / GW, BKV = 64, PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
     __shared__ __attribute__((aligned(16))) bf16_t Ksb[2][BKV * PITCH];
     __shared__ __attribute__((aligned(16))) bf16_t Vsb[2][BKV * PITCH];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 5, c = lane & 31;
+    const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hsub = wave % GW, qsub = wave / GW;
-    const int qblk = gridDim.x - 1 - blockIdx.x;
-    const int groups = a.G / GW;
-    const int kvh = blockIdx.y / groups, hq = kvh * a.G + (blockIdx.y % groups) * GW + hsub, b = blockIdx.z;
-    const int q0 = (qblk * QS + qsub) * 32, q = q0 + c;
-    const bool valid_q = q < a.S;
-    const long long qoff = b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+    const QBlock blk = decode_qblock<GW>(a);
+    const int kvh = blk.kvh, hq = kvh * a.G + blk.hgrp * GW + hsub, b = blk.b;
     const bf16_t* Kp = static_cast<const bf16_t*>(a.K) + b * a.k_sb + kvh * a.k_sh;
     const bf16_t* Vp = static_cast<const bf16_t*>(a.V) + b * a.k_sb + kvh * a.k_sh;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    bf16x8 qf[KSTEPS], dof[KSTEPS];
-    float dpart = 0.f;
-#pragma unroll
-    for (int st = 0; st < KSTEPS; st++) {
-        const int d = st * 16 + 8 * g;
-        qf[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.Q) + qoff + d) : zero8;
-        dof[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.dO) + qoff + d) : zero8;
-        const bf16x8 of = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.O) + qoff + d) : zero8;
-#pragma unroll
-        for (int e = 0; e < 8; e++) dpart += (float)dof[st][e] * (float)of[e];
-    }
-    const float Dq = dpart + __shfl_xor(dpart, 32, 64);
-    const long long stat = ((long long)b * a.Hq + hq) * a.S + q;
-    if (valid_q && g == 0) a.D[stat] = Dq;
-    const float lse2 = valid_q ? a.LSE[stat] * kLog2e : INFINITY;
+    for (int pass = 0; pass < 2; pass++) {
+        const int qblk = pass == 0 ? blk.n_qblk - 1 - blk.pair : blk.pair;
+        if (pass == 1 && (!a.paired || qblk >= blk.n_qblk - 1 - blk.pair)) break;
+        if (pass == 1) __syncthreads();
+        const int q0 = (qblk * QS + qsub) * 32, q = q0 + c;
+        const bool valid_q = q < a.S;
+        const long long qoff = b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
 
-    f32x16 dq[DT];
+        bf16x8 qf[KSTEPS], dof[KSTEPS];
+        float dpart = 0.f;
 #pragma unroll
-    for (int dt = 0; dt < DT; dt++)
+        for (int st = 0; st < KSTEPS; st++) {
+            const int d = st * 16 + 8 * g;
+            qf[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.Q) + qoff + d) : zero8;
+            dof[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.dO) + qoff + d) : zero8;
+            const bf16x8 of = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.O) + qoff + d) : zero8;
 #pragma unroll
-        for (int v = 0; v < 16; v++) dq[dt][v] = 0.f;
-
-    const int block_qmax = min(a.S - 1, (qblk * QS + QS - 1) * 32 + 31);
-    const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
-    const int my_qmax = q0 < a.S ? q0 + 31 : -1;
-
-    TilePrefetch<HD, BKV, 256> pk, pv;
-    pk.fetch(Kp, a.k_ss, 0, a.S);
-    pv.fetch(Vp, a.k_ss, 0, a.S);
-    for (int kt = 0; kt < n_kt; kt++) {
-        const bf16_t* Ks = Ksb[kt & 1];
-        const bf16_t* Vs = Vsb[kt & 1];
-        pk.commit(Ksb[kt & 1]);
-        pv.commit(Vsb[kt & 1]);
-        __syncthreads();
-        if (kt + 1 < n_kt) {
-            pk.fetch(Kp, a.k_ss, (kt + 1) * BKV, a.S);
-            pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
+            for (int e = 0; e < 8; e++) dpart += (float)dof[st][e] * (float)of[e];
         }
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++) {
-            const int k0 = kt * BKV + sub * 32;
-            if (k0 >= a.S || my_qmax < 0 || (a.causal && k0 > my_qmax)) continue;
-            f32x16 s, dp;
-#pragma unroll
-            for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
-#pragma unroll
-            for (int st = 0; st < KSTEPS; st++) {
-                const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
-                const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[st], dp, 0, 0, 0);
-            }
-            bf16x8 dsf[2];
-            const bool need_mask = (a.causal && k0 + 31 > q0) || k0 + 32 > a.S;
-            if (need_mask) {
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int key = k0 + acc_row(v, g);
-                    const bool masked = (a.causal && key > q) || key >= a.S;
-                    const float p = masked ? 0.f : fast_exp2(s[v] * a.scale_log2e - lse2);
-                    dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - Dq));
-                }
-            } else {
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const float p = fast_exp2(s[v] * a.scale_log2e - lse2);
-                    dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - Dq));
-                }
-            }
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                for (int t = 0; t < 2; t++) {
-                    const bf16x8 ktr = lds_tr_operand(Ks, PITCH, sub * 32, dt * 32, t, lane);
-                    dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsf[t], dq[dt], 0, 0, 0);
-                }
-        }
-    }
-    if (valid_q) {
-        bf16_t* dQp = static_cast<bf16_t*>(a.dQ) + qoff;
+        const float Dq = dpart + __shfl_xor(dpart, 32, 64);
+        const long long stat = ((long long)b * a.Hq + hq) * a.S + q;
+        if (valid_q && g == 0) a.D[stat] = Dq;
+        const float lse2 = valid_q ? a.LSE[stat] * kLog2e : INFINITY;
+
+        f32x16 dq[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-            for (int vg = 0; vg < 4; vg++) {
-                bf16x4 w;
-#pragma unroll
-                for (int e = 0; e < 4; e++) w[e] = (bf16_t)(dq[dt][vg * 4 + e] * a.scale);
-                *reinterpret_cast<bf16x4*>(dQp + dt * 32 + 8 * vg + 4 * g) = w;
+            for (int v = 0; v < 16; v++) dq[dt][v] = 0.f;
+
+        const int block_qmax = min(a.S - 1, (qblk * QS + QS - 1) * 32 + 31);
+        const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
+        const int my_qmax = q0 < a.S ? q0 + 31 : -1;
+
+        TilePrefetch<HD, BKV, 256> pk, pv;
+        pk.fetch(Kp, a.k_ss, 0, a.S);
+        pv.fetch(Vp, a.k_ss, 0, a.S);
+        for (int kt = 0; kt < n_kt; kt++) {
+            const bf16_t* Ks = Ksb[kt & 1];
+            const bf16_t* Vs = Vsb[kt & 1];
+            pk.commit(Ksb[kt & 1]);
+            pv.commit(Vsb[kt & 1]);
+            __syncthreads();
+            if (kt + 1 < n_kt) {
+                pk.fetch(Kp, a.k_ss, (kt + 1) * BKV, a.S);
+                pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
             }
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+                const int k0 = kt * BKV + sub * 32;
+                if (k0 >= a.S || my_qmax < 0 || (a.causal && k0 > my_qmax)) continue;
+                f32x16 s, dp;
+#pragma unroll
+                for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
+#pragma unroll
+                for (int st = 0; st < KSTEPS; st++) {
+                    const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
+                    const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
+                    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[st], dp, 0, 0, 0);
+                }
+                bf16x8 dsf[2];
+                // a query past the end has LSE = +inf and a key past the end a zero K row, so only
+                // the causal diagonal needs a mask
+                const bool diag = a.causal && k0 + 31 > q0;
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    float p = fast_exp2(fmaf(s[v], a.scale_log2e, -lse2));
+                    if (diag && k0 + acc_row(v, g) > q) p = 0.f;
+                    dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - Dq));
+                }
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const bf16x8 ktr = lds_tr_operand(Ks, PITCH, sub * 32, dt * 32, t, lane);
+                        dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsf[t], dq[dt], 0, 0, 0);
+                    }
+            }
+        }
+        if (valid_q) {
+            bf16_t* dQp = static_cast<bf16_t*>(a.dQ) + qoff;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int vg = 0; vg < 4; vg++) {
+                    bf16x4 w;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) w[e] = (bf16_t)(dq[dt][vg * 4 + e] * a.scale);
+                    *reinterpret_cast<bf16x4*>(dQp + dt * 32 + 8 * vg + 4 * g) = w;
+                }
+        }
     }
 }
 
@@ -335,8 +386,12 @@ __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
     static_assert(2 * TILE * sizeof(bf16_t) >= 32 * HD * sizeof(float), "reduction scratch reuses the tiles");
     const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int kvh = blockIdx.y, b = blockIdx.z;
     const int n_qt = (a.S + 31) / 32;
+    // grid: x = key-block pair, fastest; then KV head, then batch.  Blocks of one (batch, KV head) read
+    // the same Q/dO tiles, so they are kept on one XCD.
+    const int n_pairs = (n_qt + 1) / 2;
+    const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int pair = bid % n_pairs, kvh = (bid / n_pairs) % a.Hkv, b = bid / (n_pairs * a.Hkv);
     bf16_t* Qs = tiles[wave][0];
     bf16_t* dOs = tiles[wave][1];
     float* st = stats[wave];
@@ -346,8 +401,8 @@ __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
     for (int pass = 0; pass < 2; pass++) {
-        const int kb = pass == 0 ? (int)blockIdx.x : n_qt - 1 - (int)blockIdx.x;
-        if (pass == 1 && kb <= (int)blockIdx.x) break;  // odd block count: the middle block has no mirror
+        const int kb = pass == 0 ? pair : n_qt - 1 - pair;
+        if (pass == 1 && kb <= pair) break;  // odd block count: the middle block has no mirror
         const int k0 = kb * 32, key = k0 + c;
         const bool valid_k = key < a.S;
         const long long koff = b * a.k_sb + kvh * a.k_sh + (long long)key * a.k_ss;
@@ -638,20 +693,28 @@ static double attn_pair_flops(const AttnArgs& a) {
 }
 
 template <int HD>
-void launch_fwd(eisen_ctx* ctx, const AttnArgs& a) {
+void launch_fwd(eisen_ctx* ctx, AttnArgs a) {
     EisenProfScope prof(ctx, "attn_fwd_bf16", 2.0 * attn_pair_flops(a), true);
     const int gw = a.G % 4 == 0 ? 4 : (a.G % 2 == 0 ? 2 : 1);
     const int qs = 4 / gw;
-    dim3 grid((unsigned)eisen_ceil_div(a.S, 32 * qs), (unsigned)(a.Hkv * (a.G / gw)), (unsigned)a.B);
+    const int n_qblk = eisen_ceil_div(a.S, 32 * qs), per_q = a.Hkv * (a.G / gw) * a.B;
+    // pairing long and short query blocks balances the causal mask; it is only worth halving the
+    // number of blocks when at least two per CU remain
+    a.paired = a.causal && (long long)n_qblk * per_q >= 1024;
+    dim3 grid((unsigned)((a.paired ? (n_qblk + 1) / 2 : n_qblk) * per_q));
     if (gw == 4) fa_fwd_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
     else if (gw == 2) fa_fwd_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
     else fa_fwd_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
 }
 template <int HD>
-void launch_bwd(eisen_ctx* ctx, const AttnArgs& a) {
+void launch_bwd(eisen_ctx* ctx, AttnArgs a) {
     const int gw = a.G % 4 == 0 ? 4 : (a.G % 2 == 0 ? 2 : 1);
     const int qs = 4 / gw;
-    dim3 grid((unsigned)eisen_ceil_div(a.S, 32 * qs), (unsigned)(a.Hkv * (a.G / gw)), (unsigned)a.B);
+    const int n_qblk = eisen_ceil_div(a.S, 32 * qs), per_q = a.Hkv * (a.G / gw) * a.B;
+    // pairing long and short query blocks balances the causal mask; it is only worth halving the
+    // number of blocks when at least two per CU remain
+    a.paired = a.causal && (long long)n_qblk * per_q >= 1024;
+    dim3 grid((unsigned)((a.paired ? (n_qblk + 1) / 2 : n_qblk) * per_q));
     {   // dQ = scale dS K: one of the four backward GEMMs (S and dP are recomputed here as well)
         EisenProfScope prof(ctx, "attn_bwd_dq_bf16", 1.0 * attn_pair_flops(a), true);
         if (gw == 4) fa_bwd_dq_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
@@ -659,7 +722,7 @@ void launch_bwd(eisen_ctx* ctx, const AttnArgs& a) {
         else fa_bwd_dq_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
     }
     const int n_kb = eisen_ceil_div(a.S, 32);  // 32-key blocks, handled in heavy/light pairs
-    dim3 grid2((unsigned)((n_kb + 1) / 2), (unsigned)a.Hkv, (unsigned)a.B);
+    dim3 grid2((unsigned)((n_kb + 1) / 2 * a.Hkv * a.B));
     {   // dP, dV, dK: three of the four backward GEMMs
         EisenProfScope prof(ctx, "attn_bwd_dkv_bf16", 3.0 * attn_pair_flops(a), true);
         fa_bwd_dkv_kernel<HD><<<grid2, 256, 0, ctx->stream>>>(a);
