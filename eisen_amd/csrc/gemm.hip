@@ -14,12 +14,22 @@
 // all stream their operands through LDS as plain 16-byte copies.
 //
 // f32 path and odd shapes: a plain LDS-tiled FMA kernel (64x64 tile, 4x4 per thread).
+#include <utility>
+
 #include "device_utils.cuh"
 #include "runtime.h"
 
 namespace {
 
-constexpr int kGemmThreads = 256;
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a constant expression
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 struct GemmArgs {
     const void* A;
@@ -41,15 +51,16 @@ struct GemmArgs {
 // so no operand is ever transposed element by element.
 typedef bf16x4 __attribute__((address_space(3))) * lds_bf16x4_ptr;
 
-template <int ROWS, bool KC, int BK>
+template <int ROWS, bool KC, int BK, int THREADS>
 struct OperandTile {
-    static constexpr int PITCH = KC ? BK + 8 : ROWS + 16;
+    static constexpr int PITCH = KC ? BK + 8 : ROWS + 32;  // ROWS + 32: the transpose reads of a half-wave hit 64 distinct banks
     static constexpr int ELEMS = KC ? ROWS * PITCH : BK * PITCH;
-    static constexpr int CHUNKS = ROWS * BK / 8 / kGemmThreads;  // 16-byte chunks per thread per slab
+    static constexpr int CHUNKS = ROWS * BK / 8 / THREADS;
+    static_assert(CHUNKS >= 1 && CHUNKS * THREADS * 8 == ROWS * BK, "slab must split evenly over the threads");  // 16-byte chunks per thread per slab
 
     // global coordinates (row = m or n, k) of chunk `c` of thread `tid`
     static __device__ __forceinline__ void chunk_coords(int c, int tid, int& row, int& k) {
-        const int chunk = c * kGemmThreads + tid;
+        const int chunk = c * THREADS + tid;
         if (KC) {
             row = chunk / (BK / 8);
             k = (chunk % (BK / 8)) * 8;
@@ -58,13 +69,14 @@ struct OperandTile {
             row = (chunk % (ROWS / 8)) * 8;
         }
     }
+    template <bool EDGE>
     static __device__ __forceinline__ bf16x8 load(const bf16_t* base, int ld, int row0, int k0, int row_limit, int k_limit, int c, int tid) {
         int row, k;
         chunk_coords(c, tid, row, k);
         row += row0;
         k += k0;
         const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (row >= row_limit || k >= k_limit) return zero8;
+        if (EDGE && (row >= row_limit || k >= k_limit)) return zero8;
         return *reinterpret_cast<const bf16x8*>(KC ? base + (long long)row * ld + k : base + (long long)k * ld + row);
     }
     static __device__ __forceinline__ void store(bf16_t* tile, bf16x8 v, int c, int tid) {
@@ -87,16 +99,20 @@ struct OperandTile {
     }
 };
 
-template <int BM, int BN, int BK, bool A_KC, bool B_KC, typename TC>
-__global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
-    constexpr int WM = BM / 2, WN = BN / 2;          // wave quadrant
-    constexpr int TM = WM / 32, TN = WN / 32;        // 32x32 tiles per wave
-    using TA = OperandTile<BM, A_KC, BK>;
-    using TB = OperandTile<BN, B_KC, BK>;
+// WGM x WGN waves share a BM x BN tile of C.  EDGE = false is for shapes that are whole multiples
+// of the tile in M, N and K: no bounds checks anywhere.
+template <int BM, int BN, int BK, int WGM, int WGN, bool A_KC, bool B_KC, bool EDGE, typename TC>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
+    constexpr int THREADS = 64 * WGM * WGN;
+    constexpr int WM = BM / WGM, WN = BN / WGN;      // wave tile
+    constexpr int TM = WM / 32, TN = WN / 32;        // 32x32 MFMA tiles per wave
+    using TA = OperandTile<BM, A_KC, BK, THREADS>;
+    using TB = OperandTile<BN, B_KC, BK, THREADS>;
     __shared__ __attribute__((aligned(16))) bf16_t lds[2][TA::ELEMS + TB::ELEMS];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const bf16_t* A = static_cast<const bf16_t*>(g.A) + (long long)blockIdx.z * g.sA;
     const bf16_t* B = static_cast<const bf16_t*>(g.B) + (long long)blockIdx.z * g.sB;
@@ -110,42 +126,65 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-    bf16x8 ra[TA::CHUNKS], rb[TB::CHUNKS];
-    auto load_global = [&](int k0) {
-#pragma unroll
-        for (int c = 0; c < TA::CHUNKS; c++) ra[c] = TA::load(A, g.lda, m0, k0, g.M, g.K, c, tid);
-#pragma unroll
-        for (int c = 0; c < TB::CHUNKS; c++) rb[c] = TB::load(B, g.ldb, n0, k0, g.N, g.K, c, tid);
+    // Slab hand-over.  While slab kt is multiplied out of one LDS buffer, slab kt+1 sits in registers
+    // (its global loads were issued a whole slab earlier).  After the MFMAs of each contraction step a
+    // share of those registers is stored into the other LDS buffer and immediately refilled with
+    // slab kt+2, so LDS writes and global loads are spread between the MFMAs instead of piling up in
+    // front of the barrier.  Slabs past the end are clamped to the last one: they are loaded and
+    // stored like any other and never read.
+    constexpr int KSTEPS = BK / 16, NCH = TA::CHUNKS + TB::CHUNKS;
+    bf16x8 r[NCH];
+    auto load_chunk = [&](int h, int slab) {
+        if (h < TA::CHUNKS) r[h] = TA::template load<EDGE>(A, g.lda, m0, slab * BK, g.M, g.K, h, tid);
+        else r[h] = TB::template load<EDGE>(B, g.ldb, n0, slab * BK, g.N, g.K, h - TA::CHUNKS, tid);
     };
-    auto store_lds = [&](int buf) {
-#pragma unroll
-        for (int c = 0; c < TA::CHUNKS; c++) TA::store(lds[buf], ra[c], c, tid);
-#pragma unroll
-        for (int c = 0; c < TB::CHUNKS; c++) TB::store(lds[buf] + TA::ELEMS, rb[c], c, tid);
+    auto store_chunk = [&](int h, int buf) {
+        if (h < TA::CHUNKS) TA::store(lds[buf], r[h], h, tid);
+        else TB::store(lds[buf] + TA::ELEMS, r[h], h - TA::CHUNKS, tid);
     };
+    constexpr int kReads = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);  // LDS read instructions per step
 
     const int nk = (g.K + BK - 1) / BK;
-    load_global(0);
-    store_lds(0);
+#pragma unroll
+    for (int h = 0; h < NCH; h++) load_chunk(h, 0);
+#pragma unroll
+    for (int h = 0; h < NCH; h++) store_chunk(h, 0);
+#pragma unroll
+    for (int h = 0; h < NCH; h++) load_chunk(h, min(1, nk - 1));
     __syncthreads();
     for (int kt = 0; kt < nk; kt++) {
         const int buf = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * BK);
         const bf16_t* As = lds[buf];
         const bf16_t* Bs = lds[buf] + TA::ELEMS;
-#pragma unroll
-        for (int ks = 0; ks < BK; ks += 16) {
+        const int refill = min(kt + 2, nk - 1);
+        static_for<KSTEPS>([&](auto st_c) {
+            constexpr int st = decltype(st_c)::value;
             bf16x8 a[TM], b[TN];
 #pragma unroll
-            for (int i = 0; i < TM; i++) a[i] = TA::fragment(As, wm * WM + i * 32, ks, lane);
+            for (int i = 0; i < TM; i++) a[i] = TA::fragment(As, wm * WM + i * 32, st * 16, lane);
 #pragma unroll
-            for (int j = 0; j < TN; j++) b[j] = TB::fragment(Bs, wn * WN + j * 32, ks, lane);
+            for (int j = 0; j < TN; j++) b[j] = TB::fragment(Bs, wn * WN + j * 32, st * 16, lane);
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) store_lds(buf ^ 1);
+            constexpr int h_lo = st * NCH / KSTEPS, h_hi = (st + 1) * NCH / KSTEPS;  // this step's share of the hand-over
+#pragma unroll
+            for (int h = h_lo; h < h_hi; h++) {
+                store_chunk(h, buf ^ 1);
+                load_chunk(h, refill);
+            }
+            if (!EDGE) {  // pin the order: operand reads, then MFMA / LDS write / global load in turn
+                __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
+#pragma unroll
+                for (int h = h_lo; h < h_hi; h++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (h_hi - h_lo), 0);
+            }
+        });
         __syncthreads();
     }
 
@@ -155,11 +194,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int n = n0 + wn * WN + j * 32 + (lane & 31);
-            if (n >= g.N) continue;
+            if (EDGE && n >= g.N) continue;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                if (m < g.M) {
+                if (!EDGE || m < g.M) {
                     TC* dst = C + (long long)m * g.ldc + n;
                     const float val = acc[i][j][v];
                     *dst = from_f32<TC>(g.accumulate ? to_f32(*dst) + val : val);
@@ -222,18 +261,25 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g, int trans
         }
 }
 
-template <int BM, int BN, int BK, typename TC>
-void launch_mfma(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int batch) {
+template <int BM, int BN, int BK, int WGM, int WGN, bool EDGE, typename TC>
+void launch_mfma_t(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int batch) {
     dim3 grid((unsigned)eisen_ceil_div(g.N, BN), (unsigned)eisen_ceil_div(g.M, BM), (unsigned)batch);
-    if (a_kc && b_kc) gemm_mfma_kernel<BM, BN, BK, true, true, TC><<<grid, kGemmThreads, 0, ctx->stream>>>(g);
-    else if (a_kc && !b_kc) gemm_mfma_kernel<BM, BN, BK, true, false, TC><<<grid, kGemmThreads, 0, ctx->stream>>>(g);
-    else if (!a_kc && b_kc) gemm_mfma_kernel<BM, BN, BK, false, true, TC><<<grid, kGemmThreads, 0, ctx->stream>>>(g);
-    else gemm_mfma_kernel<BM, BN, BK, false, false, TC><<<grid, kGemmThreads, 0, ctx->stream>>>(g);
+    constexpr int T = 64 * WGM * WGN;
+    if (a_kc && b_kc) gemm_mfma_kernel<BM, BN, BK, WGM, WGN, true, true, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
+    else if (a_kc && !b_kc) gemm_mfma_kernel<BM, BN, BK, WGM, WGN, true, false, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
+    else if (!a_kc && b_kc) gemm_mfma_kernel<BM, BN, BK, WGM, WGN, false, true, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
+    else gemm_mfma_kernel<BM, BN, BK, WGM, WGN, false, false, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
 }
-template <int BM, int BN, int BK>
+template <int BM, int BN, int BK, int WGM, int WGN>
 void launch_mfma_c(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int batch, int dtype_c) {
-    if (dtype_c == EISEN_BF16) launch_mfma<BM, BN, BK, bf16_t>(ctx, g, a_kc, b_kc, batch);
-    else launch_mfma<BM, BN, BK, float>(ctx, g, a_kc, b_kc, batch);
+    const bool edge = g.M % BM != 0 || g.N % BN != 0 || g.K % BK != 0;
+    if (dtype_c == EISEN_BF16) {
+        if (edge) launch_mfma_t<BM, BN, BK, WGM, WGN, true, bf16_t>(ctx, g, a_kc, b_kc, batch);
+        else launch_mfma_t<BM, BN, BK, WGM, WGN, false, bf16_t>(ctx, g, a_kc, b_kc, batch);
+    } else {
+        if (edge) launch_mfma_t<BM, BN, BK, WGM, WGN, true, float>(ctx, g, a_kc, b_kc, batch);
+        else launch_mfma_t<BM, BN, BK, WGM, WGN, false, float>(ctx, g, a_kc, b_kc, batch);
+    }
 }
 
 template <typename TA, typename TC>
@@ -284,7 +330,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
                           (M >= 128 && N >= 128 && eisen_ceil_div(M, 128) * eisen_ceil_div(N, 128) * batch >= 128);
     snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
              dtype_c == EISEN_BF16 ? "bf16out" : "f32out",
-             !mfma_ok ? "fma64x64" : (big_tile ? ((a_kc && b_kc && K % 64 == 0) ? "128x128x64" : "128x128x32") : "64x64x32"));
+             !mfma_ok ? "fma64x64" : (big_tile ? (K % 64 == 0 ? "128x128x64" : "128x128x32") : "64x64x32"));
     EisenProfScope prof(ctx, pname, 2.0 * (double)M * (double)N * (double)K * (double)batch, true);
     if (mfma_ok) {
         // 128x128 tiles unless the problem is too small to give every CU a tile
@@ -292,10 +338,17 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         // operands read 128 contiguous bytes per tile row with BK = 64 and gain ~30 %; operands that
         // go through the LDS transpose read are faster with the higher occupancy of BK = 32.
         if (big_tile) {
-            if (a_kc && b_kc && K % 64 == 0) launch_mfma_c<128, 128, 64>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-            else launch_mfma_c<128, 128, 32>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            static const int tune = getenv("EISEN_GEMM_TUNE") ? atoi(getenv("EISEN_GEMM_TUNE")) : 0;
+            const bool k64 = K % 64 == 0;
+            if (tune == 1) launch_mfma_c<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            else if (tune == 2) launch_mfma_c<256, 128, 32, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            else if (tune == 3) launch_mfma_c<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            else if (tune == 4) launch_mfma_c<256, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            else if (tune == 5) launch_mfma_c<256, 256, 32, 2, 4>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            else if (k64) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            else launch_mfma_c<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else {
-            launch_mfma_c<64, 64, 32>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            launch_mfma_c<64, 64, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         }
     } else if (dtype_ab == EISEN_F32) {
         launch_generic<float, float>(ctx, g, trans_a, trans_b, (int)batch);
