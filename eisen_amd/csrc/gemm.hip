@@ -39,6 +39,9 @@ struct GemmArgs {
     int lda, ldb, ldc;                 // leading dimensions in elements
     long long sA, sB, sC;              // batch strides in elements
     int accumulate;
+    int split;                         // > 1: K is cut into this many parts; part p > 0 assigns into partial[p-1]
+    int k_part;                        // contraction length of one part (a multiple of the slab)
+    float* partial;                    // [batch][split-1][M][N] f32, summed into C by a second kernel
 };
 
 // ---- MFMA kernel -------------------------------------------------------------------------
@@ -114,9 +117,12 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const bf16_t* A = static_cast<const bf16_t*>(g.A) + (long long)blockIdx.z * g.sA;
-    const bf16_t* B = static_cast<const bf16_t*>(g.B) + (long long)blockIdx.z * g.sB;
-    TC* C = static_cast<TC*>(g.C) + (long long)blockIdx.z * g.sC;
+    const int split = g.split > 1 ? g.split : 1;
+    const int bz = blockIdx.z / split, part = blockIdx.z % split;
+    const int k_lo = part * g.k_part, k_hi = split > 1 ? min(g.K, k_lo + g.k_part) : g.K;
+    const bf16_t* A = static_cast<const bf16_t*>(g.A) + (long long)bz * g.sA;
+    const bf16_t* B = static_cast<const bf16_t*>(g.B) + (long long)bz * g.sB;
+    TC* C = static_cast<TC*>(g.C) + (long long)bz * g.sC;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -135,8 +141,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
     constexpr int KSTEPS = BK / 16, NCH = TA::CHUNKS + TB::CHUNKS;
     bf16x8 r[NCH];
     auto load_chunk = [&](int h, int slab) {
-        if (h < TA::CHUNKS) r[h] = TA::template load<EDGE>(A, g.lda, m0, slab * BK, g.M, g.K, h, tid);
-        else r[h] = TB::template load<EDGE>(B, g.ldb, n0, slab * BK, g.N, g.K, h - TA::CHUNKS, tid);
+        if (h < TA::CHUNKS) r[h] = TA::template load<EDGE>(A, g.lda, m0, k_lo + slab * BK, g.M, k_hi, h, tid);
+        else r[h] = TB::template load<EDGE>(B, g.ldb, n0, k_lo + slab * BK, g.N, k_hi, h - TA::CHUNKS, tid);
     };
     auto store_chunk = [&](int h, int buf) {
         if (h < TA::CHUNKS) TA::store(lds[buf], r[h], h, tid);
@@ -144,7 +150,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
     };
     constexpr int kReads = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);  // LDS read instructions per step
 
-    const int nk = (g.K + BK - 1) / BK;
+    const int nk = (k_hi - k_lo + BK - 1) / BK;
 #pragma unroll
     for (int h = 0; h < NCH; h++) load_chunk(h, 0);
 #pragma unroll
@@ -189,6 +195,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
     }
 
     // epilogue: accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile
+    float* P = part > 0 ? g.partial + ((long long)bz * (split - 1) + (part - 1)) * g.M * g.N : nullptr;
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -199,12 +206,36 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
             for (int v = 0; v < 16; v++) {
                 const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
                 if (!EDGE || m < g.M) {
-                    TC* dst = C + (long long)m * g.ldc + n;
                     const float val = acc[i][j][v];
-                    *dst = from_f32<TC>(g.accumulate ? to_f32(*dst) + val : val);
+                    if (P) {
+                        P[(long long)m * g.N + n] = val;
+                    } else {
+                        TC* dst = C + (long long)m * g.ldc + n;
+                        *dst = from_f32<TC>(g.accumulate ? to_f32(*dst) + val : val);
+                    }
                 }
             }
         }
+}
+
+// C += partial[0] + partial[1] + ... in that order, one thread per 4 consecutive elements of a row.
+template <typename TC>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs g, int batch) {
+    const long long per = (long long)g.M * g.N, quads = per / 4;
+    const long long q = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (q >= quads * batch) return;
+    const long long bz = q / quads, e = (q % quads) * 4;
+    const int m = (int)(e / g.N), n = (int)(e % g.N);
+    TC* dst = static_cast<TC*>(g.C) + bz * g.sC + (long long)m * g.ldc + n;
+    float sum[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sum[i] = to_f32(dst[i]);
+    for (int p = 0; p < g.split - 1; p++) {
+        const float4 x = *reinterpret_cast<const float4*>(g.partial + (bz * (g.split - 1) + p) * per + e);
+        sum[0] += x.x; sum[1] += x.y; sum[2] += x.z; sum[3] += x.w;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) dst[i] = from_f32<TC>(sum[i]);
 }
 
 // ---- generic kernel (f32, or bf16 with shapes the MFMA kernel does not take) ---------------
@@ -263,7 +294,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g, int trans
 
 template <int BM, int BN, int BK, int WGM, int WGN, bool EDGE, typename TC>
 void launch_mfma_t(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int batch) {
-    dim3 grid((unsigned)eisen_ceil_div(g.N, BN), (unsigned)eisen_ceil_div(g.M, BM), (unsigned)batch);
+    dim3 grid((unsigned)eisen_ceil_div(g.N, BN), (unsigned)eisen_ceil_div(g.M, BM), (unsigned)(batch * (g.split > 1 ? g.split : 1)));
     constexpr int T = 64 * WGM * WGN;
     if (a_kc && b_kc) gemm_mfma_kernel<BM, BN, BK, WGM, WGN, true, true, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
     else if (a_kc && !b_kc) gemm_mfma_kernel<BM, BN, BK, WGM, WGN, true, false, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
@@ -272,7 +303,7 @@ void launch_mfma_t(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int 
 }
 template <int BM, int BN, int BK, int WGM, int WGN>
 void launch_mfma_c(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int batch, int dtype_c) {
-    const bool edge = g.M % BM != 0 || g.N % BN != 0 || g.K % BK != 0;
+    const bool edge = g.M % BM != 0 || g.N % BN != 0 || g.K % BK != 0 || (g.split > 1 && g.k_part % BK != 0);
     if (dtype_c == EISEN_BF16) {
         if (edge) launch_mfma_t<BM, BN, BK, WGM, WGN, true, bf16_t>(ctx, g, a_kc, b_kc, batch);
         else launch_mfma_t<BM, BN, BK, WGM, WGN, false, bf16_t>(ctx, g, a_kc, b_kc, batch);
@@ -325,30 +356,50 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     if (b_kc) mfma_ok = mfma_ok && K % 8 == 0; else mfma_ok = mfma_ok && N % 8 == 0;
     // profile key = one kernel instantiation (operand orders, types, tile), so the event timing
     // lines up with a profiler's per-kernel rows
-    char pname[48];
-    const bool big_tile = (eisen_ceil_div(M, 128) * eisen_ceil_div(N, 128) * batch >= 256) ||
-                          (M >= 128 && N >= 128 && eisen_ceil_div(M, 128) * eisen_ceil_div(N, 128) * batch >= 128);
-    snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
-             dtype_c == EISEN_BF16 ? "bf16out" : "f32out",
-             !mfma_ok ? "fma64x64" : (big_tile ? (K % 64 == 0 ? "128x128x64" : "128x128x32") : "64x64x32"));
+    char pname[64];
+    const long long tiles128 = (long long)eisen_ceil_div(M, 128) * eisen_ceil_div(N, 128) * batch;
+    const bool big_tile = tiles128 >= 256 || (M >= 128 && N >= 128 && tiles128 >= 128);
+    // Few output tiles and a long contraction (the dW of a narrow projection): cut K so that every CU
+    // gets a tile.  Part 0 writes C as usual, the other parts go to an f32 scratch that a second kernel
+    // adds to C in a fixed order, so the result does not depend on scheduling.
+    int split = 1;
+    if (mfma_ok && M >= 128 && N >= 128 && tiles128 < 128 && N % 4 == 0) {
+        while (split < 8 && tiles128 * split * 2 <= 256 && K / (split * 2) >= 512 && K % (split * 2 * 64) == 0) split *= 2;
+    }
+    const bool wide = mfma_ok && split == 1 && big_tile && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && (a_kc || b_kc) &&
+                      (long long)(M / 256) * (N / 128) * batch >= 256;
+    const char* tile = !mfma_ok ? "fma64x64" : wide ? "256x128x64" : (big_tile || split > 1) ? (K % 64 == 0 ? "128x128x64" : "128x128x32") : "64x64x32";
+    snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
+             dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : "");
     EisenProfScope prof(ctx, pname, 2.0 * (double)M * (double)N * (double)K * (double)batch, true);
     if (mfma_ok) {
-        // 128x128 tiles unless the problem is too small to give every CU a tile
-        // Slab depth by operand order (measured on MI355X at the config-5 shapes): two k-contiguous
-        // operands read 128 contiguous bytes per tile row with BK = 64 and gain ~30 %; operands that
-        // go through the LDS transpose read are faster with the higher occupancy of BK = 32.
-        if (big_tile) {
-            static const int tune = getenv("EISEN_GEMM_TUNE") ? atoi(getenv("EISEN_GEMM_TUNE")) : 0;
-            const bool k64 = K % 64 == 0;
-            if (tune == 1) launch_mfma_c<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-            else if (tune == 2) launch_mfma_c<256, 128, 32, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-            else if (tune == 3) launch_mfma_c<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-            else if (tune == 4) launch_mfma_c<256, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-            else if (tune == 5) launch_mfma_c<256, 256, 32, 2, 4>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-            else if (k64) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+        if (split > 1) {
+            void* ws = nullptr;
+            int rc = eisen_workspace(ctx, (size_t)batch * (split - 1) * M * N * sizeof(float), &ws);
+            if (rc) return rc;
+            g.split = split;
+            g.k_part = (int)(K / split);
+            g.partial = static_cast<float*>(ws);
+        }
+        // Tile choice (measured on MI355X at the config-5 shapes): 256x128 with 8 waves is ~5 % ahead of
+        // 128x128 with 4 when at least one operand is k-contiguous and the grid still covers every CU; two
+        // transposed operands (dW) need too much LDS for it.  64x64 is for problems with few tiles.
+        if (wide) {
+            launch_mfma_c<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+        } else if (big_tile || split > 1) {
+            // two transposed operands (dW) fill 80 KB of LDS, one workgroup per CU: 8 waves on the tile
+            // instead of 4 keep two waves per SIMD to overlap each other's LDS reads (+7 % measured)
+            if (K % 64 == 0 && !a_kc && !b_kc) launch_mfma_c<128, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            else if (K % 64 == 0) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
             else launch_mfma_c<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else {
             launch_mfma_c<64, 64, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+        }
+        if (split > 1) {
+            const long long quads = (long long)M * N / 4 * batch;
+            const unsigned blocks = (unsigned)((quads + 255) / 256);
+            if (dtype_c == EISEN_BF16) gemm_splitk_reduce_kernel<bf16_t><<<blocks, 256, 0, ctx->stream>>>(g, (int)batch);
+            else gemm_splitk_reduce_kernel<float><<<blocks, 256, 0, ctx->stream>>>(g, (int)batch);
         }
     } else if (dtype_ab == EISEN_F32) {
         launch_generic<float, float>(ctx, g, trans_a, trans_b, (int)batch);
