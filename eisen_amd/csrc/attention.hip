@@ -399,6 +399,10 @@ __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
     const bf16_t* Qg = static_cast<const bf16_t*>(a.Q) + b * a.q_sb;
     const bf16_t* dOg = static_cast<const bf16_t*>(a.dO) + b * a.q_sb;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const float* stat_src = g == 0 ? a.LSE : a.D;  // lanes 0-31 fetch the tile's LSE, lanes 32-63 its D
+    int loff[CH];  // element offset of this lane's chunk i inside a 32-row Q / dO tile
+#pragma unroll
+    for (int i = 0; i < CH; i++) loff[i] = ((i * 64 + lane) / CPR) * (int)a.q_ss + ((i * 64 + lane) % CPR) * 8;
 
     for (int pass = 0; pass < 2; pass++) {
         const int kb = pass == 0 ? pair : n_qt - 1 - pair;
@@ -427,20 +431,27 @@ __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
         float rstat = 0.f;
         auto fetch = [&](int item) {
             const int hq = kvh * a.G + item / per_head, q0 = (qt_start + item % per_head) * 32;
-            const bf16_t* qp = Qg + hq * a.q_sh;
-            const bf16_t* dop = dOg + hq * a.q_sh;
+            // wave-uniform tile origin in scalar registers; the per-lane part of every address is loff / c
+            const bf16_t* qp = Qg + hq * a.q_sh + (long long)q0 * a.q_ss;
+            const bf16_t* dop = dOg + hq * a.q_sh + (long long)q0 * a.q_ss;
+            const long long si = ((long long)b * a.Hq + hq) * a.S + q0;
+            if (q0 + 32 <= a.S) {
 #pragma unroll
-            for (int i = 0; i < CH; i++) {
-                const int ch = i * 64 + lane, row = q0 + ch / CPR;
-                const long long off = (long long)row * a.q_ss + (ch % CPR) * 8;
-                rq[i] = row < a.S ? *reinterpret_cast<const bf16x8*>(qp + off) : zero8;
-                rdo[i] = row < a.S ? *reinterpret_cast<const bf16x8*>(dop + off) : zero8;
+                for (int i = 0; i < CH; i++) {
+                    rq[i] = *reinterpret_cast<const bf16x8*>(qp + loff[i]);
+                    rdo[i] = *reinterpret_cast<const bf16x8*>(dop + loff[i]);
+                }
+                rstat = stat_src[si + c];  // raw: any arithmetic here would wait for the load on the spot
+            } else {
+#pragma unroll
+                for (int i = 0; i < CH; i++) {
+                    const bool ok = q0 + (i * 64 + lane) / CPR < a.S;
+                    rq[i] = ok ? *reinterpret_cast<const bf16x8*>(qp + loff[i]) : zero8;
+                    rdo[i] = ok ? *reinterpret_cast<const bf16x8*>(dop + loff[i]) : zero8;
+                }
+                // a query past the end gets LSE = +inf, so its probabilities come out as exactly zero
+                rstat = q0 + c < a.S ? stat_src[si + c] : (g == 0 ? INFINITY : 0.f);
             }
-            const int qq = q0 + c;
-            const long long si = ((long long)b * a.Hq + hq) * a.S + qq;
-            // a query past the end gets LSE = +inf, so its probabilities come out as exactly zero
-            if (g == 0) rstat = qq < a.S ? a.LSE[si] * kLog2e : INFINITY;
-            else rstat = qq < a.S ? a.D[si] : 0.f;
         };
         if (wave < n_items) fetch(wave);
         for (int item = wave; item < n_items; item += 4) {
@@ -454,7 +465,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
                 *reinterpret_cast<bf16x8*>(Qs + (ch / CPR) * PITCH + (ch % CPR) * 8) = rq[i];
                 *reinterpret_cast<bf16x8*>(dOs + (ch / CPR) * PITCH + (ch % CPR) * 8) = rdo[i];
             }
-            st[lane] = rstat;
+            st[lane] = g == 0 ? rstat * kLog2e : rstat;
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -471,21 +482,31 @@ __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
                 dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[st_], dp, 0, 0, 0);
             }
             bf16x8 pf[2], dsf[2];
-            // only the diagonal tile is cut by the causal mask; rows and keys past the end need no
-            // mask (zero probability through LSE = +inf, respectively never stored)
-            const bool diag = a.causal && (item % per_head) == 0;
+            float p[16];
 #pragma unroll
             for (int vg = 0; vg < 4; vg++) {
                 const float4 l4 = *reinterpret_cast<const float4*>(st + 8 * vg + 4 * g);
+                const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) p[vg * 4 + e] = fast_exp2(fmaf(s[vg * 4 + e], a.scale_log2e, -lv[e]));
+            }
+            // only the diagonal tile is cut by the causal mask; rows and keys past the end need no
+            // mask (zero probability through LSE = +inf, respectively never stored)
+            if (a.causal && (item % per_head) == 0) {
+                asm volatile("" ::: "memory");  // keeps this a branch taken once per head, not 16 selects per tile
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    if (c > acc_row(v, g)) p[v] = 0.f;  // key k0+c is after query q0+row
+            }
+#pragma unroll
+            for (int vg = 0; vg < 4; vg++) {
                 const float4 d4 = *reinterpret_cast<const float4*>(st + 32 + 8 * vg + 4 * g);
-                const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dvv[4] = {d4.x, d4.y, d4.z, d4.w};
+                const float dvv[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int v = vg * 4 + e;
-                    float p = fast_exp2(fmaf(s[v], a.scale_log2e, -lv[e]));
-                    if (diag && c > 8 * vg + 4 * g + e) p = 0.f;  // key k0+c is after query q0+row
-                    pf[v >> 3][v & 7] = (bf16_t)p;
-                    dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - dvv[e]));
+                    pf[v >> 3][v & 7] = (bf16_t)p[v];
+                    dsf[v >> 3][v & 7] = (bf16_t)(p[v] * (dp[v] - dvv[e]));
                 }
             }
 #pragma unroll
