@@ -363,12 +363,17 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     // gets a tile.  Part 0 writes C as usual, the other parts go to an f32 scratch that a second kernel
     // adds to C in a fixed order, so the result does not depend on scheduling.
     int split = 1;
-    if (mfma_ok && M >= 128 && N >= 128 && tiles128 < 128 && N % 4 == 0) {
-        while (split < 8 && tiles128 * split * 2 <= 256 && K / (split * 2) >= 512 && K % (split * 2 * 64) == 0) split *= 2;
+    if (mfma_ok && N % 4 == 0 && K >= 1024) {
+        const bool t128 = M >= 128 && N >= 128;
+        const long long tiles = t128 ? tiles128 : (long long)eisen_ceil_div(M, 64) * eisen_ceil_div(N, 64) * batch;
+        const size_t slab = t128 ? 64 : 32, min_part = t128 ? 512 : 256;
+        if (tiles < 128)
+            while (split < 32 && tiles * split * 2 <= 256 && K / (split * 2) >= min_part && K % (split * 2 * slab) == 0) split *= 2;
     }
+    const bool split128 = split > 1 && M >= 128 && N >= 128;
     const bool wide = mfma_ok && split == 1 && big_tile && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && (a_kc || b_kc) &&
                       (long long)(M / 256) * (N / 128) * batch >= 256;
-    const char* tile = !mfma_ok ? "fma64x64" : wide ? "256x128x64" : (big_tile || split > 1) ? (K % 64 == 0 ? "128x128x64" : "128x128x32") : "64x64x32";
+    const char* tile = !mfma_ok ? "fma64x64" : wide ? "256x128x64" : (big_tile || split128) ? (K % 64 == 0 ? "128x128x64" : "128x128x32") : "64x64x32";
     snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
              dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : "");
     EisenProfScope prof(ctx, pname, 2.0 * (double)M * (double)N * (double)K * (double)batch, true);
@@ -386,7 +391,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         // transposed operands (dW) need too much LDS for it.  64x64 is for problems with few tiles.
         if (wide) {
             launch_mfma_c<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-        } else if (big_tile || split > 1) {
+        } else if (big_tile || split128) {
             // two transposed operands (dW) fill 80 KB of LDS, one workgroup per CU: 8 waves on the tile
             // instead of 4 keep two waves per SIMD to overlap each other's LDS reads (+7 % measured)
             if (K % 64 == 0 && !a_kc && !b_kc) launch_mfma_c<128, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);

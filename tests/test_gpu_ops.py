@@ -502,8 +502,8 @@ def test_gemm_reference_vector(ctx):
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
-# (512, 384, 1024) and (256, 512, 4096) take the split-K path (2 and 8 parts), (4096, 2048, 512) the 256x128 tile
-@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (128, 256, 96), (200, 72, 40), (512, 384, 1024), (256, 512, 4096), (2048, 2048, 512),
+# (512, 384, 1024), (256, 512, 4096) and (256, 64, 8192) take the split-K path (2, 8 and 16 parts), (4096, 2048, 512) the 256x128 tile
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (128, 256, 96), (200, 72, 40), (512, 384, 1024), (256, 512, 4096), (256, 64, 8192), (2048, 2048, 512),
                                    (4096, 2048, 512), (8, 8, 8)])
 def test_gemm_bf16_mfma(ctx, ta, tb, M, N, K):
     _gemm_case(ctx, M, N, K, ta, tb, BF16, BF16, False)
