@@ -69,25 +69,30 @@ __global__ __launch_bounds__(THREADS) void ce_fused_kernel(const T* __restrict__
         return;
     }
 
-    // phase 1: the row comes in once (VPT packets per lane, all loads in flight together) and is
-    // widened to f32 registers; running maximum (and, when asked for, its first index)
-    float x[VPT][N];
+    // phase 1: the row comes in once (VPT packets per lane, all loads in flight together) and stays in
+    // registers in its storage type: half the registers of an f32 copy, so twice the workgroups per CU
+    // keep loads in flight.  Running maximum (and, when asked for, its first index).
+    Pack<T> raw[VPT];
     ArgMax am{-INFINITY, 0x7fffffff};
 #pragma unroll
     for (int v = 0; v < VPT; v++) {
         const int c = (v * THREADS + threadIdx.x) * N;
+        if (c < classes) raw[v] = load_pack(xr + c);
+    }
+#pragma unroll
+    for (int v = 0; v < VPT; v++) {
+        const int c = (v * THREADS + threadIdx.x) * N;
         if (c < classes) {
-            const Pack<T> pk = load_pack(xr + c);
 #pragma unroll
             for (int j = 0; j < N; j++) {
-                x[v][j] = pk.get(j);
+                const float xv = raw[v].get(j);
                 if (WANT_ARGMAX) {
-                    if (x[v][j] > am.v) {  // ascending c within the lane: strict > keeps the first
-                        am.v = x[v][j];
+                    if (xv > am.v) {  // ascending c within the lane: strict > keeps the first
+                        am.v = xv;
                         am.i = c + j;
                     }
                 } else {
-                    am.v = fmaxf(am.v, x[v][j]);
+                    am.v = fmaxf(am.v, xv);
                 }
             }
         }
@@ -110,7 +115,8 @@ __global__ __launch_bounds__(THREADS) void ce_fused_kernel(const T* __restrict__
     }
     const float mx = am.v;
 
-    // phase 2: e = 2^(x*log2e - max*log2e), kept in the same registers; row sum
+    // phase 2: row sum of e = 2^(x*log2e - max*log2e).  The exponent is never positive, so the bare
+    // hardware exp2 (results below 2^-126 flush to zero) is exact enough.
     const float bias = -mx * kLog2e;
     float sum = 0.f;
 #pragma unroll
@@ -118,19 +124,16 @@ __global__ __launch_bounds__(THREADS) void ce_fused_kernel(const T* __restrict__
         const int c = (v * THREADS + threadIdx.x) * N;
         if (c < classes) {
 #pragma unroll
-            for (int j = 0; j < N; j++) {
-                if (c + j == target && target_logit_out) target_logit_out[row] = x[v][j];
-                x[v][j] = exp2f(fmaf(x[v][j], kLog2e, bias));
-                sum += x[v][j];
-            }
+            for (int j = 0; j < N; j++) sum += __builtin_amdgcn_exp2f(fmaf(raw[v].get(j), kLog2e, bias));
         }
     }
     sum = block_sum<THREADS>(sum, s_f);
     const float inv = 1.0f / sum;
     const float gscale = inv * scale;
 
-    // phase 3: dlogit = (e/sum - onehot) * scale, one multiply per element; the lane that holds the
-    // target fixes its element up and writes the row loss
+    // phase 3: dlogit = (e/sum - onehot) * scale with e recomputed (a second exp2 costs less than the
+    // registers that keeping it would take); the lane that holds the target fixes its element up and
+    // writes the row loss
 #pragma unroll
     for (int v = 0; v < VPT; v++) {
         const int c = (v * THREADS + threadIdx.x) * N;
@@ -139,9 +142,12 @@ __global__ __launch_bounds__(THREADS) void ce_fused_kernel(const T* __restrict__
             const bool has_target = target >= c && target < c + N;
 #pragma unroll
             for (int j = 0; j < N; j++) {
-                float gv = x[v][j] * gscale;
+                const float xv = raw[v].get(j);
+                const float e = __builtin_amdgcn_exp2f(fmaf(xv, kLog2e, bias));
+                float gv = e * gscale;
                 if (has_target && c + j == target) {
-                    row_loss[row] = -logf(x[v][j] * inv + 1e-8f);
+                    row_loss[row] = -logf(e * inv + 1e-8f);
+                    if (target_logit_out) target_logit_out[row] = xv;
                     gv -= scale;
                 }
                 g.set(j, gv);
