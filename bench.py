@@ -32,12 +32,15 @@ from tests import gen  # noqa: E402  (seeded synthetic inputs shared with the te
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM-side bytes per launch (average over the launches of the config-5 step), from the FETCH_SIZE / WRITE_SIZE
-# runs summarised in profiles/c5_step_hbm_traffic_pmc.md (fetch x 1.997, write x 1.000 after calibration on
-# the library's copy kernel).  Keys are the profile names the library reports.
+# HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic_pmc.md
+# (fetch x 1.997, write x 1.000 after calibration on the library's copy kernel), per workload and per profile
+# name the library reports.  The config-5 GEMM figure is the average over that kernel's launches in the step
+# (dW of gate/up, q/o and lm_head: 501.7, 139.1 and 5022.9 MB).
 MEASURED_TRAFFIC = {
-    "gemm_tn_bf16_f32out_128x128x32": 374.5e6,
-    "ce_fused_bf16": 524.6e6,
+    "c5": {"gemm_tn_bf16_f32out_128x128x64": 336.3e6, "ce_fused_bf16": 524.6e6},
+    "c4": {},
+    "c3": {"attn_bwd": 78.2e6 + 51.9e6},
+    "c2": {"ce_fused_bf16": 1048.9e6},
 }
 
 CONFIGS = {
@@ -60,17 +63,17 @@ def arch(c):
     return {k: c[k] for k in ("vocab", "hidden", "heads", "kv_heads", "ffn", "layers", "tie")}
 
 
-def pick_dominant(prof):
+def pick_dominant(prof, workload):
     name = max(prof, key=lambda k: prof[k]["ms"])
     e = prof[name]
     per_launch_ms = e["ms"] / e["launches"]
     if e["unit"] == "flop":
         achieved = e["work"] / e["launches"] / (per_launch_ms * 1e-3) / 1e12
         return name, dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                          frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(name))
+                          frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(workload, {}).get(name))
     achieved = e["work"] / e["launches"] / (per_launch_ms * 1e-3) / 1e9
     return name, dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(name))
+                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(workload, {}).get(name))
 
 
 def kernel_table(prof):
@@ -166,7 +169,7 @@ def bench_lm(name, steps, warmup, cpu_tokens):
     prof = ctx.profile_stop()
     tokens_per_step = c["accum"] * c["mb"] * c["seq"]
     value = steps * tokens_per_step / elapsed
-    dom, roofline = pick_dominant(prof)
+    dom, roofline = pick_dominant(prof, name)
     roofline["kernel"] = dom
     step_flops = flops_per_token(c) * tokens_per_step
     out = dict(metric="train tokens/sec (fwd+bwd+AdamW)", value=round(value, 1), unit="tokens/s", n_gpus=1, steps=steps, warmup=warmup,
@@ -227,7 +230,8 @@ def bench_c3(steps, warmup):
                 vs_baseline=None, dtype="bf16", data="synthetic",
                 config=dict(workload="config3 causal GQA flash attention fwd+bwd, B8 S1024 Hq16 Hkv4 hd64, [B,H,S,hd]"),
                 roofline=dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                              frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=None, kernel="attn_bwd (dq + dkv kernels)"),
+                              frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC["c3"]["attn_bwd"],
+                              kernel="attn_bwd (dq + dkv kernels)"),
                 kernels=kernel_table(prof),
                 cpu_baseline=dict(value=round(tokens / cpu_s, 2), unit="tokens/s", cores=1, kind="port",
                                   sample="oracle unfused attention chain fwd+bwd on 1 of 32 (batch, KV group) slices, scaled x32"))
@@ -260,7 +264,7 @@ def bench_c2(steps, warmup):
     for _ in range(steps):
         step()
     prof = ctx.profile_stop()
-    dom, roofline = pick_dominant(prof)
+    dom, roofline = pick_dominant(prof, "c2")
     roofline["kernel"] = dom
     ctx.close()
     R.set_threads(1)

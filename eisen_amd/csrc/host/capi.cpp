@@ -5,6 +5,7 @@
 #include <string>
 
 #include "eisen_graph.h"
+#include "io.hpp"
 #include "nn.hpp"
 
 using namespace eisen;
@@ -227,6 +228,89 @@ int eisen_adamw_moments_to_cpu(eisen_adamw* opt, size_t i, float* m_out, float* 
 }
 float eisen_cosine_lr(float lr_max, float lr_min, size_t warmup, size_t total, size_t step) {
     return CosineScheduler{lr_max, lr_min, warmup, total}.get_lr(step);
+}
+
+
+// ---- data loader / checkpoints -----------------------------------------------------------------
+}  // extern "C"
+
+struct eisen_data_loader {
+    std::unique_ptr<BinaryDataLoader> dl;
+};
+namespace {
+thread_local std::string io_error;
+template <typename F>
+int io_guarded(F&& f) {
+    try {
+        f();
+        return 0;
+    } catch (const std::exception& e) {
+        io_error = e.what();
+        return 1;
+    }
+}
+}  // namespace
+
+extern "C" {
+
+const char* eisen_io_last_error(void) { return io_error.c_str(); }
+
+int eisen_data_loader_open(const char* path, size_t seq_len, size_t batch_size, eisen_data_loader** out) {
+    if (!out) return -1;
+    *out = nullptr;
+    return io_guarded([&] {
+        need(path, "path");
+        auto h = std::make_unique<eisen_data_loader>();
+        h->dl = std::make_unique<BinaryDataLoader>(path, seq_len, batch_size);
+        *out = h.release();
+    });
+}
+int eisen_data_loader_close(eisen_data_loader* dl) {
+    delete dl;
+    return 0;
+}
+int eisen_data_loader_total_batches(eisen_data_loader* dl, size_t* out) {
+    if (!dl || !out) return -1;
+    *out = dl->dl->total_batches();
+    return 0;
+}
+int eisen_data_loader_next_batch(eisen_data_loader* dl, float* x, int64_t* targets, int* got) {
+    if (!dl) return -1;
+    return io_guarded([&] {
+        need(x, "x"); need(targets, "targets"); need(got, "got");
+        *got = dl->dl->next_batch(x, targets) ? 1 : 0;
+    });
+}
+int eisen_data_loader_reset(eisen_data_loader* dl) {
+    if (!dl) return -1;
+    dl->dl->reset();
+    return 0;
+}
+int eisen_graph_save_weights(eisen_graph* g, const char* path) {
+    return guarded(g, [&](Graph& G) { need(path, "path"); save_weights(G, path); });
+}
+int eisen_graph_load_weights(eisen_graph* g, const size_t* params, size_t n_params, const char* path, size_t* floats_out) {
+    return guarded(g, [&](Graph& G) {
+        need(path, "path");
+        if (n_params) need(params, "params");
+        const size_t n = load_weights(G, std::vector<size_t>(params, params + n_params), path);
+        if (floats_out) *floats_out = n;
+    });
+}
+int eisen_lm_write_safetensors(eisen_graph* g, eisen_lm* lm, const char* path) {
+    return guarded(g, [&](Graph& G) {
+        need(path, "path");
+        if (!lm || !lm->lm) throw Error("null model");
+        write_safetensors(G, lm->lm->named_params(), path);
+    });
+}
+int eisen_write_llama_config(const char* path, size_t vocab, size_t hidden, size_t ffn, size_t layers, size_t heads, size_t kv_heads,
+                             size_t max_position_embeddings, float rms_norm_eps, float rope_theta, int tie_word_embeddings) {
+    return io_guarded([&] {
+        need(path, "path");
+        write_llama_config(path, LlamaConfig{vocab, hidden, ffn, layers, heads, kv_heads, max_position_embeddings, rms_norm_eps, rope_theta,
+                                             tie_word_embeddings != 0});
+    });
 }
 
 }  // extern "C"

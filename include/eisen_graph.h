@@ -112,6 +112,34 @@ int eisen_adamw_moments_to_cpu(eisen_adamw* opt, size_t i, float* m_out, float* 
 /* CosineScheduler::get_lr (src/nn/scheduler.rs:45-55). */
 float eisen_cosine_lr(float lr_max, float lr_min, size_t warmup_steps, size_t total_steps, size_t step);
 
+/* ---- data in, weights out ------------------------------------------------------------------- */
+
+/* BinaryDataLoader (src/data/dataloader.rs:84-203), without fill-in-the-middle: a file of
+ * little-endian u16 token ids cut into windows of seq_len+1 tokens.  next_batch fills x (token ids as
+ * f32, [batch*seq]) and targets (the next token, [batch*seq]) and sets *got to 1, or sets it to 0 when
+ * the stream is exhausted (the reference returns None).  The refill pattern of the reference's 4 MiB
+ * BufReader is reproduced, so the two hand out the same batches and stop at the same one. */
+typedef struct eisen_data_loader eisen_data_loader;
+int eisen_data_loader_open(const char* path, size_t seq_len, size_t batch_size, eisen_data_loader** out);
+int eisen_data_loader_close(eisen_data_loader* dl);
+int eisen_data_loader_total_batches(eisen_data_loader* dl, size_t* out);
+int eisen_data_loader_next_batch(eisen_data_loader* dl, float* x, int64_t* targets, int* got);
+int eisen_data_loader_reset(eisen_data_loader* dl);
+/* Message of the last failed eisen_data_loader_* / eisen_write_llama_config call of this thread. */
+const char* eisen_io_last_error(void);
+
+/* save_weights (examples/train_llm.rs:93-105): parameter tensors in id order, raw f32 LE. */
+int eisen_graph_save_weights(eisen_graph* g, const char* path);
+/* load_weights (examples/chat_cli.rs:161-180): consecutive f32 runs, one per id; floats_out may be NULL. */
+int eisen_graph_load_weights(eisen_graph* g, const size_t* params, size_t n_params, const char* path, size_t* floats_out);
+/* write_safetensors over TransformerLM::named_params (src/tools/huggingface.rs:88-146,
+ * src/nn/transformer.rs:119-172): F32, linear weights transposed to [out, in]. */
+int eisen_lm_write_safetensors(eisen_graph* g, eisen_lm* lm, const char* path);
+/* write_llama_config (src/tools/huggingface.rs:38-84); num_key_value_heads is written as given
+ * (the reference repeats num_attention_heads there). */
+int eisen_write_llama_config(const char* path, size_t vocab, size_t hidden, size_t ffn, size_t layers, size_t heads, size_t kv_heads,
+                             size_t max_position_embeddings, float rms_norm_eps, float rope_theta, int tie_word_embeddings);
+
 #ifdef __cplusplus
 }
 #endif

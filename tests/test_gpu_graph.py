@@ -282,3 +282,55 @@ def test_reference_initialisers(ctx):
     wq = gg.sync_to_cpu(2)
     assert wq.shape == (8, 8) and abs(wq.std() - 0.02) < 0.01 and np.array_equal(wq, gg.sync_to_cpu(5))   # same seed per layer
     assert lm.params() == [0, 1, 2, 3, 4, 5, 6, 8, 9, 7, 10, 11]
+
+
+# ---- weights out: raw checkpoint and safetensors export ---------------------------------------
+
+@pytest.mark.parametrize("precision,tie", [(G.FP32, False), (G.BF16_MIXED, True)])
+def test_checkpoint_and_safetensors_export(ctx, tmp_path, precision, tie):
+    from safetensors.numpy import load_file
+
+    from eisen_amd import io as IO
+    from oracle import io_ref as IR
+    gr = G.Graph(ctx, precision)
+    lm = G.TransformerLM(gr, vocab=48, hidden=32, heads=4, kv_heads=2, ffn=64, layers=2, tie=tie)
+    gr.mark_params()  # everything allocated so far is a parameter (examples/train_llm.rs calls it after building the model)
+    # tensor-id (construction) order, the order of the raw checkpoint; Module::params() lists the FFN weights
+    # differently (src/nn/transformer.rs:57-66), which is why the reference's own save/load pair does not round-trip
+    params = sorted(lm.params())
+    arch = dict(vocab=48, hidden=32, heads=4, kv_heads=2, ffn=64, layers=2, tie=tie)
+    weights = [w for _, w in gen.lm_weights(77, perturb_norm=0.1, **arch)]
+    shapes = [s for _, s in gen.lm_param_shapes(**arch)]
+    assert len(params) == len(weights)
+    for pid, w in zip(params, weights):
+        gr.load_tensor_data(pid, w)
+    # raw checkpoint: every parameter in tensor-id order, f32 LE (examples/train_llm.rs:93-105)
+    ck = tmp_path / "model.bin"
+    IO.save_weights(gr, ck)
+    assert ck.read_bytes() == IR.save_weights_bytes(weights)
+    # and back (examples/chat_cli.rs:161-180) into a second model
+    lm2 = G.TransformerLM(gr, vocab=48, hidden=32, heads=4, kv_heads=2, ffn=64, layers=2, tie=tie)
+    assert IO.load_weights(gr, sorted(lm2.params()), ck) == sum(w.size for w in weights)
+    for pid, w in zip(sorted(lm2.params()), weights):
+        assert np.array_equal(gr.sync_to_cpu(pid).reshape(-1), w.reshape(-1))
+    ck.write_bytes(ck.read_bytes()[:-8])
+    with pytest.raises(EisenHipError, match="truncated"):
+        IO.load_weights(gr, lm2.params(), ck)
+    # safetensors: byte-identical to the restated writer, and readable by the safetensors library
+    st = tmp_path / "model.safetensors"
+    IO.write_safetensors(gr, lm, st)
+    names = ["model.embed_tokens.weight"]
+    for i in range(2):
+        names += [f"model.layers.{i}.{n}.weight" for n in ("input_layernorm", "self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj",
+                                                            "self_attn.o_proj", "post_attention_layernorm", "mlp.gate_proj", "mlp.up_proj",
+                                                            "mlp.down_proj")]
+    names += ["model.norm.weight"] + ([] if tie else ["lm_head.weight"])
+    assert len(names) == len(weights)
+    named = [(n, w.reshape(s)) for n, w, s in zip(names, weights, shapes)]
+    assert st.read_bytes() == IR.safetensors_bytes(named)
+    loaded = load_file(str(st))
+    assert sorted(loaded) == sorted(names)
+    for n, w in named:
+        want = w if (w.ndim != 2 or n == "model.embed_tokens.weight") else w.T
+        assert loaded[n].dtype == np.float32 and np.array_equal(loaded[n], want)
+    lm.close(); lm2.close(); gr.close()
