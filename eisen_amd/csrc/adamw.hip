@@ -30,6 +30,17 @@ __device__ __forceinline__ int find_slot(const SlotDev* __restrict__ slots, int 
     return lo;
 }
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+// streaming access: optimizer state is touched once per step and never reused from cache
+__device__ __forceinline__ float4 nt_load4(const float* p) {
+    const f32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
+    return make_float4(t[0], t[1], t[2], t[3]);
+}
+__device__ __forceinline__ void nt_store4(float* p, float4 v) {
+    f32x4_t t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<f32x4_t*>(p));
+}
+
 struct AdamParams {
     float lr, beta1, beta2, eps, wd, bc1, bc2;
 };
@@ -52,34 +63,49 @@ __global__ __launch_bounds__(kThreads) void adamw_kernel(const SlotDev* __restri
     const size_t base = (size_t)(blockIdx.x - s.first_block) * kChunk;
     const float gs = grad_scale ? grad_scale[0] : 1.0f;
     const bool vec = (s.n % 4 == 0);  // tensors come from the 256-byte-granule pool: bases are aligned
+    if (vec) {
+        // all 16 loads of the thread are issued before the first use: 16 KB per stream and workgroup in flight
+        float4 w[4], g[4], m[4], v[4];
+        bool on[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const size_t e = base + ((size_t)u * kThreads + threadIdx.x) * 4;
+            on[u] = e < s.n;
+            if (on[u]) {
+                w[u] = nt_load4(s.w + e);
+                g[u] = nt_load4(s.g + e);
+                m[u] = nt_load4(s.m + e);
+                v[u] = nt_load4(s.v + e);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (!on[u]) continue;
+            const size_t e = base + ((size_t)u * kThreads + threadIdx.x) * 4;
+            adam_elem(w[u].x, g[u].x * gs, m[u].x, v[u].x, p);
+            adam_elem(w[u].y, g[u].y * gs, m[u].y, v[u].y, p);
+            adam_elem(w[u].z, g[u].z * gs, m[u].z, v[u].z, p);
+            adam_elem(w[u].w, g[u].w * gs, m[u].w, v[u].w, p);
+            nt_store4(s.w + e, w[u]);
+            nt_store4(s.m + e, m[u]);
+            nt_store4(s.v + e, v[u]);
+            if (s.wb) {
+                bf16x4 b;
+                b[0] = (bf16_t)w[u].x; b[1] = (bf16_t)w[u].y; b[2] = (bf16_t)w[u].z; b[3] = (bf16_t)w[u].w;
+                *reinterpret_cast<bf16x4*>(s.wb + e) = b;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int u = 0; u < 4; u++) {
         const size_t e = base + ((size_t)u * kThreads + threadIdx.x) * 4;
         if (e >= s.n) break;
-        if (vec) {
-            float4 w = *reinterpret_cast<float4*>(s.w + e);
-            float4 g = *reinterpret_cast<const float4*>(s.g + e);
-            float4 m = *reinterpret_cast<float4*>(s.m + e);
-            float4 v = *reinterpret_cast<float4*>(s.v + e);
-            adam_elem(w.x, g.x * gs, m.x, v.x, p);
-            adam_elem(w.y, g.y * gs, m.y, v.y, p);
-            adam_elem(w.z, g.z * gs, m.z, v.z, p);
-            adam_elem(w.w, g.w * gs, m.w, v.w, p);
-            *reinterpret_cast<float4*>(s.w + e) = w;
-            *reinterpret_cast<float4*>(s.m + e) = m;
-            *reinterpret_cast<float4*>(s.v + e) = v;
-            if (s.wb) {
-                bf16x4 b;
-                b[0] = (bf16_t)w.x; b[1] = (bf16_t)w.y; b[2] = (bf16_t)w.z; b[3] = (bf16_t)w.w;
-                *reinterpret_cast<bf16x4*>(s.wb + e) = b;
-            }
-        } else {
-            for (int j = 0; j < 4 && e + j < s.n; j++) {
-                float w = s.w[e + j], m = s.m[e + j], v = s.v[e + j];
-                adam_elem(w, s.g[e + j] * gs, m, v, p);
-                s.w[e + j] = w; s.m[e + j] = m; s.v[e + j] = v;
-                if (s.wb) s.wb[e + j] = (bf16_t)w;
-            }
+        for (int j = 0; j < 4 && e + j < s.n; j++) {
+            float w = s.w[e + j], m = s.m[e + j], v = s.v[e + j];
+            adam_elem(w, s.g[e + j] * gs, m, v, p);
+            s.w[e + j] = w; s.m[e + j] = m; s.v[e + j] = v;
+            if (s.wb) s.wb[e + j] = (bf16_t)w;
         }
     }
 }
@@ -107,13 +133,29 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const SlotDev* __restri
     const SlotDev s = slots[si];
     const size_t base = (size_t)(blockIdx.x - s.first_block) * kChunk;
     double acc = 0.0;
+    if (s.n % 4 == 0) {
+        float4 g[4];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-        const size_t e = base + ((size_t)u * kThreads + threadIdx.x) * 4;
-        if (e >= s.n) break;
-        for (int j = 0; j < 4 && e + j < s.n; j++) {
-            const double x = (double)s.g[e + j];
-            acc += x * x;
+        for (int u = 0; u < 4; u++) {
+            const size_t e = base + ((size_t)u * kThreads + threadIdx.x) * 4;
+            g[u] = e < s.n ? *reinterpret_cast<const float4*>(s.g + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            acc += (double)g[u].x * (double)g[u].x;
+            acc += (double)g[u].y * (double)g[u].y;
+            acc += (double)g[u].z * (double)g[u].z;
+            acc += (double)g[u].w * (double)g[u].w;
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const size_t e = base + ((size_t)u * kThreads + threadIdx.x) * 4;
+            if (e >= s.n) break;
+            for (int j = 0; j < 4 && e + j < s.n; j++) {
+                const double x = (double)s.g[e + j];
+                acc += x * x;
+            }
         }
     }
     acc = wave_sum_f64(acc);
