@@ -87,6 +87,15 @@ struct TilePrefetch {
     bf16x8 r[CH];
     __device__ __forceinline__ void fetch(const bf16_t* src, long long row_stride, int first_row, int limit_rows) {
         const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (first_row + ROWS <= limit_rows) {  // whole tile in range (uniform): plain loads, no selects
+#pragma unroll
+            for (int i = 0; i < CH; i++) {
+                const int c = i * THREADS + threadIdx.x;
+                if (TOTAL % THREADS == 0 || c < TOTAL)
+                    r[i] = *reinterpret_cast<const bf16x8*>(src + (long long)(first_row + c / CPR) * row_stride + (c % CPR) * 8);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < CH; i++) {
             const int c = i * THREADS + threadIdx.x;
@@ -196,13 +205,13 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
             }
             // only tiles that touch the diagonal or the end of the sequence need the mask
             if ((a.causal && k0 + 63 > q0) || k0 + 64 > a.S) {
+                asm volatile("" ::: "memory");  // a real branch: off-diagonal tiles skip the 32 compares and selects
+                const int lim = min(a.causal ? q : a.S - 1, a.S - 1) - k0;  // tile rows above lim are masked
 #pragma unroll
                 for (int sub = 0; sub < 2; sub++)
 #pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        const int key = k0 + sub * 32 + acc_row(v, g);
-                        if ((a.causal && key > q) || key >= a.S) s[sub][v] = -INFINITY;
-                    }
+                    for (int v = 0; v < 16; v++)
+                        if (sub * 32 + acc_row(v, g) > lim) s[sub][v] = -INFINITY;
             }
             float mx = -INFINITY;  // of the raw scores; the (positive) scale is folded into the exponent's fma
 #pragma unroll
@@ -341,13 +350,18 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                 bf16x8 dsf[2];
                 // a query past the end has LSE = +inf and a key past the end a zero K row, so only
                 // the causal diagonal needs a mask
-                const bool diag = a.causal && k0 + 31 > q0;
+                float p[16];
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    float p = fast_exp2(fmaf(s[v], a.scale_log2e, -lse2));
-                    if (diag && k0 + acc_row(v, g) > q) p = 0.f;
-                    dsf[v >> 3][v & 7] = (bf16_t)(p * (dp[v] - Dq));
+                for (int v = 0; v < 16; v++) p[v] = fast_exp2(fmaf(s[v], a.scale_log2e, -lse2));
+                if (a.causal && k0 + 31 > q0) {
+                    asm volatile("" ::: "memory");  // keeps this a branch taken on the diagonal tile, not 16 selects on every tile
+                    const int rel = q - k0;       // keys k0 + row > q are masked
+#pragma unroll
+                    for (int v = 0; v < 16; v++)
+                        if (acc_row(v, g) > rel) p[v] = 0.f;
                 }
+#pragma unroll
+                for (int v = 0; v < 16; v++) dsf[v >> 3][v & 7] = (bf16_t)(p[v] * (dp[v] - Dq));
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
