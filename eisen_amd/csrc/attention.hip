@@ -22,6 +22,8 @@
 //     every query head of the group and every visible query tile; Q/dO tiles go through LDS.
 //     No atomics anywhere: dQ has its own query-stationary pass, so results are reproducible.
 // f32 path (any head_dim): one wave per query row / key row, plain FMA, for small shapes.
+#include <type_traits>
+
 #include "device_utils.cuh"
 #include "runtime.h"
 
@@ -177,7 +179,10 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
         TilePrefetch<HD, BKV, 256> pk, pv;
         pk.fetch(Kp, a.k_ss, 0, a.S);
         pv.fetch(Vp, a.k_ss, 0, a.S);
-        for (int kt = 0; kt < n_kt; kt++) {
+        // One 64-key tile.  MASKED is a compile-time flag: the tiles entirely below the diagonal and inside
+        // the sequence run a loop body with no mask code and no branches at all.
+        auto tile = [&](int kt, auto masked_c) {
+            constexpr bool MASKED = decltype(masked_c)::value;
             const bf16_t* Ks = Ksb[kt & 1];
             const bf16_t* Vs = Vsb[kt & 1];
             pk.commit(Ksb[kt & 1]);
@@ -188,8 +193,8 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                 pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
             }
             const int k0 = kt * BKV;
-            if (my_qmax < 0 || (a.causal && k0 > my_qmax)) continue;              // wave-uniform
-            const bool two = k0 + 32 < a.S && !(a.causal && k0 + 32 > my_qmax);  // the second 32 keys are visible
+            if (my_qmax < 0 || (a.causal && k0 > my_qmax)) return;                // wave-uniform
+            const bool two = !MASKED || (k0 + 32 < a.S && !(a.causal && k0 + 32 > my_qmax));  // the second 32 keys are visible
             f32x16 s[2];
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
@@ -204,8 +209,7 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                 }
             }
             // only tiles that touch the diagonal or the end of the sequence need the mask
-            if ((a.causal && k0 + 63 > q0) || k0 + 64 > a.S) {
-                asm volatile("" ::: "memory");  // a real branch: off-diagonal tiles skip the 32 compares and selects
+            if (MASKED) {
                 const int lim = min(a.causal ? q : a.S - 1, a.S - 1) - k0;  // tile rows above lim are masked
 #pragma unroll
                 for (int sub = 0; sub < 2; sub++)
@@ -253,7 +257,12 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt, pf[t], o[dt], 0, 0, 0);
                     }
             }
-        }
+        };
+        // tiles [0, n_plain) need no mask for any query of this wave: all their keys are <= q0 and < S
+        const int n_plain = min(n_kt, min(a.causal ? (q0 + 1) / BKV : n_kt, a.S / BKV));
+        int kt = 0;
+        for (; kt < n_plain; kt++) tile(kt, std::false_type{});
+        for (; kt < n_kt; kt++) tile(kt, std::true_type{});
         if (valid_q) {
             const float inv = l > 0.f ? 1.0f / l : 0.f;
             bf16_t* Op = static_cast<bf16_t*>(a.Out) + b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
@@ -323,7 +332,8 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
         TilePrefetch<HD, BKV, 256> pk, pv;
         pk.fetch(Kp, a.k_ss, 0, a.S);
         pv.fetch(Vp, a.k_ss, 0, a.S);
-        for (int kt = 0; kt < n_kt; kt++) {
+        auto tile = [&](int kt, auto masked_c) {
+            constexpr bool MASKED = decltype(masked_c)::value;  // false: no key of the tile is masked for this wave
             const bf16_t* Ks = Ksb[kt & 1];
             const bf16_t* Vs = Vsb[kt & 1];
             pk.commit(Ksb[kt & 1]);
@@ -336,7 +346,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
                 const int k0 = kt * BKV + sub * 32;
-                if (k0 >= a.S || my_qmax < 0 || (a.causal && k0 > my_qmax)) continue;
+                if (MASKED && (k0 >= a.S || my_qmax < 0 || (a.causal && k0 > my_qmax))) continue;
                 f32x16 s, dp;
 #pragma unroll
                 for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
@@ -353,8 +363,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                 float p[16];
 #pragma unroll
                 for (int v = 0; v < 16; v++) p[v] = fast_exp2(fmaf(s[v], a.scale_log2e, -lse2));
-                if (a.causal && k0 + 31 > q0) {
-                    asm volatile("" ::: "memory");  // keeps this a branch taken on the diagonal tile, not 16 selects on every tile
+                if (MASKED && a.causal && k0 + 31 > q0) {
                     const int rel = q - k0;       // keys k0 + row > q are masked
 #pragma unroll
                     for (int v = 0; v < 16; v++)
@@ -370,7 +379,11 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                         dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsf[t], dq[dt], 0, 0, 0);
                     }
             }
-        }
+        };
+        const int n_plain = my_qmax < 0 ? 0 : min(n_kt, min(a.causal ? (q0 + 1) / BKV : n_kt, a.S / BKV));
+        int kt = 0;
+        for (; kt < n_plain; kt++) tile(kt, std::false_type{});
+        for (; kt < n_kt; kt++) tile(kt, std::true_type{});
         if (valid_q) {
             bf16_t* dQp = static_cast<bf16_t*>(a.dQ) + qoff;
 #pragma unroll
