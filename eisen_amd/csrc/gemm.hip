@@ -42,6 +42,7 @@ struct GemmArgs {
     int split;                         // > 1: K is cut into this many parts; part p > 0 assigns into partial[p-1]
     int k_part;                        // contraction length of one part (a multiple of the slab)
     float* partial;                    // [batch][split-1][M][N] f32, summed into C by a second kernel
+    int vec_c;                         // C rows are 16-byte aligned at every 8th column: the epilogue may use 16-byte accesses
 };
 
 // ---- MFMA kernel -------------------------------------------------------------------------
@@ -196,6 +197,56 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
 
     // epilogue: accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile
     float* P = part > 0 ? g.partial + ((long long)bz * (split - 1) + (part - 1)) * g.M * g.N : nullptr;
+    constexpr int SP = WN + 4;  // staging pitch in floats
+    constexpr bool kCanStage = sizeof(lds) >= (size_t)WGM * WGN * 32 * SP * sizeof(float);
+    if (kCanStage && !EDGE && g.vec_c) {
+        // Each wave turns its accumulators, one 32-row band at a time, through a private piece of the
+        // (now idle) operand LDS so that a lane ends up with 8 consecutive columns of one row: C leaves in
+        // 16-byte stores covering whole 128/256-byte row segments instead of 2- or 4-byte ones.
+        float* stage = reinterpret_cast<float*>(&lds[0][0]) + wave * (32 * SP);
+        constexpr int LPR = WN / 8, PASSES = 32 * LPR / 64;  // lanes per row, passes per band
+        static_assert(32 * LPR % 64 == 0, "band must split evenly over the wave");
+        const int c = lane & 31, gh = lane >> 5;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) stage[(8 * (v / 4) + 4 * gh + (v % 4)) * SP + j * 32 + c] = acc[i][j][v];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ps++) {
+                const int idx = ps * 64 + lane, r = idx / LPR, cg = idx % LPR;
+                const float4 lo = *reinterpret_cast<const float4*>(stage + r * SP + cg * 8);
+                const float4 hi = *reinterpret_cast<const float4*>(stage + r * SP + cg * 8 + 4);
+                float val[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                const int m = m0 + wm * WM + i * 32 + r, n = n0 + wn * WN + cg * 8;
+                if (P) {
+                    float* dst = P + (long long)m * g.N + n;
+                    *reinterpret_cast<float4*>(dst) = lo;
+                    *reinterpret_cast<float4*>(dst + 4) = hi;
+                } else {
+                    TC* dst = C + (long long)m * g.ldc + n;
+                    Pack<TC> o[8 / Pack<TC>::N];
+                    if (g.accumulate) {
+#pragma unroll
+                        for (int k = 0; k < 8 / Pack<TC>::N; k++) o[k] = load_pack(dst + k * Pack<TC>::N);
+#pragma unroll
+                        for (int e = 0; e < 8; e++) val[e] += o[e / Pack<TC>::N].get(e % Pack<TC>::N);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; e++) o[e / Pack<TC>::N].set(e % Pack<TC>::N, val[e]);
+#pragma unroll
+                    for (int k = 0; k < 8 / Pack<TC>::N; k++) store_pack(dst + k * Pack<TC>::N, o[k]);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -229,10 +280,20 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs g, int
     TC* dst = static_cast<TC*>(g.C) + bz * g.sC + (long long)m * g.ldc + n;
     float sum[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) sum[i] = to_f32(dst[i]);
-    for (int p = 0; p < g.split - 1; p++) {
-        const float4 x = *reinterpret_cast<const float4*>(g.partial + (bz * (g.split - 1) + p) * per + e);
-        sum[0] += x.x; sum[1] += x.y; sum[2] += x.z; sum[3] += x.w;
+    for (int i = 0; i < 4; i++) sum[i] = to_f32(dst[i]);  // part 0 already went into C (assigned or accumulated)
+    // the partials are fetched eight at a time (independent loads in flight) and added in part order
+    const float* part0 = g.partial + bz * (g.split - 1) * per + e;
+    for (int p0 = 0; p0 < g.split - 1; p0 += 8) {
+        float4 x[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            x[i] = p0 + i < g.split - 1 ? *reinterpret_cast<const float4*>(part0 + (long long)(p0 + i) * per) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (p0 + i < g.split - 1) {
+                sum[0] += x[i].x; sum[1] += x[i].y; sum[2] += x[i].z; sum[3] += x[i].w;
+            }
+        }
     }
 #pragma unroll
     for (int i = 0; i < 4; i++) dst[i] = from_f32<TC>(sum[i]);
@@ -339,6 +400,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     g.ldc = (int)N;
     g.sA = sA; g.sB = sB; g.sC = sC;
     g.accumulate = accumulate;
+    g.vec_c = eisen_aligned(C, 16) && N % 8 == 0 && (sC * eisen_dtype_size(dtype_c)) % 16 == 0;
     if (K == 0) {  // empty contraction: C (+)= 0
         if (!accumulate) {
             for (size_t b = 0; b < batch; b++) {
