@@ -450,14 +450,12 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         }
         // Tile choice (measured on MI355X at the config-5 shapes): 256x128 with 8 waves is ~5 % ahead of
         // 128x128 with 4 when at least one operand is k-contiguous and the grid still covers every CU; two
-        // transposed operands (dW) need too much LDS for it.  64x64 is for problems with few tiles.
+        // transposed operands (dW) need too much LDS for it and run 128x128 with 4 waves.  64x64 is for
+        // problems with few tiles.
         if (wide) {
             launch_mfma_c<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else if (big_tile || split128) {
-            // two transposed operands (dW) fill 80 KB of LDS, one workgroup per CU: 8 waves on the tile
-            // instead of 4 keep two waves per SIMD to overlap each other's LDS reads (+7 % measured)
-            if (K % 64 == 0 && !a_kc && !b_kc) launch_mfma_c<128, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-            else if (K % 64 == 0) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            if (K % 64 == 0) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
             else launch_mfma_c<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else {
             launch_mfma_c<64, 64, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
