@@ -433,8 +433,10 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
             while (split < 32 && tiles * split * 2 <= 256 && K / (split * 2) >= min_part && K % (split * 2 * slab) == 0) split *= 2;
     }
     const bool split128 = split > 1 && M >= 128 && N >= 128;
-    const bool wide = mfma_ok && split == 1 && big_tile && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && (a_kc || b_kc) &&
-                      (long long)(M / 256) * (N / 128) * batch >= 256;
+    // 256x128 tiles only when they fill whole rounds of the 256 CUs well (one workgroup per CU)
+    const long long wide_tiles = (long long)(M / 256) * (N / 128) * batch;
+    const bool wide = mfma_ok && split == 1 && big_tile && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && wide_tiles >= 256 &&
+                      (double)wide_tiles / (double)(256 * ((wide_tiles + 255) / 256)) >= 0.85;
     const char* tile = !mfma_ok ? "fma64x64" : wide ? "256x128x64" : (big_tile || split128) ? (K % 64 == 0 ? "128x128x64" : "128x128x32") : "64x64x32";
     snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
              dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : "");
