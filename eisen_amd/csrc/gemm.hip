@@ -489,3 +489,10 @@ extern "C" int eisen_hip_bmm(eisen_ctx* ctx, const void* A, const void* B, void*
     return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, batch, (long long)(M * K), (long long)(K * N),
                        (long long)(M * N), accumulate, "eisen_hip_bmm");
 }
+
+extern "C" int eisen_hip_gemm_strided_batched(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
+                                              int trans_b, size_t batch, size_t M, size_t N, size_t K, long long stride_a,
+                                              long long stride_b, long long stride_c, int accumulate) {
+    return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, batch, stride_a, stride_b, stride_c, accumulate,
+                       "eisen_hip_gemm_strided_batched");
+}

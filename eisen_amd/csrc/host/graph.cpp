@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <memory>
 #include <numeric>
 
 namespace eisen {
@@ -246,6 +247,7 @@ void Graph::materialize_grad(size_t id) {
 void Graph::backward(size_t loss_id) {
     if (no_grad) return;
     backward_root_ = loss_id;
+    backward_epoch_++;
     int acc = 0;
     Storage& lg = grad_for_write(loss_id, &acc);
     check(eisen_hip_fill(ctx_, lg.ptr, lg.dtype, 1.0f, lg.numel), "backward seed");
@@ -373,6 +375,68 @@ size_t Graph::matmul(size_t a, size_t b) {
         g.check(eisen_hip_gemm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul backward dB");
     });
     return out;
+}
+
+// Two Graph::matmul calls that share their left operand (K and V projections, gate and up projections:
+// src/nn/attention.rs:300-302, src/nn/transformer.rs:41-44) as one batched launch forward and one for
+// the two dW; results are those of the two separate matmuls.  The operands of the pair are addressed as a
+// batch of two whose "stride" is the distance between the two tensors.
+std::pair<size_t, size_t> Graph::matmul_pair(size_t a, size_t b1, size_t b2) {
+    const std::vector<size_t> sa = at(a).shape, sb = at(b1).shape;
+    const Storage w1 = compute_data(b1), w2 = compute_data(b2);
+    const size_t es = w1.dtype == EISEN_BF16 ? 2 : 4;
+    const ptrdiff_t wdiff = (const char*)w2.ptr - (const char*)w1.ptr;
+    const bool pairable = sb.size() == 2 && at(b2).shape == sb && !sa.empty() && sa.back() == sb[0] && w1.dtype == w2.dtype &&
+                          compute_data(a).dtype == w1.dtype && wdiff % (ptrdiff_t)(8 * es) == 0 && b1 != b2;
+    if (!pairable) return {matmul(a, b1), matmul(a, b2)};
+    const size_t K = sa.back(), M = numel_of(sa) / std::max<size_t>(K, 1), N = sb[1];
+    const Storage da = compute_data(a);
+    const size_t o1 = push_tensor({M, N}, da.dtype, true), o2 = push_tensor({M, N}, da.dtype, true);
+    const ptrdiff_t odiff = (const char*)at(o2).data.ptr - (const char*)at(o1).data.ptr;
+    if (odiff % (ptrdiff_t)(8 * es) != 0) throw Error("matmul_pair: outputs are not 16-byte congruent");
+    check(eisen_hip_gemm_strided_batched(ctx_, da.ptr, w1.ptr, at(o1).data.ptr, da.dtype, da.dtype, 0, 0, 2, M, N, K, 0,
+                                         wdiff / (ptrdiff_t)es, odiff / (ptrdiff_t)es, 0), "matmul_pair");
+    auto epoch = std::make_shared<size_t>((size_t)-1);
+    auto fn = [=](Graph& g) {
+        if (*epoch == g.backward_epoch()) return;  // the node is on the tape once per output; it runs once per backward
+        *epoch = g.backward_epoch();
+        const bool h1 = g.has_grad(o1), h2 = g.has_grad(o2);
+        // dA (+)= dY2 W2^T (+) dY1 W1^T: the later matmul first, as the reversed tape of two separate matmuls would
+        for (int which = 1; which >= 0; which--) {
+            if (!(which == 0 ? h1 : h2)) continue;
+            const Storage& go = g.grad_for_read(which == 0 ? o1 : o2);
+            int acc = 0;
+            Storage& ga = g.grad_for_write(a, &acc);
+            g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(which == 0 ? b1 : b2).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc),
+                    "matmul_pair backward dA");
+        }
+        // dW1, dW2 (+)= A^T dY1, A^T dY2: one launch when both exist and are in the same accumulate state
+        const Storage xa = g.compute_data(a);
+        if (h1 && h2) {
+            const Storage& go1 = g.grad_for_read(o1);
+            const Storage& go2 = g.grad_for_read(o2);
+            int acc1 = 0, acc2 = 0;
+            Storage& g1 = g.grad_for_write(b1, &acc1);
+            Storage& g2 = g.grad_for_write(b2, &acc2);
+            const size_t gs = g1.dtype == EISEN_BF16 ? 2 : 4, os = go1.dtype == EISEN_BF16 ? 2 : 4;
+            const ptrdiff_t gd = (const char*)g2.ptr - (const char*)g1.ptr, od = (const char*)go2.ptr - (const char*)go1.ptr;
+            if (acc1 == acc2 && g1.dtype == g2.dtype && go1.dtype == go2.dtype && gd % (ptrdiff_t)16 == 0 && od % (ptrdiff_t)16 == 0) {
+                g.check(eisen_hip_gemm_strided_batched(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, 2, K, N, M, 0,
+                                                       od / (ptrdiff_t)os, gd / (ptrdiff_t)gs, acc1), "matmul_pair backward dW");
+            } else {
+                g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, K, N, M, acc1), "matmul_pair backward dW1");
+                g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go2.ptr, g2.ptr, go2.dtype, g2.dtype, 1, 0, K, N, M, acc2), "matmul_pair backward dW2");
+            }
+        } else if (h1 || h2) {
+            const Storage& go = g.grad_for_read(h1 ? o1 : o2);
+            int acc = 0;
+            Storage& gb = g.grad_for_write(h1 ? b1 : b2, &acc);
+            g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul_pair backward dW");
+        }
+    };
+    record({a, b1, b2}, o1, fn);
+    record({a, b1, b2}, o2, fn);
+    return {o1, o2};
 }
 
 // Graph::matmul_trans_b (src/graph/ops/linear.rs:301-523; GPU arm semantics): C = A B^T with

@@ -7,6 +7,7 @@
 // bf16 in mixed mode, parameters keep f32 master weights next to a bf16 copy, and nothing
 // synchronises the stream unless the caller reads a value back.
 #pragma once
+#include <utility>
 #include <cstdint>
 #include <functional>
 #include <stdexcept>
@@ -104,6 +105,8 @@ class Graph {
     size_t silu(size_t a);
     size_t swiglu(size_t gate, size_t up);                      // fused silu(gate) * up
     size_t matmul(size_t a, size_t b);
+    // two matmuls of the same input against two equally shaped weights, as one launch each way
+    std::pair<size_t, size_t> matmul_pair(size_t a, size_t b1, size_t b2);
     size_t matmul_bf16(size_t a, size_t b) { return matmul(a, b); }
     size_t matmul_trans_b(size_t a, size_t b);
     size_t bmm(size_t a, size_t b, bool trans_b);
@@ -137,10 +140,13 @@ class Graph {
     void refresh_shadow(size_t id);           // re-cast the master weight into the bf16 copy
     void check(int rc, const char* what) const;
     size_t backward_root() const { return backward_root_; }
+    size_t backward_epoch() const { return backward_epoch_; }  // counts backward() calls
+    bool has_grad(size_t id) { const Tensor& t = at(id); return t.is_param || (t.grad.valid() && t.grad_written); }
 
    private:
     eisen_ctx* ctx_;
     size_t backward_root_ = (size_t)-1;
+    size_t backward_epoch_ = 0;
     size_t push_tensor(const std::vector<size_t>& shape, int dtype, bool pooled);
     Storage device_alloc(size_t numel, int dtype, bool zero);
     void device_free(Storage& s);

@@ -88,7 +88,20 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
     const std::vector<size_t> xs = g.at(x_id).shape;
     if (xs.size() != 3) throw Error("GQA requires [Batch, Seq, Dim]");
     const size_t batch = xs[0], seq = xs[1];
-    const size_t q = q_proj.forward(g, x_id), k = k_proj.forward(g, x_id), v = v_proj.forward(g, x_id);
+    const size_t q = q_proj.forward(g, x_id);
+    size_t k, v;
+    if (fused && !k_proj.has_bias && !v_proj.has_bias) {
+        // K and V projections read the same input and have the same shape: one launch for both
+        const std::pair<size_t, size_t> kv = g.matmul_pair(x_id, k_proj.weight_id, v_proj.weight_id);
+        k = kv.first;
+        v = kv.second;
+        const size_t kv_dim = g.at(k_proj.weight_id).shape[1];
+        g.reinterpret_shape(k, {batch, seq, kv_dim});
+        g.reinterpret_shape(v, {batch, seq, kv_dim});
+    } else {
+        k = k_proj.forward(g, x_id);
+        v = v_proj.forward(g, x_id);
+    }
     const size_t q_rope = g.rope(q, head_dim), k_rope = g.rope(k, head_dim);
     const float scale = 1.0f / std::sqrt((float)head_dim);
     if (fused) {
@@ -150,12 +163,23 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
     const size_t attn_out = attn.forward_with_mask(g, norm1_out, causal);
     const size_t res1 = g.add(x_id, attn_out);
     const size_t norm2_out = norm2.forward(g, res1);
-    const size_t gate_out = ffn_gate.forward(g, norm2_out);
     size_t gated;
-    if (attn.fused) {
+    if (attn.fused && !ffn_gate.has_bias && !ffn1.has_bias) {
+        // gate and up projections as one launch, then the fused SwiGLU
+        const std::pair<size_t, size_t> gu = g.matmul_pair(norm2_out, ffn_gate.weight_id, ffn1.weight_id);
+        const std::vector<size_t> ns = g.at(norm2_out).shape;
+        if (ns.size() == 3) {
+            const size_t f = g.at(ffn_gate.weight_id).shape[1];
+            g.reinterpret_shape(gu.first, {ns[0], ns[1], f});
+            g.reinterpret_shape(gu.second, {ns[0], ns[1], f});
+        }
+        gated = g.swiglu(gu.first, gu.second);
+    } else if (attn.fused) {
+        const size_t gate_out = ffn_gate.forward(g, norm2_out);
         const size_t up = ffn1.forward(g, norm2_out);
         gated = g.swiglu(gate_out, up);
     } else {
+        const size_t gate_out = ffn_gate.forward(g, norm2_out);
         const size_t gate = g.silu(gate_out);
         const size_t up = ffn1.forward(g, norm2_out);
         gated = g.mul(gate, up);

@@ -259,6 +259,11 @@ class Context:
     def bmm(self, A, B, Cbuf, dtype_ab, dtype_c, trans_a, trans_b, batch, M, N, K, accumulate=0):
         self._call("eisen_hip_bmm", _ptr(A), _ptr(B), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(batch), _sz(M), _sz(N), _sz(K), _i(accumulate))
 
+    def gemm_strided_batched(self, A, B, Cbuf, dtype_ab, dtype_c, trans_a, trans_b, batch, M, N, K, stride_a, stride_b, stride_c, accumulate=0):
+        """Batch strides in elements; 0 shares the operand, negative walks backwards."""
+        self._call("eisen_hip_gemm_strided_batched", _ptr(A), _ptr(B), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(batch),
+                   _sz(M), _sz(N), _sz(K), C.c_longlong(stride_a), C.c_longlong(stride_b), C.c_longlong(stride_c), _i(accumulate))
+
     # ---- attention --------------------------------------------------------------------
     @staticmethod
     def _strides(v):

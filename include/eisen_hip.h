@@ -200,6 +200,13 @@ int eisen_hip_gemm(eisen_ctx* ctx, const void* A, const void* B, void* C, int dt
  * kernels/ops_f32.cu:342-510; Graph::bmm, src/graph/ops/linear.rs:1198-1511). */
 int eisen_hip_bmm(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
                   int trans_b, size_t batch, size_t M, size_t N, size_t K, int accumulate);
+/* The same with explicit batch strides in elements (any sign, 0 = operand shared by every batch).  This is how
+ * linear layers that read the same input run as one launch: K and V projections, or the gate and up
+ * projections of the MLP (src/nn/attention.rs:300-302, src/nn/transformer.rs:41-44 issue them as separate
+ * matmuls): A shared, B and C "strided" by the distance between the two weight / output tensors. */
+int eisen_hip_gemm_strided_batched(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
+                                   int trans_b, size_t batch, size_t M, size_t N, size_t K, long long stride_a,
+                                   long long stride_b, long long stride_c, int accumulate);
 
 /* ---- attention ------------------------------------------------------------------------- */
 

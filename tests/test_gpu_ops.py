@@ -3,6 +3,8 @@
 Run on an MI355X with `pytest -m gpu`.  All calls go through libeisen_hip.so's C-ABI
 (eisen_amd.hip is a ctypes mirror of include/eisen_hip.h); the oracle is only the checker.
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -516,6 +518,44 @@ def test_gemm_f32_and_odd_shapes(ctx, ta, tb, M, N, K):
     _gemm_case(ctx, M, N, K, ta, tb, F32, F32, False)
     _gemm_case(ctx, M, N, K, ta, tb, F32, F32, True)
     _gemm_case(ctx, M, N, K, ta, tb, BF16, BF16, False)        # odd shapes fall back to the FMA kernel
+
+
+def test_gemm_strided_batched_shared_operand(ctx):
+    # two projections of one input as a single launch: A shared (stride 0), the second weight / output
+    # addressed by the distance between the tensors (here the second one lies *before* the first: negative stride)
+    M, N, K = 256, 128, 192
+    a = prep(gen.normal(430, (M, K)), BF16)
+    w = [prep(gen.normal(431 + i, (K, N)), BF16) for i in range(2)]
+    da = up(ctx, a, BF16)
+    wbuf, obuf = ctx.malloc(2 * K * N * 2 + 4096), ctx.malloc(2 * M * N * 2 + 4096)
+    gap_w, gap_o = K * N + 1024, M * N + 512              # elements between the tensors (multiples of 8)
+    w_ptrs = [wbuf.ptr + gap_w * 2, wbuf.ptr]              # tensor 0 behind tensor 1
+    o_ptrs = [obuf.ptr + gap_o * 2, obuf.ptr]
+    def put(ptr, arr):
+        bits = hip.f32_to_bf16_bits(arr)
+        ctx._call("eisen_hip_htod", C.c_void_p(ptr), bits.ctypes.data_as(C.c_void_p), C.c_size_t(bits.nbytes))
+
+    def get(ptr, shape, dtype):
+        return ctx.download(ptr, shape, dtype)
+
+    for i in range(2):
+        put(w_ptrs[i], w[i])
+    ctx.gemm_strided_batched(da, w_ptrs[0], o_ptrs[0], BF16, BF16, 0, 0, 2, M, N, K, 0, -gap_w, -gap_o)
+    for i in range(2):
+        got = get(o_ptrs[i], (M, N), BF16)
+        assert_close(got, a.astype(np.float64) @ w[i].astype(np.float64), 2e-2, f"pair {i}")
+    # dW of both at once: A^T shared, f32 outputs accumulate
+    go = [prep(gen.normal(440 + i, (M, N)), BF16) for i in range(2)]
+    gbuf, dwbuf = ctx.malloc(2 * M * N * 2 + 4096), ctx.malloc(2 * K * N * 4 + 8192, zero=True)
+    g_ptrs = [gbuf.ptr, gbuf.ptr + gap_o * 2]
+    d_ptrs = [dwbuf.ptr, dwbuf.ptr + (K * N + 1024) * 4]
+    for i in range(2):
+        put(g_ptrs[i], go[i])
+    for _ in range(2):  # second call accumulates
+        ctx.gemm_strided_batched(da, g_ptrs[0], d_ptrs[0], BF16, F32, 1, 0, 2, K, N, M, 0, gap_o, K * N + 1024, 1)
+    for i in range(2):
+        got = get(d_ptrs[i], (K, N), F32)
+        assert_close(got, 2 * (a.astype(np.float64).T @ go[i].astype(np.float64)), 1e-3, f"pair dW {i}")
 
 
 def test_gemm_f32_matches_oracle_order_tolerance(ctx):
