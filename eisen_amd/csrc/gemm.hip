@@ -43,6 +43,13 @@ struct GemmArgs {
     int k_part;                        // contraction length of one part (a multiple of the slab)
     float* partial;                    // [batch][split-1][M][N] f32, summed into C by a second kernel
     int vec_c;                         // C rows are 16-byte aligned at every 8th column: the epilogue may use 16-byte accesses
+    // K made of up to three segments with their own operands, C (+)= sum_s op(A_s) op(B_s): segment 0 is A/B/lda/ldb,
+    // seg_end[s] is the contraction offset at which segment s ends (multiples of 64); nseg <= 1 means plain
+    int nseg;
+    const void* A_seg[2];
+    const void* B_seg[2];
+    int lda_seg[2], ldb_seg[2];
+    int seg_end[2];
 };
 
 // ---- MFMA kernel -------------------------------------------------------------------------
@@ -142,8 +149,20 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
     constexpr int KSTEPS = BK / 16, NCH = TA::CHUNKS + TB::CHUNKS;
     bf16x8 r[NCH];
     auto load_chunk = [&](int h, int slab) {
-        if (h < TA::CHUNKS) r[h] = TA::template load<EDGE>(A, g.lda, m0, k_lo + slab * BK, g.M, k_hi, h, tid);
-        else r[h] = TB::template load<EDGE>(B, g.ldb, n0, k_lo + slab * BK, g.N, k_hi, h - TA::CHUNKS, tid);
+        // the slab's segment (uniform): selected with scalar selects, no branch in the main loop
+        int k0 = k_lo + slab * BK, lda = g.lda, ldb = g.ldb;
+        const bf16_t* Ap = A;
+        const bf16_t* Bp = B;
+        if (g.nseg > 1) {
+            const bool s1 = k0 >= g.seg_end[0], s2 = g.nseg > 2 && k0 >= g.seg_end[1];
+            Ap = s2 ? static_cast<const bf16_t*>(g.A_seg[1]) : s1 ? static_cast<const bf16_t*>(g.A_seg[0]) : A;
+            Bp = s2 ? static_cast<const bf16_t*>(g.B_seg[1]) : s1 ? static_cast<const bf16_t*>(g.B_seg[0]) : B;
+            lda = s2 ? g.lda_seg[1] : s1 ? g.lda_seg[0] : lda;
+            ldb = s2 ? g.ldb_seg[1] : s1 ? g.ldb_seg[0] : ldb;
+            k0 -= s2 ? g.seg_end[1] : s1 ? g.seg_end[0] : 0;
+        }
+        if (h < TA::CHUNKS) r[h] = TA::template load<EDGE>(Ap, lda, m0, k0, g.M, k_hi, h, tid);
+        else r[h] = TB::template load<EDGE>(Bp, ldb, n0, k0, g.N, k_hi, h - TA::CHUNKS, tid);
     };
     auto store_chunk = [&](int h, int buf) {
         if (h < TA::CHUNKS) TA::store(lds[buf], r[h], h, tid);
@@ -383,15 +402,36 @@ void launch_generic(eisen_ctx* ctx, const GemmArgs& g, int trans_a, int trans_b,
 }  // namespace
 
 // Internal entry shared by eisen_hip_gemm and eisen_hip_bmm.
+struct KSegments {  // further (A, B, K) segments after the first one
+    int n = 0;
+    const void* A[2];
+    const void* B[2];
+    size_t K[2];
+};
 static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
                        int trans_b, size_t M, size_t N, size_t K, size_t batch, long long sA, long long sB, long long sC,
-                       int accumulate, const char* who) {
+                       int accumulate, const char* who, const KSegments* segs = nullptr) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, A && B && C, EISEN_E_ARG, "%s: null pointer", who);
     EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype_ab) && eisen_dtype_ok(dtype_c), EISEN_E_ARG, "%s: unknown dtype", who);
     EISEN_REQUIRE(ctx, !(dtype_ab == EISEN_F32 && dtype_c == EISEN_BF16), EISEN_E_ARG, "%s: f32 operands with bf16 output is not a supported combination", who);
     EISEN_REQUIRE(ctx, M < (size_t(1) << 30) && N < (size_t(1) << 30) && K < (size_t(1) << 30) && batch < 65536, EISEN_E_SHAPE, "%s: dimension out of range", who);
     if (M == 0 || N == 0 || batch == 0) return 0;
+    const int n_more = segs ? segs->n : 0;
+    if (n_more > 0) {
+        // one launch needs bf16 operands, no batch and every segment a whole number of 64-deep slabs;
+        // anything else runs as one accumulating GEMM per segment
+        bool one = dtype_ab == EISEN_BF16 && batch == 1 && K % 64 == 0 && K > 0 && n_more <= 2 && eisen_aligned(A, 16) && eisen_aligned(B, 16) &&
+                   (trans_a ? M % 8 == 0 : true) && (trans_b ? true : N % 8 == 0);
+        for (int i = 0; i < n_more && one; i++)
+            one = segs->A[i] && segs->B[i] && segs->K[i] % 64 == 0 && segs->K[i] > 0 && eisen_aligned(segs->A[i], 16) && eisen_aligned(segs->B[i], 16);
+        if (!one) {
+            int rc = gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, batch, sA, sB, sC, accumulate, who);
+            for (int i = 0; i < n_more && !rc; i++)
+                rc = gemm_common(ctx, segs->A[i], segs->B[i], C, dtype_ab, dtype_c, trans_a, trans_b, M, N, segs->K[i], batch, sA, sB, sC, 1, who);
+            return rc;
+        }
+    }
     GemmArgs g{};
     g.A = A; g.B = B; g.C = C;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
@@ -401,6 +441,21 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     g.sA = sA; g.sB = sB; g.sC = sC;
     g.accumulate = accumulate;
     g.vec_c = eisen_aligned(C, 16) && N % 8 == 0 && (sC * eisen_dtype_size(dtype_c)) % 16 == 0;
+    if (n_more > 0) {
+        size_t end = K;
+        for (int i = 0; i < n_more; i++) {
+            g.A_seg[i] = segs->A[i];
+            g.B_seg[i] = segs->B[i];
+            g.lda_seg[i] = (int)(trans_a ? M : segs->K[i]);
+            g.ldb_seg[i] = (int)(trans_b ? segs->K[i] : N);
+            g.seg_end[i] = (int)end;   // segment i+1 starts where the previous ones end
+            end += segs->K[i];
+        }
+        g.nseg = n_more + 1;
+        K = end;                       // from here on: the whole contraction
+        g.K = (int)K;
+        EISEN_REQUIRE(ctx, K < (size_t(1) << 30), EISEN_E_SHAPE, "%s: dimension out of range", who);
+    }
     if (K == 0) {  // empty contraction: C (+)= 0
         if (!accumulate) {
             for (size_t b = 0; b < batch; b++) {
@@ -416,6 +471,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     // the contiguous dimension of each operand must be a whole number of 8-element chunks
     if (a_kc) mfma_ok = mfma_ok && K % 8 == 0; else mfma_ok = mfma_ok && M % 8 == 0;
     if (b_kc) mfma_ok = mfma_ok && K % 8 == 0; else mfma_ok = mfma_ok && N % 8 == 0;
+    EISEN_REQUIRE(ctx, n_more == 0 || mfma_ok, EISEN_E_ARG, "%s: segmented contraction reached a shape the MFMA kernel does not take", who);
     // profile key = one kernel instantiation (operand orders, types, tile), so the event timing
     // lines up with a profiler's per-kernel rows
     char pname[64];
@@ -425,7 +481,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     // gets a tile.  Part 0 writes C as usual, the other parts go to an f32 scratch that a second kernel
     // adds to C in a fixed order, so the result does not depend on scheduling.
     int split = 1;
-    if (mfma_ok && N % 4 == 0 && K >= 1024) {
+    if (mfma_ok && N % 4 == 0 && K >= 1024 && n_more == 0) {
         const bool t128 = M >= 128 && N >= 128;
         const long long tiles = t128 ? tiles128 : (long long)eisen_ceil_div(M, 64) * eisen_ceil_div(N, 64) * batch;
         const size_t slab = t128 ? 64 : 32, min_part = t128 ? 512 : 256;
@@ -495,4 +551,18 @@ extern "C" int eisen_hip_gemm_strided_batched(eisen_ctx* ctx, const void* A, con
                                               long long stride_b, long long stride_c, int accumulate) {
     return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, batch, stride_a, stride_b, stride_c, accumulate,
                        "eisen_hip_gemm_strided_batched");
+}
+
+extern "C" int eisen_hip_gemm_ksegments(eisen_ctx* ctx, size_t n_segments, const void* const* A, const void* const* B, const size_t* K,
+                                        void* C, int dtype_ab, int dtype_c, int trans_a, int trans_b, size_t M, size_t N, int accumulate) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, A && B && K && C && n_segments >= 1 && n_segments <= 3, EISEN_E_ARG, "eisen_hip_gemm_ksegments: 1 to 3 segments, no null pointers");
+    KSegments more;
+    more.n = (int)n_segments - 1;
+    for (int i = 0; i < more.n; i++) {
+        more.A[i] = A[i + 1];
+        more.B[i] = B[i + 1];
+        more.K[i] = K[i + 1];
+    }
+    return gemm_common(ctx, A[0], B[0], C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K[0], 1, 0, 0, 0, accumulate, "eisen_hip_gemm_ksegments", &more);
 }

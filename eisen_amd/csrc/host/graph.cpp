@@ -377,66 +377,106 @@ size_t Graph::matmul(size_t a, size_t b) {
     return out;
 }
 
-// Two Graph::matmul calls that share their left operand (K and V projections, gate and up projections:
-// src/nn/attention.rs:300-302, src/nn/transformer.rs:41-44) as one batched launch forward and one for
-// the two dW; results are those of the two separate matmuls.  The operands of the pair are addressed as a
-// batch of two whose "stride" is the distance between the two tensors.
-std::pair<size_t, size_t> Graph::matmul_pair(size_t a, size_t b1, size_t b2) {
-    const std::vector<size_t> sa = at(a).shape, sb = at(b1).shape;
-    const Storage w1 = compute_data(b1), w2 = compute_data(b2);
-    const size_t es = w1.dtype == EISEN_BF16 ? 2 : 4;
-    const ptrdiff_t wdiff = (const char*)w2.ptr - (const char*)w1.ptr;
-    const bool pairable = sb.size() == 2 && at(b2).shape == sb && !sa.empty() && sa.back() == sb[0] && w1.dtype == w2.dtype &&
-                          compute_data(a).dtype == w1.dtype && wdiff % (ptrdiff_t)(8 * es) == 0 && b1 != b2;
-    if (!pairable) return {matmul(a, b1), matmul(a, b2)};
-    const size_t K = sa.back(), M = numel_of(sa) / std::max<size_t>(K, 1), N = sb[1];
+// Several Graph::matmul calls that share their left operand (Q/K/V projections, gate and up projections:
+// src/nn/attention.rs:300-302, src/nn/transformer.rs:41-44), with the results of the separate matmuls but
+// fewer launches: equally shaped neighbours (K and V, gate and up) run as a batch of two whose "stride" is the
+// distance between the two tensors, forward and for dW; the input gradient of the whole group is one GEMM
+// whose contraction runs over the outputs of all members, written once.
+std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws) {
+    const std::vector<size_t> sa = at(a).shape;
+    const size_t n = ws.size();
     const Storage da = compute_data(a);
-    const size_t o1 = push_tensor({M, N}, da.dtype, true), o2 = push_tensor({M, N}, da.dtype, true);
-    const ptrdiff_t odiff = (const char*)at(o2).data.ptr - (const char*)at(o1).data.ptr;
-    if (odiff % (ptrdiff_t)(8 * es) != 0) throw Error("matmul_pair: outputs are not 16-byte congruent");
-    check(eisen_hip_gemm_strided_batched(ctx_, da.ptr, w1.ptr, at(o1).data.ptr, da.dtype, da.dtype, 0, 0, 2, M, N, K, 0,
-                                         wdiff / (ptrdiff_t)es, odiff / (ptrdiff_t)es, 0), "matmul_pair");
+    bool ok = n >= 2 && n <= 3 && !sa.empty() && da.dtype == EISEN_BF16;
+    for (size_t i = 0; i < n && ok; i++)
+        ok = at(ws[i]).shape.size() == 2 && at(ws[i]).shape[0] == sa.back() && compute_data(ws[i]).dtype == da.dtype &&
+             std::count(ws.begin(), ws.end(), ws[i]) == 1;
+    if (!ok) {
+        std::vector<size_t> outs;
+        for (size_t w : ws) outs.push_back(matmul(a, w));
+        return outs;
+    }
+    const size_t K = sa.back(), M = numel_of(sa) / std::max<size_t>(K, 1);
+    std::vector<size_t> outs(n), N(n);
+    for (size_t i = 0; i < n; i++) {
+        N[i] = at(ws[i]).shape[1];
+        outs[i] = push_tensor({M, N[i]}, da.dtype, true);
+    }
+    // pair[i]: member i runs batched with member i+1
+    std::vector<char> pair(n, 0);
+    auto congruent = [](const void* p, const void* q, size_t elem) { return ((const char*)q - (const char*)p) % (ptrdiff_t)(8 * elem) == 0; };
+    for (size_t i = 0; i + 1 < n; i++)
+        if (!(i > 0 && pair[i - 1]) && at(ws[i]).shape == at(ws[i + 1]).shape &&
+            congruent(compute_data(ws[i]).ptr, compute_data(ws[i + 1]).ptr, 2) && congruent(at(outs[i]).data.ptr, at(outs[i + 1]).data.ptr, 2))
+            pair[i] = 1;
+    for (size_t i = 0; i < n; i++) {
+        const Storage w = compute_data(ws[i]);
+        if (pair[i]) {
+            const ptrdiff_t wd = ((const char*)compute_data(ws[i + 1]).ptr - (const char*)w.ptr) / 2;
+            const ptrdiff_t od = ((const char*)at(outs[i + 1]).data.ptr - (const char*)at(outs[i]).data.ptr) / 2;
+            check(eisen_hip_gemm_strided_batched(ctx_, da.ptr, w.ptr, at(outs[i]).data.ptr, da.dtype, da.dtype, 0, 0, 2, M, N[i], K, 0, wd, od, 0), "matmul_group");
+            i++;
+        } else {
+            check(eisen_hip_gemm(ctx_, da.ptr, w.ptr, at(outs[i]).data.ptr, da.dtype, da.dtype, 0, 0, M, N[i], K, 0), "matmul_group");
+        }
+    }
     auto epoch = std::make_shared<size_t>((size_t)-1);
     auto fn = [=](Graph& g) {
         if (*epoch == g.backward_epoch()) return;  // the node is on the tape once per output; it runs once per backward
         *epoch = g.backward_epoch();
-        const bool h1 = g.has_grad(o1), h2 = g.has_grad(o2);
-        // dA (+)= dY2 W2^T (+) dY1 W1^T: the later matmul first, as the reversed tape of two separate matmuls would
-        for (int which = 1; which >= 0; which--) {
-            if (!(which == 0 ? h1 : h2)) continue;
-            const Storage& go = g.grad_for_read(which == 0 ? o1 : o2);
+        std::vector<char> has(n);
+        bool all = true;
+        for (size_t i = 0; i < n; i++) {
+            has[i] = g.has_grad(outs[i]);
+            all = all && has[i];
+        }
+        // dA (+)= sum_i dY_i W_i^T, the last member first as the reversed tape of separate matmuls would
+        {
             int acc = 0;
             Storage& ga = g.grad_for_write(a, &acc);
-            g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(which == 0 ? b1 : b2).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc),
-                    "matmul_pair backward dA");
-        }
-        // dW1, dW2 (+)= A^T dY1, A^T dY2: one launch when both exist and are in the same accumulate state
-        const Storage xa = g.compute_data(a);
-        if (h1 && h2) {
-            const Storage& go1 = g.grad_for_read(o1);
-            const Storage& go2 = g.grad_for_read(o2);
-            int acc1 = 0, acc2 = 0;
-            Storage& g1 = g.grad_for_write(b1, &acc1);
-            Storage& g2 = g.grad_for_write(b2, &acc2);
-            const size_t gs = g1.dtype == EISEN_BF16 ? 2 : 4, os = go1.dtype == EISEN_BF16 ? 2 : 4;
-            const ptrdiff_t gd = (const char*)g2.ptr - (const char*)g1.ptr, od = (const char*)go2.ptr - (const char*)go1.ptr;
-            if (acc1 == acc2 && g1.dtype == g2.dtype && go1.dtype == go2.dtype && gd % (ptrdiff_t)16 == 0 && od % (ptrdiff_t)16 == 0) {
-                g.check(eisen_hip_gemm_strided_batched(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, 2, K, N, M, 0,
-                                                       od / (ptrdiff_t)os, gd / (ptrdiff_t)gs, acc1), "matmul_pair backward dW");
-            } else {
-                g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, K, N, M, acc1), "matmul_pair backward dW1");
-                g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go2.ptr, g2.ptr, go2.dtype, g2.dtype, 1, 0, K, N, M, acc2), "matmul_pair backward dW2");
+            const void* As[3];
+            const void* Bs[3];
+            size_t Ks[3];
+            size_t m = 0;
+            for (size_t i = n; i-- > 0;) {
+                if (!has[i]) continue;
+                As[m] = g.grad_for_read(outs[i]).ptr;
+                Bs[m] = g.compute_data(ws[i]).ptr;
+                Ks[m] = N[i];
+                m++;
             }
-        } else if (h1 || h2) {
-            const Storage& go = g.grad_for_read(h1 ? o1 : o2);
-            int acc = 0;
-            Storage& gb = g.grad_for_write(h1 ? b1 : b2, &acc);
-            g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul_pair backward dW");
+            if (m > 0)
+                g.check(eisen_hip_gemm_ksegments(g.ctx(), m, As, Bs, Ks, ga.ptr, EISEN_BF16, ga.dtype, 0, 1, M, K, acc), "matmul_group backward dA");
         }
+        // dW_i (+)= A^T dY_i, pairs as one launch when both halves exist and are in the same accumulate state
+        const Storage xa = g.compute_data(a);
+        for (size_t i = 0; i < n; i++) {
+            if (pair[i] && has[i] && has[i + 1]) {
+                const Storage& go1 = g.grad_for_read(outs[i]);
+                const Storage& go2 = g.grad_for_read(outs[i + 1]);
+                int acc1 = 0, acc2 = 0;
+                Storage& g1 = g.grad_for_write(ws[i], &acc1);
+                Storage& g2 = g.grad_for_write(ws[i + 1], &acc2);
+                const size_t gs = g1.dtype == EISEN_BF16 ? 2 : 4;
+                const ptrdiff_t gd = (const char*)g2.ptr - (const char*)g1.ptr, od = (const char*)go2.ptr - (const char*)go1.ptr;
+                if (acc1 == acc2 && g1.dtype == g2.dtype && gd % 16 == 0 && od % 16 == 0) {
+                    g.check(eisen_hip_gemm_strided_batched(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, 2, K, N[i], M, 0, od / 2,
+                                                           gd / (ptrdiff_t)gs, acc1), "matmul_group backward dW");
+                } else {
+                    g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, K, N[i], M, acc1), "matmul_group backward dW");
+                    g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go2.ptr, g2.ptr, go2.dtype, g2.dtype, 1, 0, K, N[i + 1], M, acc2), "matmul_group backward dW");
+                }
+                i++;
+            } else if (has[i]) {
+                const Storage& go = g.grad_for_read(outs[i]);
+                int acc = 0;
+                Storage& gb = g.grad_for_write(ws[i], &acc);
+                g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N[i], M, acc), "matmul_group backward dW");
+            }
+        }
+        (void)all;
     };
-    record({a, b1, b2}, o1, fn);
-    record({a, b1, b2}, o2, fn);
-    return {o1, o2};
+    for (size_t i = 0; i < n; i++) record(std::vector<size_t>(ws.begin(), ws.end()), outs[i], fn);
+    return outs;
 }
 
 // Graph::matmul_trans_b (src/graph/ops/linear.rs:301-523; GPU arm semantics): C = A B^T with

@@ -105,8 +105,8 @@ class Graph {
     size_t silu(size_t a);
     size_t swiglu(size_t gate, size_t up);                      // fused silu(gate) * up
     size_t matmul(size_t a, size_t b);
-    // two matmuls of the same input against two equally shaped weights, as one launch each way
-    std::pair<size_t, size_t> matmul_pair(size_t a, size_t b1, size_t b2);
+    // matmuls of one input against 2-3 weights with fewer launches (bf16 graphs; otherwise plain matmuls)
+    std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights);
     size_t matmul_bf16(size_t a, size_t b) { return matmul(a, b); }
     size_t matmul_trans_b(size_t a, size_t b);
     size_t bmm(size_t a, size_t b, bool trans_b);

@@ -88,17 +88,14 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
     const std::vector<size_t> xs = g.at(x_id).shape;
     if (xs.size() != 3) throw Error("GQA requires [Batch, Seq, Dim]");
     const size_t batch = xs[0], seq = xs[1];
-    const size_t q = q_proj.forward(g, x_id);
-    size_t k, v;
-    if (fused && !k_proj.has_bias && !v_proj.has_bias) {
-        // K and V projections read the same input and have the same shape: one launch for both
-        const std::pair<size_t, size_t> kv = g.matmul_pair(x_id, k_proj.weight_id, v_proj.weight_id);
-        k = kv.first;
-        v = kv.second;
-        const size_t kv_dim = g.at(k_proj.weight_id).shape[1];
-        g.reinterpret_shape(k, {batch, seq, kv_dim});
-        g.reinterpret_shape(v, {batch, seq, kv_dim});
+    size_t q, k, v;
+    if (fused && !q_proj.has_bias && !k_proj.has_bias && !v_proj.has_bias) {
+        // the three projections read the same input: K and V as one launch, one input-gradient GEMM for all
+        const std::vector<size_t> qkv = g.matmul_group(x_id, {q_proj.weight_id, k_proj.weight_id, v_proj.weight_id});
+        q = qkv[0]; k = qkv[1]; v = qkv[2];
+        for (size_t t : qkv) g.reinterpret_shape(t, {batch, seq, g.at(t).shape.back()});
     } else {
+        q = q_proj.forward(g, x_id);
         k = k_proj.forward(g, x_id);
         v = v_proj.forward(g, x_id);
     }
@@ -166,7 +163,8 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
     size_t gated;
     if (attn.fused && !ffn_gate.has_bias && !ffn1.has_bias) {
         // gate and up projections as one launch, then the fused SwiGLU
-        const std::pair<size_t, size_t> gu = g.matmul_pair(norm2_out, ffn_gate.weight_id, ffn1.weight_id);
+        const std::vector<size_t> guv = g.matmul_group(norm2_out, {ffn_gate.weight_id, ffn1.weight_id});
+        const std::pair<size_t, size_t> gu{guv[0], guv[1]};
         const std::vector<size_t> ns = g.at(norm2_out).shape;
         if (ns.size() == 3) {
             const size_t f = g.at(ffn_gate.weight_id).shape[1];

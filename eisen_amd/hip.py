@@ -264,6 +264,14 @@ class Context:
         self._call("eisen_hip_gemm_strided_batched", _ptr(A), _ptr(B), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(batch),
                    _sz(M), _sz(N), _sz(K), C.c_longlong(stride_a), C.c_longlong(stride_b), C.c_longlong(stride_c), _i(accumulate))
 
+    def gemm_ksegments(self, As, Bs, Ks, Cbuf, dtype_ab, dtype_c, trans_a, trans_b, M, N, accumulate=0):
+        """C (+)= sum_s op(A_s) op(B_s) over up to three (A, B, K) segments."""
+        n = len(Ks)
+        pa = (_vp * n)(*[_ptr(a) for a in As])
+        pb = (_vp * n)(*[_ptr(b) for b in Bs])
+        ks = (C.c_size_t * n)(*Ks)
+        self._call("eisen_hip_gemm_ksegments", _sz(n), pa, pb, ks, _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(M), _sz(N), _i(accumulate))
+
     # ---- attention --------------------------------------------------------------------
     @staticmethod
     def _strides(v):

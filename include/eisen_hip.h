@@ -208,6 +208,14 @@ int eisen_hip_gemm_strided_batched(eisen_ctx* ctx, const void* A, const void* B,
                                    int trans_b, size_t batch, size_t M, size_t N, size_t K, long long stride_a,
                                    long long stride_b, long long stride_c, int accumulate);
 
+/* C (+)= sum over up to three segments s of op(A_s) * op(B_s), each segment with its own operands and
+ * contraction length K_s (A_s is [M,K_s] or, transposed, [K_s,M]; B_s is [K_s,N] or [N,K_s]).  This is the
+ * input gradient of several linear layers that read the same tensor (dX = dQ Wq^T + dK Wk^T + dV Wv^T, which
+ * the reference accumulates with three matmul backward calls, src/graph/ops/linear.rs:266-277) as one launch
+ * and one write of dX.  Segments that are not multiples of 64 run as consecutive accumulating GEMMs. */
+int eisen_hip_gemm_ksegments(eisen_ctx* ctx, size_t n_segments, const void* const* A, const void* const* B, const size_t* K, void* C,
+                             int dtype_ab, int dtype_c, int trans_a, int trans_b, size_t M, size_t N, int accumulate);
+
 /* ---- attention ------------------------------------------------------------------------- */
 
 /* Causal grouped-query attention with saved log-sum-exp, and its backward.  Computes what

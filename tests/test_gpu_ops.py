@@ -558,6 +558,24 @@ def test_gemm_strided_batched_shared_operand(ctx):
         assert_close(got, 2 * (a.astype(np.float64).T @ go[i].astype(np.float64)), 1e-3, f"pair dW {i}")
 
 
+@pytest.mark.parametrize("Ks", [(128, 64, 64), (192, 64), (256,), (96, 64)])  # the last one is not slab-aligned: consecutive GEMMs
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_gemm_ksegments_input_gradient_of_a_group(ctx, Ks, accumulate):
+    # dX = sum_s dY_s W_s^T with dY_s [M, K_s] and W_s [N, K_s]: one contraction over the outputs of all members
+    M, N = 256, 128
+    dys = [prep(gen.normal(450 + i, (M, k)), BF16) for i, k in enumerate(Ks)]
+    wts = [prep(gen.normal(460 + i, (N, k)), BF16) for i, k in enumerate(Ks)]
+    c0 = prep(gen.normal(470, (M, N)), BF16)
+    exp = sum(d.astype(np.float64) @ w.astype(np.float64).T for d, w in zip(dys, wts)) + (c0 if accumulate else 0)
+    dA = [up(ctx, d, BF16) for d in dys]
+    dB = [up(ctx, w, BF16) for w in wts]
+    dc = up(ctx, c0, BF16)
+    ctx.gemm_ksegments(dA, dB, list(Ks), dc, BF16, BF16, 0, 1, M, N, accumulate)
+    assert_close(dn(ctx, dc, (M, N), BF16), exp, 2e-2, f"ksegments {Ks}")
+    for x in dA + dB + [dc]:
+        x.free()
+
+
 def test_gemm_f32_matches_oracle_order_tolerance(ctx):
     # config-1 sized linear against the sequential-order f32 oracle, rtol 1e-4
     a, b, go = gen.normal(410, (64, 64)), gen.normal(411, (64, 256), 0.02), gen.normal(412, (64, 256))
