@@ -39,6 +39,7 @@ struct GemmArgs {
     int lda, ldb, ldc;                 // leading dimensions in elements
     long long sA, sB, sC;              // batch strides in elements
     int accumulate;
+    const void* R;                     // optional residual with C's layout: C = R + A*B (accumulate must be 0)
     int split;                         // > 1: K is cut into this many parts; part p > 0 assigns into partial[p-1]
     int k_part;                        // contraction length of one part (a multiple of the slab)
     float* partial;                    // [batch][split-1][M][N] f32, summed into C by a second kernel
@@ -131,6 +132,9 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
     const bf16_t* A = static_cast<const bf16_t*>(g.A) + (long long)bz * g.sA;
     const bf16_t* B = static_cast<const bf16_t*>(g.B) + (long long)bz * g.sB;
     TC* C = static_cast<TC*>(g.C) + (long long)bz * g.sC;
+    // what the epilogue adds to the product: the old C (accumulate), a residual tensor, or nothing
+    const TC* Rsrc = g.R ? static_cast<const TC*>(g.R) + (long long)bz * g.sC : C;
+    const bool add_old = g.accumulate || g.R != nullptr;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -251,9 +255,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
                 } else {
                     TC* dst = C + (long long)m * g.ldc + n;
                     Pack<TC> o[8 / Pack<TC>::N];
-                    if (g.accumulate) {
+                    if (add_old) {
+                        const TC* src = Rsrc + (long long)m * g.ldc + n;
 #pragma unroll
-                        for (int k = 0; k < 8 / Pack<TC>::N; k++) o[k] = load_pack(dst + k * Pack<TC>::N);
+                        for (int k = 0; k < 8 / Pack<TC>::N; k++) o[k] = load_pack(src + k * Pack<TC>::N);
 #pragma unroll
                         for (int e = 0; e < 8; e++) val[e] += o[e / Pack<TC>::N].get(e % Pack<TC>::N);
                     }
@@ -281,7 +286,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
                         P[(long long)m * g.N + n] = val;
                     } else {
                         TC* dst = C + (long long)m * g.ldc + n;
-                        *dst = from_f32<TC>(g.accumulate ? to_f32(*dst) + val : val);
+                        *dst = from_f32<TC>(add_old ? to_f32(Rsrc[(long long)m * g.ldc + n]) + val : val);
                     }
                 }
             }
@@ -367,7 +372,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g, int trans
             const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
             if (m < g.M && n < g.N) {
                 TC* dst = C + (long long)m * g.ldc + n;
-                *dst = from_f32<TC>(g.accumulate ? to_f32(*dst) + acc[i][j] : acc[i][j]);
+                const TC* src = g.R ? static_cast<const TC*>(g.R) + (long long)blockIdx.z * g.sC + (long long)m * g.ldc + n : dst;
+                *dst = from_f32<TC>((g.accumulate || g.R) ? to_f32(*src) + acc[i][j] : acc[i][j]);
             }
         }
 }
@@ -410,7 +416,7 @@ struct KSegments {  // further (A, B, K) segments after the first one
 };
 static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
                        int trans_b, size_t M, size_t N, size_t K, size_t batch, long long sA, long long sB, long long sC,
-                       int accumulate, const char* who, const KSegments* segs = nullptr) {
+                       int accumulate, const char* who, const KSegments* segs = nullptr, const void* residual = nullptr) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, A && B && C, EISEN_E_ARG, "%s: null pointer", who);
     EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype_ab) && eisen_dtype_ok(dtype_c), EISEN_E_ARG, "%s: unknown dtype", who);
@@ -440,7 +446,8 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     g.ldc = (int)N;
     g.sA = sA; g.sB = sB; g.sC = sC;
     g.accumulate = accumulate;
-    g.vec_c = eisen_aligned(C, 16) && N % 8 == 0 && (sC * eisen_dtype_size(dtype_c)) % 16 == 0;
+    g.R = residual;
+    g.vec_c = (!residual || eisen_aligned(residual, 16)) && eisen_aligned(C, 16) && N % 8 == 0 && (sC * eisen_dtype_size(dtype_c)) % 16 == 0;
     if (n_more > 0) {
         size_t end = K;
         for (int i = 0; i < n_more; i++) {
@@ -565,4 +572,15 @@ extern "C" int eisen_hip_gemm_ksegments(eisen_ctx* ctx, size_t n_segments, const
         more.K[i] = K[i + 1];
     }
     return gemm_common(ctx, A[0], B[0], C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K[0], 1, 0, 0, 0, accumulate, "eisen_hip_gemm_ksegments", &more);
+}
+
+extern "C" int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void* B, const void* R, void* C, int dtype_ab, int dtype_c,
+                                       int trans_a, int trans_b, size_t M, size_t N, size_t K) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, R != nullptr, EISEN_E_ARG, "eisen_hip_gemm_residual: null residual");
+    if (K == 0) {  // C = R
+        if (R != C && M * N > 0) return eisen_hip_dtod(ctx, C, R, M * N * eisen_dtype_size(dtype_c));
+        return 0;
+    }
+    return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, 1, 0, 0, 0, 0, "eisen_hip_gemm_residual", nullptr, R);
 }

@@ -377,6 +377,32 @@ size_t Graph::matmul(size_t a, size_t b) {
     return out;
 }
 
+// Graph::matmul followed by Graph::add of a residual (src/nn/transformer.rs:36, :47) as one kernel:
+// out = r + a b, with r and out [.., N].  Backward is that of the two ops: dR += dOut, dA += dOut B^T,
+// dB += A^T dOut.
+size_t Graph::matmul_residual(size_t a, size_t b, size_t r) {
+    const std::vector<size_t> sa = at(a).shape, sb = at(b).shape, sr = at(r).shape;
+    if (sb.size() != 2 || sa.empty() || sr.empty()) throw Error("matmul_residual: expects a [..,K], b [K,N], r [..,N]");
+    const size_t K = sa.back(), M = numel_of(sa) / std::max<size_t>(K, 1), N = sb[1];
+    if (sb[0] != K || sr.back() != N || numel_of(sr) != M * N) throw Error("matmul_residual: shapes do not match: " + shape_str(sa) + " x " + shape_str(sb) + " + " + shape_str(sr));
+    const Storage da = compute_data(a), db = compute_data(b), dr = compute_data(r);
+    if (da.dtype != db.dtype || dr.dtype != da.dtype) throw Error("matmul_residual: operands have different element types");
+    const size_t out = push_tensor(sr, da.dtype, true);
+    check(eisen_hip_gemm_residual(ctx_, da.ptr, db.ptr, dr.ptr, at(out).data.ptr, da.dtype, da.dtype, 0, 0, M, N, K), "matmul_residual");
+    record({a, b, r}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Storage& gr = g.grad_for_write(r, &acc);
+        if (gr.dtype != go.dtype) throw Error("matmul_residual backward: gradient element types differ");
+        g.check(eisen_hip_accumulate(g.ctx(), gr.ptr, go.ptr, go.dtype, M * N, acc), "matmul_residual backward dR");
+        Storage& ga = g.grad_for_write(a, &acc);
+        g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc), "matmul_residual backward dA");
+        Storage& gb = g.grad_for_write(b, &acc);
+        g.check(eisen_hip_gemm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul_residual backward dB");
+    });
+    return out;
+}
+
 // Several Graph::matmul calls that share their left operand (Q/K/V projections, gate and up projections:
 // src/nn/attention.rs:300-302, src/nn/transformer.rs:41-44), with the results of the separate matmuls but
 // fewer launches: equally shaped neighbours (K and V, gate and up) run as a batch of two whose "stride" is the

@@ -84,7 +84,7 @@ GroupedQueryAttention::GroupedQueryAttention(Graph& g, size_t hidden, size_t hea
 }
 
 // GroupedQueryAttention::forward_with_mask (src/nn/attention.rs:289-388).
-size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool causal) const {
+size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool causal, size_t residual) const {
     const std::vector<size_t> xs = g.at(x_id).shape;
     if (xs.size() != 3) throw Error("GQA requires [Batch, Seq, Dim]");
     const size_t batch = xs[0], seq = xs[1];
@@ -104,6 +104,7 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
     if (fused) {
         // one op for steps 3-11: head split, GQA repeat, scores, scale, mask, softmax, P V, merge
         const size_t ctx = g.attention_gqa(q_rope, k_rope, v, num_heads, num_kv_heads, scale, causal);
+        if (residual != (size_t)-1 && !out_proj.has_bias) return g.matmul_residual(ctx, out_proj.weight_id, residual);
         return out_proj.forward(g, ctx);
     }
     const size_t q4 = g.reshape(q_rope, {batch, seq, num_heads, head_dim});
@@ -157,8 +158,13 @@ TransformerBlock::TransformerBlock(Graph& g, size_t hidden, size_t heads, size_t
 // TransformerBlock::forward_with_mask (src/nn/transformer.rs:31-49).
 size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) const {
     const size_t norm1_out = norm1.forward(g, x_id);
-    const size_t attn_out = attn.forward_with_mask(g, norm1_out, causal);
-    const size_t res1 = g.add(x_id, attn_out);
+    size_t res1;
+    if (attn.fused && !attn.out_proj.has_bias) {
+        res1 = attn.forward_with_mask(g, norm1_out, causal, x_id);  // the output projection adds the residual itself
+    } else {
+        const size_t attn_out = attn.forward_with_mask(g, norm1_out, causal);
+        res1 = g.add(x_id, attn_out);
+    }
     const size_t norm2_out = norm2.forward(g, res1);
     size_t gated;
     if (attn.fused && !ffn_gate.has_bias && !ffn1.has_bias) {
@@ -182,6 +188,7 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
         const size_t up = ffn1.forward(g, norm2_out);
         gated = g.mul(gate, up);
     }
+    if (attn.fused && !ffn2.has_bias) return g.matmul_residual(gated, ffn2.weight_id, res1);  // down projection + residual
     const size_t ffn2_out = ffn2.forward(g, gated);
     return g.add(res1, ffn2_out);
 }

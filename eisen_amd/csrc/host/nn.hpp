@@ -55,7 +55,9 @@ struct GroupedQueryAttention : Module {
     bool fused = true;
     GroupedQueryAttention() = default;
     GroupedQueryAttention(Graph& g, size_t hidden_dim, size_t num_heads, size_t num_kv_heads);
-    size_t forward_with_mask(Graph& g, size_t x_id, bool causal) const;
+    // residual != npos (fused path only): the output projection also adds this tensor, i.e. the result is
+    // residual + attention(x) as the transformer block computes it
+    size_t forward_with_mask(Graph& g, size_t x_id, bool causal, size_t residual = (size_t)-1) const;
     size_t forward(Graph& g, size_t x_id) const override { return forward_with_mask(g, x_id, true); }
     std::vector<size_t> params() const override;
 };

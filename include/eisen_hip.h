@@ -208,6 +208,11 @@ int eisen_hip_gemm_strided_batched(eisen_ctx* ctx, const void* A, const void* B,
                                    int trans_b, size_t batch, size_t M, size_t N, size_t K, long long stride_a,
                                    long long stride_b, long long stride_c, int accumulate);
 
+/* C = R + op(A) * op(B), R with C's shape and element type (R may be C).  A linear layer followed by the
+ * residual add of the transformer block (src/nn/transformer.rs:36, :47: `g.add(x_id, attn_out)`,
+ * `g.add(res1_out, ffn2_out)`) as one kernel: the product is added to the residual in f32 and rounded once. */
+int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void* B, const void* R, void* C, int dtype_ab, int dtype_c,
+                            int trans_a, int trans_b, size_t M, size_t N, size_t K);
 /* C (+)= sum over up to three segments s of op(A_s) * op(B_s), each segment with its own operands and
  * contraction length K_s (A_s is [M,K_s] or, transposed, [K_s,M]; B_s is [K_s,N] or [N,K_s]).  This is the
  * input gradient of several linear layers that read the same tensor (dX = dQ Wq^T + dK Wk^T + dV Wv^T, which

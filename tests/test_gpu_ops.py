@@ -576,6 +576,22 @@ def test_gemm_ksegments_input_gradient_of_a_group(ctx, Ks, accumulate):
         x.free()
 
 
+@pytest.mark.parametrize("M,N,K,dtype", [(256, 128, 192, BF16), (512, 384, 1024, BF16), (4096, 2048, 512, BF16), (200, 72, 40, BF16), (64, 48, 32, F32)])
+def test_gemm_residual(ctx, M, N, K, dtype):
+    # a linear layer and the residual add after it as one kernel: C = R + A B, rounded once
+    a, b, r = prep(gen.normal(480, (M, K)), dtype), prep(gen.normal(481, (K, N)), dtype), prep(gen.normal(482, (M, N)), dtype)
+    exp = r.astype(np.float64) + a.astype(np.float64) @ b.astype(np.float64)
+    da, db, dr = up(ctx, a, dtype), up(ctx, b, dtype), up(ctx, r, dtype)
+    dc = ctx.malloc(M * N * 4)
+    ctx.gemm_residual(da, db, dr, dc, dtype, dtype, 0, 0, M, N, K)
+    assert_close(dn(ctx, dc, (M, N), dtype), exp, 2e-2 if dtype == BF16 else 2e-4, "gemm_residual")
+    assert np.array_equal(dn(ctx, dr, (M, N), dtype), r)          # the residual itself is left alone
+    ctx.gemm_residual(da, db, dr, dr, dtype, dtype, 0, 0, M, N, K)  # in place: R may be C
+    assert_close(dn(ctx, dr, (M, N), dtype), exp, 2e-2 if dtype == BF16 else 2e-4, "gemm_residual in place")
+    for x in (da, db, dr, dc):
+        x.free()
+
+
 def test_gemm_f32_matches_oracle_order_tolerance(ctx):
     # config-1 sized linear against the sequential-order f32 oracle, rtol 1e-4
     a, b, go = gen.normal(410, (64, 64)), gen.normal(411, (64, 256), 0.02), gen.normal(412, (64, 256))
