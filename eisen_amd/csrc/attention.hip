@@ -114,6 +114,70 @@ struct TilePrefetch {
     }
 };
 
+// ---- tiles loaded straight into LDS ----------------------------------------------------------
+// global_load_lds_dwordx4 writes the 64 lanes' 16-byte chunks to 1 KB of consecutive LDS, so a tile
+// loaded this way has unpadded rows of HD bf16.  Bank conflicts are avoided by permuting the chunks
+// of a row instead: chunk cc of row r sits at chunk position cc ^ tile_swz(r).  The permutation is
+// chosen so that both access patterns of the kernels are conflict-free: 8 consecutive rows at one
+// chunk position (MFMA operand rows, 16-byte reads) and 4 consecutive rows x 32 bytes (the
+// transposing 8-byte reads).
+template <int HD>
+__device__ __forceinline__ int tile_swz(int row) {
+    return HD >= 64 ? (((row & 3) << 1) | ((row >> 2) & 1)) : ((row & 2) | ((row >> 2) & 1));
+}
+template <int HD>
+__device__ __forceinline__ int tile_at(int row, int col) {
+    return row * HD + ((((col >> 3) ^ tile_swz<HD>(row)) << 3) | (col & 7));
+}
+// lds_tr_operand for a swizzled tile (the two reads are 8 rows apart: same permutation)
+template <int HD>
+__device__ __forceinline__ bf16x8 lds_tr_operand_swz(const bf16_t* tile, int row0, int col0, int t, int lane) {
+    const int g = lane >> 5, L = lane & 15, half = (lane >> 4) & 1;
+    const bf16_t* p = tile + tile_at<HD>(row0 + 16 * t + 4 * g + (L >> 2), col0 + 16 * half + 4 * (L & 3));
+    return concat4(lds_read_tr(p), lds_read_tr(p + 8 * HD));
+}
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef __attribute__((address_space(1))) const void* global_void_ptr;
+
+// A ROWS x HD bf16 tile of a strided global tensor, loaded into a swizzled LDS tile by WAVES waves with
+// no registers in between.  Each wave instruction moves 1 KB (512 / HD rows).  Rows past `limit_rows`
+// re-read the last valid row: the kernels mask or zero-weight them, they only have to be finite.
+// The loads are asynchronous: wait_direct_loads() before the barrier that publishes the tile.
+template <int HD, int ROWS, int WAVES>
+struct DirectTile {
+    static constexpr int CPR = HD / 8, RPB = 64 / CPR, BLOCKS = ROWS / RPB, PER_WAVE = BLOCKS / WAVES;
+    static_assert(ROWS % RPB == 0 && BLOCKS % WAVES == 0, "tile does not split into whole wave loads");
+    unsigned off[PER_WAVE];  // byte offset of this lane's chunk from the tile's first row (loop-invariant)
+    __device__ __forceinline__ static int lane_row(int wave, int i, int lane) { return (wave * PER_WAVE + i) * RPB + lane / CPR; }
+    __device__ __forceinline__ static int lane_chunk(int row, int lane) { return (lane % CPR) ^ tile_swz<HD>(row); }
+    __device__ __forceinline__ void init(long long row_stride, int wave, int lane) {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) {
+            const int row = lane_row(wave, i, lane);
+            off[i] = (unsigned)((row * row_stride + lane_chunk(row, lane) * 8) * 2);
+        }
+    }
+    __device__ __forceinline__ void load(const bf16_t* src, long long row_stride, int first_row, int limit_rows, bf16_t* lds_tile,
+                                         int wave, int lane) const {
+        if (first_row + ROWS <= limit_rows) {  // whole tile in range (uniform)
+            const char* base = reinterpret_cast<const char*>(src + (long long)first_row * row_stride);
+#pragma unroll
+            for (int i = 0; i < PER_WAVE; i++)
+                __builtin_amdgcn_global_load_lds((global_void_ptr)(base + off[i]), (lds_void_ptr)(lds_tile + (wave * PER_WAVE + i) * 512), 16, 0, 0);
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) {
+            const int row = lane_row(wave, i, lane);
+            const int gr = min(first_row + row, limit_rows - 1);
+            __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (long long)gr * row_stride + lane_chunk(row, lane) * 8),
+                                             (lds_void_ptr)(lds_tile + (wave * PER_WAVE + i) * 512), 16, 0, 0);
+        }
+    }
+};
+__device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // ---- forward -------------------------------------------------------------------------------
 // Grid of the two query-stationary kernels: one block per (pair of query blocks, GW query heads of a
 // KV head, batch), pair index fastest.  A block runs query block `pair` and then its mirror image
@@ -139,9 +203,9 @@ __device__ __forceinline__ QBlock decode_qblock(const AttnArgs& a) {
 
 template <int HD, int GW>
 __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
-    constexpr int QS = 4 / GW, BKV = 64, PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
-    __shared__ __attribute__((aligned(16))) bf16_t Ksb[2][BKV * PITCH];
-    __shared__ __attribute__((aligned(16))) bf16_t Vsb[2][BKV * PITCH];
+    constexpr int QS = 4 / GW, BKV = 64, KSTEPS = HD / 16, DT = HD / 32;
+    __shared__ __attribute__((aligned(1024))) bf16_t Ksb[2][BKV * HD];  // swizzled tiles, see DirectTile
+    __shared__ __attribute__((aligned(1024))) bf16_t Vsb[2][BKV * HD];
     const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hsub = wave % GW, qsub = wave / GW;
@@ -151,6 +215,8 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
     const bf16_t* Kp = static_cast<const bf16_t*>(a.K) + b * a.k_sb + kvh * a.k_sh;
     const bf16_t* Vp = static_cast<const bf16_t*>(a.V) + b * a.k_sb + kvh * a.k_sh;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    DirectTile<HD, BKV, 4> kv_tile;
+    kv_tile.init(a.k_ss, wave, lane);
 
     for (int pass = 0; pass < 2; pass++) {
         const int qblk = pass == 0 ? blk.n_qblk - 1 - blk.pair : blk.pair;  // the long one first
@@ -176,21 +242,19 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
         const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
         const int my_qmax = q0 < a.S ? q0 + 31 : -1;
 
-        TilePrefetch<HD, BKV, 256> pk, pv;
-        pk.fetch(Kp, a.k_ss, 0, a.S);
-        pv.fetch(Vp, a.k_ss, 0, a.S);
+        kv_tile.load(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
+        kv_tile.load(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
         // One 64-key tile.  MASKED is a compile-time flag: the tiles entirely below the diagonal and inside
         // the sequence run a loop body with no mask code and no branches at all.
         auto tile = [&](int kt, auto masked_c) {
             constexpr bool MASKED = decltype(masked_c)::value;
             const bf16_t* Ks = Ksb[kt & 1];
             const bf16_t* Vs = Vsb[kt & 1];
-            pk.commit(Ksb[kt & 1]);
-            pv.commit(Vsb[kt & 1]);
-            __syncthreads();  // one barrier per tile: the other buffer is only rewritten after the next barrier
+            wait_direct_loads();  // this wave's part of tile kt has landed
+            __syncthreads();      // one barrier per tile: every wave is done with tile kt-1, whose buffer the next loads overwrite
             if (kt + 1 < n_kt) {
-                pk.fetch(Kp, a.k_ss, (kt + 1) * BKV, a.S);
-                pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
+                kv_tile.load(Kp, a.k_ss, (kt + 1) * BKV, a.S, Ksb[(kt + 1) & 1], wave, lane);
+                kv_tile.load(Vp, a.k_ss, (kt + 1) * BKV, a.S, Vsb[(kt + 1) & 1], wave, lane);
             }
             const int k0 = kt * BKV;
             if (my_qmax < 0 || (a.causal && k0 > my_qmax)) return;                // wave-uniform
@@ -203,7 +267,7 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                 if (sub == 0 || two) {
 #pragma unroll
                     for (int st = 0; st < KSTEPS; st++) {
-                        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
+                        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + tile_at<HD>(sub * 32 + c, st * 16 + 8 * g));
                         s[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s[sub], 0, 0, 0);
                     }
                 }
@@ -253,7 +317,7 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                     for (int t = 0; t < 2; t++) {
-                        const bf16x8 vt = lds_tr_operand(Vs, PITCH, sub * 32, dt * 32, t, lane);
+                        const bf16x8 vt = lds_tr_operand_swz<HD>(Vs, sub * 32, dt * 32, t, lane);
                         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vt, pf[t], o[dt], 0, 0, 0);
                     }
             }
@@ -283,9 +347,9 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
 // ---- backward: dQ (query-stationary); also writes D = rowsum(dO o O) for the dK/dV pass ------
 template <int HD, int GW>
 __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
-    constexpr int QS = 4 / GW, BKV = 64, PITCH = HD + 8, KSTEPS = HD / 16, DT = HD / 32;
-    __shared__ __attribute__((aligned(16))) bf16_t Ksb[2][BKV * PITCH];
-    __shared__ __attribute__((aligned(16))) bf16_t Vsb[2][BKV * PITCH];
+    constexpr int QS = 4 / GW, BKV = 64, KSTEPS = HD / 16, DT = HD / 32;
+    __shared__ __attribute__((aligned(1024))) bf16_t Ksb[2][BKV * HD];  // swizzled tiles, see DirectTile
+    __shared__ __attribute__((aligned(1024))) bf16_t Vsb[2][BKV * HD];
     const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hsub = wave % GW, qsub = wave / GW;
@@ -294,6 +358,8 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
     const bf16_t* Kp = static_cast<const bf16_t*>(a.K) + b * a.k_sb + kvh * a.k_sh;
     const bf16_t* Vp = static_cast<const bf16_t*>(a.V) + b * a.k_sb + kvh * a.k_sh;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    DirectTile<HD, BKV, 4> kv_tile;
+    kv_tile.init(a.k_ss, wave, lane);
 
     for (int pass = 0; pass < 2; pass++) {
         const int qblk = pass == 0 ? blk.n_qblk - 1 - blk.pair : blk.pair;
@@ -329,19 +395,17 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
         const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
         const int my_qmax = q0 < a.S ? q0 + 31 : -1;
 
-        TilePrefetch<HD, BKV, 256> pk, pv;
-        pk.fetch(Kp, a.k_ss, 0, a.S);
-        pv.fetch(Vp, a.k_ss, 0, a.S);
+        kv_tile.load(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
+        kv_tile.load(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
         auto tile = [&](int kt, auto masked_c) {
             constexpr bool MASKED = decltype(masked_c)::value;  // false: no key of the tile is masked for this wave
             const bf16_t* Ks = Ksb[kt & 1];
             const bf16_t* Vs = Vsb[kt & 1];
-            pk.commit(Ksb[kt & 1]);
-            pv.commit(Vsb[kt & 1]);
-            __syncthreads();
+            wait_direct_loads();  // this wave's part of tile kt has landed
+            __syncthreads();      // every wave is done with tile kt-1, whose buffer the next loads overwrite
             if (kt + 1 < n_kt) {
-                pk.fetch(Kp, a.k_ss, (kt + 1) * BKV, a.S);
-                pv.fetch(Vp, a.k_ss, (kt + 1) * BKV, a.S);
+                kv_tile.load(Kp, a.k_ss, (kt + 1) * BKV, a.S, Ksb[(kt + 1) & 1], wave, lane);
+                kv_tile.load(Vp, a.k_ss, (kt + 1) * BKV, a.S, Vsb[(kt + 1) & 1], wave, lane);
             }
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
@@ -352,19 +416,19 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                 for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
 #pragma unroll
                 for (int st = 0; st < KSTEPS; st++) {
-                    const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
-                    const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + (sub * 32 + c) * PITCH + st * 16 + 8 * g);
+                    const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + tile_at<HD>(sub * 32 + c, st * 16 + 8 * g));
+                    const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + tile_at<HD>(sub * 32 + c, st * 16 + 8 * g));
                     s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
                     dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[st], dp, 0, 0, 0);
                 }
                 bf16x8 dsf[2];
-                // a query past the end has LSE = +inf and a key past the end a zero K row, so only
-                // the causal diagonal needs a mask
+                // a query past the end has LSE = +inf; keys past the end (their tile rows repeat the last
+                // key) and keys above the causal diagonal are masked
                 float p[16];
 #pragma unroll
                 for (int v = 0; v < 16; v++) p[v] = fast_exp2(fmaf(s[v], a.scale_log2e, -lse2));
-                if (MASKED && a.causal && k0 + 31 > q0) {
-                    const int rel = q - k0;       // keys k0 + row > q are masked
+                if (MASKED && ((a.causal && k0 + 31 > q0) || k0 + 32 > a.S)) {
+                    const int rel = min(a.causal ? q : a.S - 1, a.S - 1) - k0;  // keys k0 + row > rel are masked
 #pragma unroll
                     for (int v = 0; v < 16; v++)
                         if (acc_row(v, g) > rel) p[v] = 0.f;
@@ -375,7 +439,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                     for (int t = 0; t < 2; t++) {
-                        const bf16x8 ktr = lds_tr_operand(Ks, PITCH, sub * 32, dt * 32, t, lane);
+                        const bf16x8 ktr = lds_tr_operand_swz<HD>(Ks, sub * 32, dt * 32, t, lane);
                         dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsf[t], dq[dt], 0, 0, 0);
                     }
             }

@@ -492,7 +492,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         const bool t128 = M >= 128 && N >= 128;
         const long long tiles = t128 ? tiles128 : (long long)eisen_ceil_div(M, 64) * eisen_ceil_div(N, 64) * batch;
         const size_t slab = t128 ? 64 : 32, min_part = t128 ? 512 : 256;
-        if (tiles < 128)
+        if (tiles <= 128)
             while (split < 32 && tiles * split * 2 <= 256 && K / (split * 2) >= min_part && K % (split * 2 * slab) == 0) split *= 2;
     }
     const bool split128 = split > 1 && M >= 128 && N >= 128;

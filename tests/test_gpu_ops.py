@@ -701,6 +701,9 @@ def test_attention_bf16_mfma(ctx, B, S, Hq, Hkv, hd):
 def test_attention_bf16_layout_bhsd_and_non_causal(ctx):
     _attn_case(ctx, BF16, 2, 96, 8, 2, 64, layout="bhsd")
     _attn_case(ctx, BF16, 1, 70, 4, 2, 64, causal=False)
+    # keys past the end of a ragged last tile, for the other two head sizes' LDS tile layouts
+    _attn_case(ctx, BF16, 1, 200, 4, 2, 32, causal=False)
+    _attn_case(ctx, BF16, 1, 70, 2, 1, 128, causal=False)
 
 
 def test_attention_config3_full_size_properties(ctx):
