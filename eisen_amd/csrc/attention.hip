@@ -115,26 +115,19 @@ struct TilePrefetch {
 };
 
 // ---- tiles loaded straight into LDS ----------------------------------------------------------
-// global_load_lds_dwordx4 writes the 64 lanes' 16-byte chunks to 1 KB of consecutive LDS, so a tile
-// loaded this way has unpadded rows of HD bf16.  Bank conflicts are avoided by permuting the chunks
-// of a row instead: chunk cc of row r sits at chunk position cc ^ tile_swz(r).  The permutation is
-// chosen so that both access patterns of the kernels are conflict-free: 8 consecutive rows at one
-// chunk position (MFMA operand rows, 16-byte reads) and 4 consecutive rows x 32 bytes (the
-// transposing 8-byte reads).
+// Unpadded rows of HD bf16 with permuted chunks (lds_swz in device_utils.cuh).
 template <int HD>
-__device__ __forceinline__ int tile_swz(int row) {
-    return HD >= 64 ? (((row & 3) << 1) | ((row >> 2) & 1)) : ((row & 2) | ((row >> 2) & 1));
-}
+__device__ __forceinline__ int tile_swz(int row) { return lds_swz<HD * 2>(row); }
 template <int HD>
 __device__ __forceinline__ int tile_at(int row, int col) {
     return row * HD + ((((col >> 3) ^ tile_swz<HD>(row)) << 3) | (col & 7));
 }
-// lds_tr_operand for a swizzled tile (the two reads are 8 rows apart: same permutation)
+// lds_tr_operand for a swizzled tile
 template <int HD>
 __device__ __forceinline__ bf16x8 lds_tr_operand_swz(const bf16_t* tile, int row0, int col0, int t, int lane) {
     const int g = lane >> 5, L = lane & 15, half = (lane >> 4) & 1;
-    const bf16_t* p = tile + tile_at<HD>(row0 + 16 * t + 4 * g + (L >> 2), col0 + 16 * half + 4 * (L & 3));
-    return concat4(lds_read_tr(p), lds_read_tr(p + 8 * HD));
+    const int row = row0 + 16 * t + 4 * g + (L >> 2), col = col0 + 16 * half + 4 * (L & 3);
+    return concat4(lds_read_tr(tile + tile_at<HD>(row, col)), lds_read_tr(tile + tile_at<HD>(row + 8, col)));
 }
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;

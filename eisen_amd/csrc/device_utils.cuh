@@ -82,3 +82,18 @@ template <int THREADS> __device__ __forceinline__ float block_max(float v, float
     for (int i = 0; i < W; i++) r = fmaxf(r, smem[i]);
     return r;
 }
+
+// ---- LDS tiles filled by direct-to-LDS loads -------------------------------------------------------
+// global_load_lds_dwordx4 writes the 64 lanes' 16-byte chunks to 1 KB of consecutive LDS, so such a tile has
+// unpadded rows; bank conflicts are avoided by permuting the chunks of a row instead: chunk cc of row r sits at
+// chunk position cc ^ lds_swz<row bytes>(r).  With 64 banks of 4 bytes (a 256-byte bank span) the permutation
+// makes both MFMA operand read patterns conflict-free: 16 consecutive rows at one chunk position fall into 16
+// different 16-byte slots of the span (16-byte reads of a k-contiguous operand), and 4 consecutive rows x 64
+// bytes into 4 different 64-byte slots (the transposing 8-byte reads).
+template <int ROW_BYTES>
+__device__ __forceinline__ int lds_swz(int row) {
+    static_assert(ROW_BYTES == 64 || ROW_BYTES == 128 || ROW_BYTES == 256 || ROW_BYTES == 512, "LDS row length not covered");
+    if (ROW_BYTES == 64) return (row >> 2) & 3;                                                          // four rows per bank span
+    if (ROW_BYTES == 128) return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);  // two rows per bank span
+    return ((row & 3) << 2) | ((row >> 2) & 3);                                                          // a row is one or two bank spans
+}

@@ -5,13 +5,15 @@
 //   dW       dB = A^T * dC       (A stored [K',M'], B [K',N'])  src/graph/ops/linear.rs:279-287
 //   tied lm_head / bmm with trans_b                             src/graph/ops/linear.rs:456-481, :1430-1446
 //
-// bf16 path: MFMA v_mfma_f32_32x32x16_bf16, f32 accumulate.  A workgroup of 4 waves owns a
-// BM x BN tile of C; each wave owns a (BM/2) x (BN/2) quadrant made of 32x32 MFMA tiles.  K is walked in slabs of
-// 32 through double-buffered LDS (one barrier per slab) with the next slab's global loads in
-// flight during the current slab's MFMAs.  The MFMA operand registers want 8 consecutive k per
-// lane: a k-contiguous operand gets them with one ds_read_b128, an operand stored the other
-// way round with two ds_read_b64_tr_b16 (LDS transpose reads), so dX, dW and the forward GEMM
-// all stream their operands through LDS as plain 16-byte copies.
+// bf16 path: MFMA v_mfma_f32_32x32x16_bf16, f32 accumulate.  A workgroup of 4 or 8 waves owns a
+// BM x BN tile of C; each wave owns a 64x64 part of it made of 32x32 MFMA tiles.  K is walked in slabs of
+// 64 (32 for odd K) through LDS, one barrier per slab, with the following slabs' global loads in flight during
+// the current slab's MFMAs.  Two kernels: gemm_mfma_direct_kernel loads its operands straight into three LDS
+// stages (whole-tile shapes, 256x128 tile); gemm_mfma_kernel stages them through registers into two LDS
+// buffers and handles edges.  The MFMA operand registers want 8 consecutive k per lane: a k-contiguous
+// operand gets them with one ds_read_b128, an operand stored the other way round with two
+// ds_read_b64_tr_b16 (LDS transpose reads), so dX, dW and the forward GEMM all stream their operands through
+// LDS as plain 16-byte copies.
 //
 // f32 path and odd shapes: a plain LDS-tiled FMA kernel (64x64 tile, 4x4 per thread).
 #include <utility>
@@ -110,6 +112,88 @@ struct OperandTile {
         return r;
     }
 };
+
+// Epilogue shared by the MFMA kernels.  Accumulator register v of lane l holds
+// C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.  `lds_f32` is the operand LDS (LDS_BYTES bytes), idle by now
+// and used as a staging area.
+template <int BM, int BN, int WGM, int WGN, bool EDGE, size_t LDS_BYTES, typename TC>
+__device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], float* lds_f32, TC* C,
+                                                const TC* Rsrc, bool add_old, int bz, int split, int part, int m0, int n0, int wave,
+                                                int wm, int wn, int lane) {
+    constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+    float* P = part > 0 ? g.partial + ((long long)bz * (split - 1) + (part - 1)) * g.M * g.N : nullptr;
+    constexpr int SP = WN + 4;  // staging pitch in floats
+    constexpr bool kCanStage = LDS_BYTES >= (size_t)WGM * WGN * 32 * SP * sizeof(float);
+    if (kCanStage && !EDGE && g.vec_c) {
+        // Each wave turns its accumulators, one 32-row band at a time, through a private piece of the
+        // (now idle) operand LDS so that a lane ends up with 8 consecutive columns of one row: C leaves in
+        // 16-byte stores covering whole 128/256-byte row segments instead of 2- or 4-byte ones.
+        float* stage = lds_f32 + wave * (32 * SP);
+        constexpr int LPR = WN / 8, PASSES = 32 * LPR / 64;  // lanes per row, passes per band
+        static_assert(32 * LPR % 64 == 0, "band must split evenly over the wave");
+        const int c = lane & 31, gh = lane >> 5;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) stage[(8 * (v / 4) + 4 * gh + (v % 4)) * SP + j * 32 + c] = acc[i][j][v];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ps++) {
+                const int idx = ps * 64 + lane, r = idx / LPR, cg = idx % LPR;
+                const float4 lo = *reinterpret_cast<const float4*>(stage + r * SP + cg * 8);
+                const float4 hi = *reinterpret_cast<const float4*>(stage + r * SP + cg * 8 + 4);
+                float val[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                const int m = m0 + wm * WM + i * 32 + r, n = n0 + wn * WN + cg * 8;
+                if (P) {
+                    float* dst = P + (long long)m * g.N + n;
+                    *reinterpret_cast<float4*>(dst) = lo;
+                    *reinterpret_cast<float4*>(dst + 4) = hi;
+                } else {
+                    TC* dst = C + (long long)m * g.ldc + n;
+                    Pack<TC> o[8 / Pack<TC>::N];
+                    if (add_old) {
+                        const TC* src = Rsrc + (long long)m * g.ldc + n;
+#pragma unroll
+                        for (int k = 0; k < 8 / Pack<TC>::N; k++) o[k] = load_pack(src + k * Pack<TC>::N);
+#pragma unroll
+                        for (int e = 0; e < 8; e++) val[e] += o[e / Pack<TC>::N].get(e % Pack<TC>::N);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; e++) o[e / Pack<TC>::N].set(e % Pack<TC>::N, val[e]);
+#pragma unroll
+                    for (int k = 0; k < 8 / Pack<TC>::N; k++) store_pack(dst + k * Pack<TC>::N, o[k]);
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WN + j * 32 + (lane & 31);
+            if (EDGE && n >= g.N) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (!EDGE || m < g.M) {
+                    const float val = acc[i][j][v];
+                    if (P) {
+                        P[(long long)m * g.N + n] = val;
+                    } else {
+                        TC* dst = C + (long long)m * g.ldc + n;
+                        *dst = from_f32<TC>(add_old ? to_f32(Rsrc[(long long)m * g.ldc + n]) + val : val);
+                    }
+                }
+            }
+        }
+}
 
 // WGM x WGN waves share a BM x BN tile of C.  EDGE = false is for shapes that are whole multiples
 // of the tile in M, N and K: no bounds checks anywhere.
@@ -218,79 +302,187 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_kernel(GemmArgs g) {
         __syncthreads();
     }
 
-    // epilogue: accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile
-    float* P = part > 0 ? g.partial + ((long long)bz * (split - 1) + (part - 1)) * g.M * g.N : nullptr;
-    constexpr int SP = WN + 4;  // staging pitch in floats
-    constexpr bool kCanStage = sizeof(lds) >= (size_t)WGM * WGN * 32 * SP * sizeof(float);
-    if (kCanStage && !EDGE && g.vec_c) {
-        // Each wave turns its accumulators, one 32-row band at a time, through a private piece of the
-        // (now idle) operand LDS so that a lane ends up with 8 consecutive columns of one row: C leaves in
-        // 16-byte stores covering whole 128/256-byte row segments instead of 2- or 4-byte ones.
-        float* stage = reinterpret_cast<float*>(&lds[0][0]) + wave * (32 * SP);
-        constexpr int LPR = WN / 8, PASSES = 32 * LPR / 64;  // lanes per row, passes per band
-        static_assert(32 * LPR % 64 == 0, "band must split evenly over the wave");
-        const int c = lane & 31, gh = lane >> 5;
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) stage[(8 * (v / 4) + 4 * gh + (v % 4)) * SP + j * 32 + c] = acc[i][j][v];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ps++) {
-                const int idx = ps * 64 + lane, r = idx / LPR, cg = idx % LPR;
-                const float4 lo = *reinterpret_cast<const float4*>(stage + r * SP + cg * 8);
-                const float4 hi = *reinterpret_cast<const float4*>(stage + r * SP + cg * 8 + 4);
-                float val[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-                const int m = m0 + wm * WM + i * 32 + r, n = n0 + wn * WN + cg * 8;
-                if (P) {
-                    float* dst = P + (long long)m * g.N + n;
-                    *reinterpret_cast<float4*>(dst) = lo;
-                    *reinterpret_cast<float4*>(dst + 4) = hi;
-                } else {
-                    TC* dst = C + (long long)m * g.ldc + n;
-                    Pack<TC> o[8 / Pack<TC>::N];
-                    if (add_old) {
-                        const TC* src = Rsrc + (long long)m * g.ldc + n;
-#pragma unroll
-                        for (int k = 0; k < 8 / Pack<TC>::N; k++) o[k] = load_pack(src + k * Pack<TC>::N);
-#pragma unroll
-                        for (int e = 0; e < 8; e++) val[e] += o[e / Pack<TC>::N].get(e % Pack<TC>::N);
-                    }
-#pragma unroll
-                    for (int e = 0; e < 8; e++) o[e / Pack<TC>::N].set(e % Pack<TC>::N, val[e]);
-#pragma unroll
-                    for (int k = 0; k < 8 / Pack<TC>::N; k++) store_pack(dst + k * Pack<TC>::N, o[k]);
-                }
-            }
-        }
-        return;
+    gemm_store_tile<BM, BN, WGM, WGN, EDGE, sizeof(lds), TC>(g, acc, reinterpret_cast<float*>(&lds[0][0]), C, Rsrc, add_old, bz, split, part,
+                                                             m0, n0, wave, wm, wn, lane);
+}
+
+// ---- MFMA kernel with operands loaded straight into LDS ------------------------------------------
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory into LDS without passing through
+// registers: no staging registers, no LDS store instructions, no address arithmetic per chunk.  One wave
+// instruction fills 1 KB of consecutive LDS, so the tiles are unpadded and their rows are chunk-permuted
+// (lds_swz in device_utils.cuh) to keep the operand reads free of bank conflicts.
+// Three LDS stages: slab kt is multiplied while slabs kt+1 and kt+2 are in flight, one barrier per slab.
+// The loads are issued from inline assembly so that waiting for them stays in this file's hands
+// (vmcnt counts them in issue order); the kernel has no other vector memory loads in its main loop.
+template <int ROWS, bool KC, int BK, int WAVES>
+struct DirectOperandTile {
+    static constexpr int LDS_ROW = KC ? BK : ROWS;  // elements of one LDS row = one contiguous run of the operand in memory
+    static constexpr int ELEMS = ROWS * BK;
+    static constexpr int CPR = LDS_ROW / 8;         // 16-byte chunks per LDS row
+    static constexpr int RPB = 64 / CPR;            // LDS rows filled by one wave instruction
+    static constexpr int LOADS = ELEMS / 512 / WAVES;  // wave instructions per wave and slab
+    static_assert(CPR >= 8 && 64 % CPR == 0 && ELEMS % (512 * WAVES) == 0, "slab must split into whole 1 KB wave loads");
+
+    // LDS row and (permuted) chunk this lane fetches in load i of its wave
+    static __device__ __forceinline__ void lane_chunk(int i, int wave, int lane, int& row, int& chunk) {
+        row = (wave * LOADS + i) * RPB + lane / CPR;
+        chunk = (lane % CPR) ^ lds_swz<LDS_ROW * 2>(row);
     }
+    static __device__ __forceinline__ int lds_block(int i, int wave) { return (wave * LOADS + i) * 512; }  // element offset in the tile
+
+    // MFMA operand of the 32 operand rows starting at `row0` for contraction offsets ks..ks+15 (same register
+    // contents as OperandTile::fragment)
+    static __device__ __forceinline__ bf16x8 fragment(const bf16_t* tile, int row0, int ks, int lane) {
+        if (KC) {
+            const int r = row0 + (lane & 31);
+            return *reinterpret_cast<const bf16x8*>(tile + r * BK + ((((ks >> 3) + (lane >> 5)) ^ lds_swz<BK * 2>(r)) << 3));
+        }
+        const int L = lane & 15, half = (lane >> 4) & 1;
+        const int k = ks + 8 * (lane >> 5) + (L >> 2), col = row0 + 16 * half + 4 * (L & 3);
+        const bf16_t* p_lo = tile + k * ROWS + ((((col >> 3) ^ lds_swz<ROWS * 2>(k)) << 3) | (col & 7));
+        const bf16_t* p_hi = tile + (k + 4) * ROWS + ((((col >> 3) ^ lds_swz<ROWS * 2>(k + 4)) << 3) | (col & 7));
+        const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p_lo));
+        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p_hi));
+        bf16x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    }
+};
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+// one wave instruction: lane l's 16 bytes at `src` land at lds_dst + 16*l (lds_dst is wave-uniform)
+__device__ __forceinline__ void load_to_lds_16(const void* src, bf16_t* lds_dst) {
+    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {  // until at most N of this wave's vector memory loads are outstanding
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// barrier without the memory fence of __syncthreads (which would wait for every outstanding load)
+__device__ __forceinline__ void barrier_no_fence() {
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_s_barrier();
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+
+// For shapes that are whole multiples of the tile in M, N and K (no bounds checks anywhere).
+template <int BM, int BN, int BK, int WGM, int WGN, bool A_KC, bool B_KC, typename TC>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmArgs g) {
+    constexpr int WAVES = WGM * WGN, STAGES = 3;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int KSTEPS = BK / 16;
+    using TA = DirectOperandTile<BM, A_KC, BK, WAVES>;
+    using TB = DirectOperandTile<BN, B_KC, BK, WAVES>;
+    constexpr int NLOADS = TA::LOADS + TB::LOADS;
+    __shared__ __attribute__((aligned(1024))) bf16_t lds[STAGES][TA::ELEMS + TB::ELEMS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int split = g.split > 1 ? g.split : 1;
+    const int bz = blockIdx.z / split, part = blockIdx.z % split;
+    const int k_lo = part * g.k_part, k_hi = split > 1 ? min(g.K, k_lo + g.k_part) : g.K;
+    const bf16_t* A = static_cast<const bf16_t*>(g.A) + (long long)bz * g.sA;
+    const bf16_t* B = static_cast<const bf16_t*>(g.B) + (long long)bz * g.sB;
+    TC* C = static_cast<TC*>(g.C) + (long long)bz * g.sC;
+    const TC* Rsrc = g.R ? static_cast<const TC*>(g.R) + (long long)bz * g.sC : C;
+    const bool add_old = g.accumulate || g.R != nullptr;
+
+    f32x16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int n = n0 + wn * WN + j * 32 + (lane & 31);
-            if (EDGE && n >= g.N) continue;
+        for (int j = 0; j < TN; j++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                if (!EDGE || m < g.M) {
-                    const float val = acc[i][j][v];
-                    if (P) {
-                        P[(long long)m * g.N + n] = val;
-                    } else {
-                        TC* dst = C + (long long)m * g.ldc + n;
-                        *dst = from_f32<TC>(add_old ? to_f32(Rsrc[(long long)m * g.ldc + n]) + val : val);
-                    }
-                }
-            }
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    // this lane's chunk of each of its wave's loads (the same for every slab)
+    int a_row[TA::LOADS], a_chunk[TA::LOADS], b_row[TB::LOADS], b_chunk[TB::LOADS];
+#pragma unroll
+    for (int i = 0; i < TA::LOADS; i++) TA::lane_chunk(i, wave, lane, a_row[i], a_chunk[i]);
+#pragma unroll
+    for (int i = 0; i < TB::LOADS; i++) TB::lane_chunk(i, wave, lane, b_row[i], b_chunk[i]);
+
+    // Where a slab's loads come from and go to (uniform values): the slab's K segment is picked with scalar selects.
+    struct SlabSource {
+        const bf16_t *a0, *b0;
+        int lda, ldb;
+        bf16_t *As, *Bs;
+    };
+    auto locate = [&](int slab, int stage) {
+        int k0 = k_lo + slab * BK, lda = g.lda, ldb = g.ldb;
+        const bf16_t* Ap = A;
+        const bf16_t* Bp = B;
+        if (g.nseg > 1) {
+            const bool s1 = k0 >= g.seg_end[0], s2 = g.nseg > 2 && k0 >= g.seg_end[1];
+            Ap = s2 ? static_cast<const bf16_t*>(g.A_seg[1]) : s1 ? static_cast<const bf16_t*>(g.A_seg[0]) : A;
+            Bp = s2 ? static_cast<const bf16_t*>(g.B_seg[1]) : s1 ? static_cast<const bf16_t*>(g.B_seg[0]) : B;
+            lda = s2 ? g.lda_seg[1] : s1 ? g.lda_seg[0] : lda;
+            ldb = s2 ? g.ldb_seg[1] : s1 ? g.ldb_seg[0] : ldb;
+            k0 -= s2 ? g.seg_end[1] : s1 ? g.seg_end[0] : 0;
         }
+        SlabSource src;
+        // slab origin: an LDS row is an operand row (k-contiguous storage) or a contraction index (the other storage)
+        src.a0 = A_KC ? Ap + (long long)m0 * lda + k0 : Ap + (long long)k0 * lda + m0;
+        src.b0 = B_KC ? Bp + (long long)n0 * ldb + k0 : Bp + (long long)k0 * ldb + n0;
+        src.lda = lda;
+        src.ldb = ldb;
+        src.As = lds[stage];
+        src.Bs = lds[stage] + TA::ELEMS;
+        return src;
+    };
+    // loads h_lo..h_hi-1 of the NLOADS this wave issues per slab
+    auto issue = [&](const SlabSource& src, auto h_lo_c, auto h_hi_c) {
+        constexpr int h_lo = decltype(h_lo_c)::value, h_hi = decltype(h_hi_c)::value;
+#pragma unroll
+        for (int h = h_lo; h < h_hi; h++) {
+            if (h < TA::LOADS) load_to_lds_16(src.a0 + (long long)a_row[h] * src.lda + a_chunk[h] * 8, src.As + TA::lds_block(h, wave));
+            else load_to_lds_16(src.b0 + (long long)b_row[h - TA::LOADS] * src.ldb + b_chunk[h - TA::LOADS] * 8, src.Bs + TB::lds_block(h - TA::LOADS, wave));
+        }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using IN = std::integral_constant<int, NLOADS>;
+    const int nk = (k_hi - k_lo) / BK;
+    issue(locate(0, 0), I0{}, IN{});
+    if (nk > 1) issue(locate(1, 1), I0{}, IN{});
+    int stage = 0;
+    // One slab.  REFILL: the loads of slab kt+2 are issued, spread over the contraction steps behind each step's
+    // MFMAs, into the stage that held slab kt-1.  The last two slabs run the body without them.
+    auto slab = [&](int kt, auto refill_c) {
+        constexpr bool REFILL = decltype(refill_c)::value;
+        // slab kt has landed when at most the loads of slab kt+1 are outstanding
+        if (REFILL || kt + 1 < nk) wait_loads_but<NLOADS>();
+        else wait_loads_but<0>();
+        barrier_no_fence();  // slab kt is complete in LDS; every wave is done with slab kt-1
+        const SlabSource next = locate(REFILL ? kt + 2 : kt, stage == 0 ? 2 : stage - 1);
+        const bf16_t* As = lds[stage];
+        const bf16_t* Bs = lds[stage] + TA::ELEMS;
+        static_for<KSTEPS>([&](auto st_c) {
+            constexpr int st = decltype(st_c)::value;
+            bf16x8 a[TM], b[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) a[i] = TA::fragment(As, wm * WM + i * 32, st * 16, lane);
+#pragma unroll
+            for (int j = 0; j < TN; j++) b[j] = TB::fragment(Bs, wn * WN + j * 32, st * 16, lane);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+            if (REFILL)
+                issue(next, std::integral_constant<int, st * NLOADS / KSTEPS>{}, std::integral_constant<int, (st + 1) * NLOADS / KSTEPS>{});
+        });
+        stage = stage == 2 ? 0 : stage + 1;
+    };
+    int kt = 0;
+    for (; kt + 2 < nk; kt++) slab(kt, std::true_type{});
+    for (; kt < nk; kt++) slab(kt, std::false_type{});
+    barrier_no_fence();  // the staging epilogue reuses the operand LDS
+    gemm_store_tile<BM, BN, WGM, WGN, false, sizeof(lds), TC>(g, acc, reinterpret_cast<float*>(&lds[0][0]), C, Rsrc, add_old, bz, split, part,
+                                                              m0, n0, wave, wm, wn, lane);
 }
 
 // C += partial[0] + partial[1] + ... in that order, one thread per 4 consecutive elements of a row.
@@ -386,6 +578,24 @@ void launch_mfma_t(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int 
     else if (a_kc && !b_kc) gemm_mfma_kernel<BM, BN, BK, WGM, WGN, true, false, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
     else if (!a_kc && b_kc) gemm_mfma_kernel<BM, BN, BK, WGM, WGN, false, true, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
     else gemm_mfma_kernel<BM, BN, BK, WGM, WGN, false, false, EDGE, TC><<<grid, T, 0, ctx->stream>>>(g);
+}
+template <int BM, int BN, int BK, int WGM, int WGN>
+void launch_mfma_direct(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int batch, int dtype_c) {
+    dim3 grid((unsigned)(g.N / BN), (unsigned)(g.M / BM), (unsigned)(batch * (g.split > 1 ? g.split : 1)));
+    constexpr int T = 64 * WGM * WGN;
+#define EISEN_DIRECT(AK, BKC, TC) gemm_mfma_direct_kernel<BM, BN, BK, WGM, WGN, AK, BKC, TC><<<grid, T, 0, ctx->stream>>>(g)
+    if (dtype_c == EISEN_BF16) {
+        if (a_kc && b_kc) EISEN_DIRECT(true, true, bf16_t);
+        else if (a_kc) EISEN_DIRECT(true, false, bf16_t);
+        else if (b_kc) EISEN_DIRECT(false, true, bf16_t);
+        else EISEN_DIRECT(false, false, bf16_t);
+    } else {
+        if (a_kc && b_kc) EISEN_DIRECT(true, true, float);
+        else if (a_kc) EISEN_DIRECT(true, false, float);
+        else if (b_kc) EISEN_DIRECT(false, true, float);
+        else EISEN_DIRECT(false, false, float);
+    }
+#undef EISEN_DIRECT
 }
 template <int BM, int BN, int BK, int WGM, int WGN>
 void launch_mfma_c(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int batch, int dtype_c) {
@@ -513,12 +723,12 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
             g.k_part = (int)(K / split);
             g.partial = static_cast<float*>(ws);
         }
-        // Tile choice (measured on MI355X at the config-5 shapes): 256x128 with 8 waves is ~5 % ahead of
-        // 128x128 with 4 when at least one operand is k-contiguous and the grid still covers every CU; two
-        // transposed operands (dW) need too much LDS for it and run 128x128 with 4 waves.  64x64 is for
-        // problems with few tiles.
+        // Tile choice (measured on MI355X at the config-5 shapes): 256x128 with 8 waves and operands loaded
+        // straight into three LDS stages is the fastest kernel whenever the shape is a whole number of such tiles
+        // and they fill the CUs evenly (it is 5-13 % ahead of the same tile staged through registers); other
+        // large shapes run 128x128 with 4 waves, two workgroups per CU.  64x64 is for problems with few tiles.
         if (wide) {
-            launch_mfma_c<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            launch_mfma_direct<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else if (big_tile || split128) {
             if (K % 64 == 0) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
             else launch_mfma_c<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
