@@ -730,7 +730,11 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         if (wide) {
             launch_mfma_direct<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else if (big_tile || split128) {
-            if (K % 64 == 0) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            // whole tiles: the direct-to-LDS kernel (one workgroup per CU) is up to 16 % ahead when the grid has at most
+            // one tile per CU and level with the register-staged kernel (two workgroups per CU) beyond that
+            const bool whole = M % 128 == 0 && N % 128 == 0 && K % 64 == 0 && (split == 1 || g.k_part % 64 == 0);
+            if (whole) launch_mfma_direct<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            else if (K % 64 == 0) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
             else launch_mfma_c<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else {
             launch_mfma_c<64, 64, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
