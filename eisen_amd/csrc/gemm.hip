@@ -322,7 +322,7 @@ struct DirectOperandTile {
     static constexpr int CPR = LDS_ROW / 8;         // 16-byte chunks per LDS row
     static constexpr int RPB = 64 / CPR;            // LDS rows filled by one wave instruction
     static constexpr int LOADS = ELEMS / 512 / WAVES;  // wave instructions per wave and slab
-    static_assert(CPR >= 8 && 64 % CPR == 0 && ELEMS % (512 * WAVES) == 0, "slab must split into whole 1 KB wave loads");
+    static_assert(CPR >= 4 && 64 % CPR == 0 && ELEMS % (512 * WAVES) == 0, "slab must split into whole 1 KB wave loads");
 
     // LDS row and (permuted) chunk this lane fetches in load i of its wave
     static __device__ __forceinline__ void lane_chunk(int i, int wave, int lane, int& row, int& chunk) {

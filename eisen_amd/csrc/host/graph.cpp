@@ -82,7 +82,7 @@ void Graph::device_free(Storage& s) {
 }
 void Graph::release(Tensor& t) {
     if (t.data.ptr) eisen_hip_free(ctx_, t.data.ptr);
-    if (t.grad.ptr) eisen_hip_free(ctx_, t.grad.ptr);
+    if (t.grad.ptr && !t.grad_borrowed) eisen_hip_free(ctx_, t.grad.ptr);
     if (t.shadow.ptr) eisen_hip_free(ctx_, t.shadow.ptr);
     t.data = t.grad = t.shadow = Storage();
 }
@@ -392,9 +392,21 @@ size_t Graph::matmul_residual(size_t a, size_t b, size_t r) {
     record({a, b, r}, out, [=](Graph& g) {
         const Storage& go = g.grad_for_read(out);
         int acc = 0;
-        Storage& gr = g.grad_for_write(r, &acc);
-        if (gr.dtype != go.dtype) throw Error("matmul_residual backward: gradient element types differ");
-        g.check(eisen_hip_accumulate(g.ctx(), gr.ptr, go.ptr, go.dtype, M * N, acc), "matmul_residual backward dR");
+        Tensor& tr = g.at(r);
+        Tensor& to = g.at(out);
+        if (!tr.is_param && !tr.grad.valid() && !to.is_param && !to.grad_borrowed && tr.data.dtype == go.dtype) {
+            // The first gradient to reach the residual is dOut itself: hand the buffer over instead of copying it.
+            // Nothing reads dOut after this node (its consumers ran before it), and later contributions to dR
+            // accumulate into the buffer in place.
+            tr.grad = to.grad;
+            tr.grad_written = true;
+            to.grad_borrowed = true;
+        } else {
+            Storage& gr = g.grad_for_write(r, &acc);
+            if (gr.dtype != go.dtype) throw Error("matmul_residual backward: gradient element types differ");
+            if (gr.ptr == go.ptr) throw Error("matmul_residual backward: a second backward pass over the same activations is not supported");
+            g.check(eisen_hip_accumulate(g.ctx(), gr.ptr, go.ptr, go.dtype, M * N, acc), "matmul_residual backward dR");
+        }
         Storage& ga = g.grad_for_write(a, &acc);
         g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc), "matmul_residual backward dA");
         Storage& gb = g.grad_for_write(b, &acc);

@@ -44,6 +44,7 @@ struct Tensor {
     bool is_pooled = false;
     bool is_param = false;        // allocated through alloc()/alloc_param_bf16(): owns an f32 grad
     bool grad_written = false;    // this backward pass already stored into grad (next store accumulates)
+    bool grad_borrowed = false;   // grad's buffer now belongs to another tensor's grad (see matmul_residual): not freed with this one
     bool grad_zero_pending = false;  // zero_grad() was requested; materialised on first use
     std::vector<float> host_copy;    // kept for small host-loaded tensors (token ids)
     size_t size() const {
