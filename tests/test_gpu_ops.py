@@ -592,6 +592,36 @@ def test_gemm_residual(ctx, M, N, K, dtype):
         x.free()
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_bf16_wide_tile_grouped_order(ctx, ta, tb):
+    # 15 x 68 tiles of 256x128: C is walked in groups of 32 N tiles, the last group only 4 wide
+    _gemm_case(ctx, 3840, 8704, 64, ta, tb, BF16, BF16, False, seed=480)
+    _gemm_case(ctx, 3840, 8704, 192, ta, tb, BF16, F32, True, seed=483)
+
+
+def test_gemm_wide_tile_batched_and_segmented(ctx):
+    # the launch-saving entry points at a shape that takes the 256x128 tile (256 tiles)
+    M, N, K = 4096, 1024, 128
+    a = prep(gen.normal(490, (M, K)), BF16)
+    w = prep(gen.normal(491, (2, K, N)), BF16)
+    da, dw, dc = up(ctx, a, BF16), up(ctx, w, BF16), ctx.malloc(2 * M * N * 2)
+    ctx.gemm_strided_batched(da, dw, dc, BF16, BF16, 0, 0, 2, M, N, K, 0, K * N, M * N)
+    got = dn(ctx, dc, (2, M, N), BF16)
+    for i in range(2):
+        assert_close(got[i], a.astype(np.float64) @ w[i].astype(np.float64), 2e-2, f"wide pair {i}")
+    for x in (da, dw, dc):
+        x.free()
+    M, N, Ks = 4096, 2048, (128, 64, 192)
+    dys = [prep(gen.normal(492 + i, (M, k)), BF16) for i, k in enumerate(Ks)]
+    wts = [prep(gen.normal(496 + i, (N, k)), BF16) for i, k in enumerate(Ks)]
+    exp = sum(d.astype(np.float64) @ x.astype(np.float64).T for d, x in zip(dys, wts))
+    dA, dB, dc = [up(ctx, d, BF16) for d in dys], [up(ctx, x, BF16) for x in wts], ctx.malloc(M * N * 2)
+    ctx.gemm_ksegments(dA, dB, list(Ks), dc, BF16, BF16, 0, 1, M, N, 0)
+    assert_close(dn(ctx, dc, (M, N), BF16), exp, 2e-2, "wide ksegments")
+    for x in dA + dB + [dc]:
+        x.free()
+
+
 def test_gemm_f32_matches_oracle_order_tolerance(ctx):
     # config-1 sized linear against the sequential-order f32 oracle, rtol 1e-4
     a, b, go = gen.normal(410, (64, 64)), gen.normal(411, (64, 256), 0.02), gen.normal(412, (64, 256))
