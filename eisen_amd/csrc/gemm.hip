@@ -758,7 +758,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     const long long wide_tiles = (long long)(M / 256) * (N / 128) * batch;
     const bool wide = mfma_ok && split == 1 && big_tile && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && wide_tiles >= 256 &&
                       (double)wide_tiles / (double)(256 * ((wide_tiles + 255) / 256)) >= 0.85;
-    const char* tile = !mfma_ok ? "fma64x64" : wide ? "256x128x64" : (big_tile || split128) ? (K % 64 == 0 ? "128x128x64" : "128x128x32") : "64x64x32";
+    const char* tile = !mfma_ok ? "fma64x64" : wide ? (!a_kc && !b_kc && wide_tiles >= 512 ? "256x128x32" : "256x128x64") : (big_tile || split128) ? (K % 64 == 0 ? "128x128x64" : "128x128x32") : "64x64x32";
     snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
              dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : "");
     EisenProfScope prof(ctx, pname, 2.0 * (double)M * (double)N * (double)K * (double)batch, true);
@@ -775,7 +775,11 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         // straight into three LDS stages is the fastest kernel whenever the shape is a whole number of such tiles
         // and they fill the CUs evenly (it is 5-13 % ahead of the same tile staged through registers); other
         // large shapes run 128x128 with 4 waves, two workgroups per CU.  64x64 is for problems with few tiles.
-        if (wide) {
+        if (wide && !a_kc && !b_kc && wide_tiles >= 512) {
+            // both operands through the (slower) transposing LDS reads and at least two tiles per CU: slabs of 32 need
+            // half the LDS, so two workgroups share a CU and cover each other's barrier waits and epilogues (6-7 % faster)
+            launch_mfma_direct<256, 128, 32, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+        } else if (wide) {
             launch_mfma_direct<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else if (big_tile || split128) {
             // whole tiles: the direct-to-LDS kernel (one workgroup per CU) is up to 16 % ahead when the grid has at most
