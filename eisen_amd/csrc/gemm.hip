@@ -45,6 +45,11 @@ struct GemmArgs {
     int split;                         // > 1: K is cut into this many parts; part p > 0 assigns into partial[p-1]
     int k_part;                        // contraction length of one part (a multiple of the slab)
     float* partial;                    // [batch][split-1][M][N] f32, summed into C by a second kernel
+    // SwiGLU-backward epilogue (gate != nullptr): the product is dH, the gradient of h = silu(gate) * up; C receives
+    // dgate = dH * up * silu'(gate) and C2 receives dup = dH * silu(gate) (all with C's layout, no accumulation, no split-K)
+    const void* gate;
+    const void* up;
+    void* C2;
     int tile_group;                    // direct kernel: > 0 = N tiles per group of the tile order (see the kernel), 0 = row-major order
     int vec_c;                         // C rows are 16-byte aligned at every 8th column: the epilogue may use 16-byte accesses
     // K made of up to three segments with their own operands, C (+)= sum_s op(A_s) op(B_s): segment 0 is A/B/lda/ldb,
@@ -114,6 +119,14 @@ struct OperandTile {
     }
 };
 
+// d(silu(gate) * up) for one element, given dh (src/graph/ops/elementwise.rs:442-455 for silu, :294-331 for mul)
+__device__ __forceinline__ void swiglu_backward_elem(float gate, float up, float dh, float& dgate, float& dup) {
+    const float sig = 1.0f / (1.0f + __expf(-gate));
+    const float silu = gate * sig;
+    dgate = (dh * up) * (silu + sig * (1.0f - silu));
+    dup = dh * silu;
+}
+
 // Epilogue shared by the MFMA kernels.  Accumulator register v of lane l holds
 // C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.  `lds_f32` is the operand LDS (LDS_BYTES bytes), idle by now
 // and used as a staging area.
@@ -155,6 +168,30 @@ __device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)
                     float* dst = P + (long long)m * g.N + n;
                     *reinterpret_cast<float4*>(dst) = lo;
                     *reinterpret_cast<float4*>(dst + 4) = hi;
+                } else if (g.gate) {
+                    const long long at = (long long)bz * g.sC + (long long)m * g.ldc + n;
+                    const TC* gsrc = static_cast<const TC*>(g.gate) + at;
+                    const TC* usrc = static_cast<const TC*>(g.up) + at;
+                    Pack<TC> og[8 / Pack<TC>::N], ou[8 / Pack<TC>::N];
+#pragma unroll
+                    for (int k = 0; k < 8 / Pack<TC>::N; k++) {
+                        og[k] = load_pack(gsrc + k * Pack<TC>::N);
+                        ou[k] = load_pack(usrc + k * Pack<TC>::N);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        float dgate, dup;
+                        swiglu_backward_elem(og[e / Pack<TC>::N].get(e % Pack<TC>::N), ou[e / Pack<TC>::N].get(e % Pack<TC>::N), val[e], dgate, dup);
+                        og[e / Pack<TC>::N].set(e % Pack<TC>::N, dgate);
+                        ou[e / Pack<TC>::N].set(e % Pack<TC>::N, dup);
+                    }
+                    TC* d1 = C + (long long)m * g.ldc + n;
+                    TC* d2 = static_cast<TC*>(g.C2) + at;
+#pragma unroll
+                    for (int k = 0; k < 8 / Pack<TC>::N; k++) {
+                        store_pack(d1 + k * Pack<TC>::N, og[k]);
+                        store_pack(d2 + k * Pack<TC>::N, ou[k]);
+                    }
                 } else {
                     TC* dst = C + (long long)m * g.ldc + n;
                     Pack<TC> o[8 / Pack<TC>::N];
@@ -187,6 +224,12 @@ __device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)
                     const float val = acc[i][j][v];
                     if (P) {
                         P[(long long)m * g.N + n] = val;
+                    } else if (g.gate) {
+                        const long long at = (long long)bz * g.sC + (long long)m * g.ldc + n;
+                        float dgate, dup;
+                        swiglu_backward_elem(to_f32(static_cast<const TC*>(g.gate)[at]), to_f32(static_cast<const TC*>(g.up)[at]), val, dgate, dup);
+                        C[(long long)m * g.ldc + n] = from_f32<TC>(dgate);
+                        static_cast<TC*>(g.C2)[at] = from_f32<TC>(dup);
                     } else {
                         TC* dst = C + (long long)m * g.ldc + n;
                         *dst = from_f32<TC>(add_old ? to_f32(Rsrc[(long long)m * g.ldc + n]) + val : val);
@@ -672,9 +715,16 @@ struct KSegments {  // further (A, B, K) segments after the first one
     const void* B[2];
     size_t K[2];
 };
+struct SwigluBackwardEpilogue {  // see GemmArgs::gate
+    const void* gate;
+    const void* up;
+    void* dup;
+};
+constexpr int kEpilogueNotFusable = -7001;  // internal: the shape takes a kernel without the fused epilogue
 static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
                        int trans_b, size_t M, size_t N, size_t K, size_t batch, long long sA, long long sB, long long sC,
-                       int accumulate, const char* who, const KSegments* segs = nullptr, const void* residual = nullptr) {
+                       int accumulate, const char* who, const KSegments* segs = nullptr, const void* residual = nullptr,
+                       const SwigluBackwardEpilogue* swiglu = nullptr) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, A && B && C, EISEN_E_ARG, "%s: null pointer", who);
     EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype_ab) && eisen_dtype_ok(dtype_c), EISEN_E_ARG, "%s: unknown dtype", who);
@@ -737,6 +787,13 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     if (a_kc) mfma_ok = mfma_ok && K % 8 == 0; else mfma_ok = mfma_ok && M % 8 == 0;
     if (b_kc) mfma_ok = mfma_ok && K % 8 == 0; else mfma_ok = mfma_ok && N % 8 == 0;
     EISEN_REQUIRE(ctx, n_more == 0 || mfma_ok, EISEN_E_ARG, "%s: segmented contraction reached a shape the MFMA kernel does not take", who);
+    if (swiglu) {
+        if (!mfma_ok) return kEpilogueNotFusable;
+        g.gate = swiglu->gate;
+        g.up = swiglu->up;
+        g.C2 = swiglu->dup;
+        g.vec_c = g.vec_c && eisen_aligned(swiglu->gate, 16) && eisen_aligned(swiglu->up, 16) && eisen_aligned(swiglu->dup, 16);
+    }
     // profile key = one kernel instantiation (operand orders, types, tile), so the event timing
     // lines up with a profiler's per-kernel rows
     char pname[64];
@@ -746,7 +803,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     // gets a tile.  Part 0 writes C as usual, the other parts go to an f32 scratch that a second kernel
     // adds to C in a fixed order, so the result does not depend on scheduling.
     int split = 1;
-    if (mfma_ok && N % 4 == 0 && K >= 1024 && n_more == 0) {
+    if (mfma_ok && N % 4 == 0 && K >= 1024 && n_more == 0 && !swiglu) {
         const bool t128 = M >= 128 && N >= 128;
         const long long tiles = t128 ? tiles128 : (long long)eisen_ceil_div(M, 64) * eisen_ceil_div(N, 64) * batch;
         const size_t slab = t128 ? 64 : 32, min_part = t128 ? 512 : 256;
@@ -852,4 +909,25 @@ extern "C" int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void
         return 0;
     }
     return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, 1, 0, 0, 0, 0, "eisen_hip_gemm_residual", nullptr, R);
+}
+
+extern "C" int eisen_hip_gemm_swiglu_backward(eisen_ctx* ctx, const void* A, const void* B, const void* gate, const void* up, void* dgate,
+                                              void* dup, int dtype, int trans_a, int trans_b, size_t M, size_t N, size_t K) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, gate && up && dgate && dup, EISEN_E_ARG, "eisen_hip_gemm_swiglu_backward: null pointer");
+    if (M * N == 0) return 0;
+    if (K > 0) {
+        const SwigluBackwardEpilogue fuse{gate, up, dup};
+        const int rc = gemm_common(ctx, A, B, dgate, dtype, dtype, trans_a, trans_b, M, N, K, 1, 0, 0, 0, 0, "eisen_hip_gemm_swiglu_backward", nullptr,
+                                   nullptr, &fuse);
+        if (rc != kEpilogueNotFusable) return rc;
+    }
+    // shapes and types the MFMA kernels do not take: the product through a temporary, then the element-wise kernel
+    void* dh = nullptr;
+    int rc = eisen_hip_malloc(ctx, M * N * eisen_dtype_size(dtype), &dh);
+    if (rc) return rc;
+    rc = gemm_common(ctx, A, B, dh, dtype, dtype, trans_a, trans_b, M, N, K, 1, 0, 0, 0, 0, "eisen_hip_gemm_swiglu_backward");
+    if (!rc) rc = eisen_hip_swiglu_backward(ctx, gate, up, dh, dgate, dup, dtype, M * N, 0, 0);
+    const int rc_free = eisen_hip_free(ctx, dh);
+    return rc ? rc : rc_free;
 }

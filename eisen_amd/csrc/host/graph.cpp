@@ -415,6 +415,57 @@ size_t Graph::matmul_residual(size_t a, size_t b, size_t r) {
     return out;
 }
 
+// The feed-forward tail of the transformer block, `ffn2(g.mul(g.silu(gate), up)) + res1` (src/nn/transformer.rs:44-47),
+// as one node: forward = the SwiGLU kernel + the residual GEMM; backward = dR (buffer hand-over as in
+// matmul_residual), dW += h^T dOut, and one GEMM whose epilogue turns dH = dOut W^T straight into dgate and dup
+// (dH itself is never stored).
+size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r) {
+    const std::vector<size_t> sg = at(gate).shape, sb = at(b).shape, sr = at(r).shape;
+    if (sb.size() != 2 || sg.empty() || sr.empty() || at(up).shape != sg) throw Error("swiglu_matmul_residual: expects gate/up [..,K], b [K,N], r [..,N]");
+    const size_t K = sg.back(), M = numel_of(sg) / std::max<size_t>(K, 1), N = sb[1];
+    if (sb[0] != K || sr.back() != N || numel_of(sr) != M * N) throw Error("swiglu_matmul_residual: shapes do not match: " + shape_str(sg) + " x " + shape_str(sb) + " + " + shape_str(sr));
+    const Storage dg = compute_data(gate), du = compute_data(up), db = compute_data(b), dr = compute_data(r);
+    if (dg.dtype != du.dtype || dg.dtype != db.dtype || dr.dtype != dg.dtype) throw Error("swiglu_matmul_residual: operands have different element types");
+    const size_t h = push_tensor(sg, dg.dtype, true);  // kept for dW
+    check(eisen_hip_swiglu(ctx_, dg.ptr, du.ptr, at(h).data.ptr, dg.dtype, dg.numel), "swiglu");
+    const size_t out = push_tensor(sr, dg.dtype, true);
+    check(eisen_hip_gemm_residual(ctx_, at(h).data.ptr, db.ptr, dr.ptr, at(out).data.ptr, dg.dtype, dg.dtype, 0, 0, M, N, K), "swiglu_matmul_residual");
+    record({gate, up, b, r}, out, [=](Graph& g) {
+        const Storage& go = g.grad_for_read(out);
+        int acc = 0;
+        Tensor& tr = g.at(r);
+        Tensor& to = g.at(out);
+        if (!tr.is_param && !tr.grad.valid() && !to.is_param && !to.grad_borrowed && tr.data.dtype == go.dtype) {
+            tr.grad = to.grad;  // see matmul_residual
+            tr.grad_written = true;
+            to.grad_borrowed = true;
+        } else {
+            Storage& gr = g.grad_for_write(r, &acc);
+            if (gr.dtype != go.dtype) throw Error("swiglu_matmul_residual backward: gradient element types differ");
+            if (gr.ptr == go.ptr) throw Error("swiglu_matmul_residual backward: a second backward pass over the same activations is not supported");
+            g.check(eisen_hip_accumulate(g.ctx(), gr.ptr, go.ptr, go.dtype, M * N, acc), "swiglu_matmul_residual backward dR");
+        }
+        int ag = 0, au = 0;
+        Storage& gg = g.grad_for_write(gate, &ag);
+        Storage& gu = g.grad_for_write(up, &au);
+        const Storage wb = g.compute_data(b);
+        if (!ag && !au && gg.dtype == go.dtype && gu.dtype == go.dtype) {
+            g.check(eisen_hip_gemm_swiglu_backward(g.ctx(), go.ptr, wb.ptr, g.compute_data(gate).ptr, g.compute_data(up).ptr, gg.ptr, gu.ptr, go.dtype, 0, 1, M,
+                                                   K, N),
+                    "swiglu_matmul_residual backward dgate/dup");
+        } else {  // gate or up already carries a gradient: dH through a temporary, then the accumulating element-wise kernel
+            Storage dh = g.device_alloc(M * K, go.dtype, false);
+            g.check(eisen_hip_gemm(g.ctx(), go.ptr, wb.ptr, dh.ptr, go.dtype, go.dtype, 0, 1, M, K, N, 0), "swiglu_matmul_residual backward dH");
+            g.check(eisen_hip_swiglu_backward(g.ctx(), g.compute_data(gate).ptr, g.compute_data(up).ptr, dh.ptr, gg.ptr, gu.ptr, go.dtype, M * K, ag, au),
+                    "swiglu_matmul_residual backward");
+            g.device_free(dh);
+        }
+        Storage& gb = g.grad_for_write(b, &acc);
+        g.check(eisen_hip_gemm(g.ctx(), g.at(h).data.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "swiglu_matmul_residual backward dB");
+    });
+    return out;
+}
+
 // Several Graph::matmul calls that share their left operand (Q/K/V projections, gate and up projections:
 // src/nn/attention.rs:300-302, src/nn/transformer.rs:41-44), with the results of the separate matmuls but
 // fewer launches: equally shaped neighbours (K and V, gate and up) run as a batch of two whose "stride" is the

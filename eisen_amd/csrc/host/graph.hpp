@@ -107,6 +107,7 @@ class Graph {
     size_t swiglu(size_t gate, size_t up);                      // fused silu(gate) * up
     size_t matmul(size_t a, size_t b);
     size_t matmul_residual(size_t a, size_t b, size_t r);  // r + a b in one kernel
+    size_t swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r);  // r + (silu(gate) * up) b; backward forms dgate, dup in the dX GEMM
     // matmuls of one input against 2-3 weights with fewer launches (bf16 graphs; otherwise plain matmuls)
     std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights);
     size_t matmul_bf16(size_t a, size_t b) { return matmul(a, b); }

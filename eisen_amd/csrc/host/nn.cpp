@@ -167,6 +167,7 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
     }
     const size_t norm2_out = norm2.forward(g, res1);
     size_t gated;
+    size_t gate_id = (size_t)-1, up_id = (size_t)-1;  // set when gate and up are available unfused-multiplied (SwiGLU folded into the down projection node)
     if (attn.fused && !ffn_gate.has_bias && !ffn1.has_bias) {
         // gate and up projections as one launch, then the fused SwiGLU
         const std::vector<size_t> guv = g.matmul_group(norm2_out, {ffn_gate.weight_id, ffn1.weight_id});
@@ -177,7 +178,13 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
             g.reinterpret_shape(gu.first, {ns[0], ns[1], f});
             g.reinterpret_shape(gu.second, {ns[0], ns[1], f});
         }
-        gated = g.swiglu(gu.first, gu.second);
+        if (!ffn2.has_bias) {
+            gate_id = gu.first;
+            up_id = gu.second;
+            gated = (size_t)-1;
+        } else {
+            gated = g.swiglu(gu.first, gu.second);
+        }
     } else if (attn.fused) {
         const size_t gate_out = ffn_gate.forward(g, norm2_out);
         const size_t up = ffn1.forward(g, norm2_out);
@@ -188,6 +195,7 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
         const size_t up = ffn1.forward(g, norm2_out);
         gated = g.mul(gate, up);
     }
+    if (gate_id != (size_t)-1) return g.swiglu_matmul_residual(gate_id, up_id, ffn2.weight_id, res1);  // SwiGLU + down projection + residual
     if (attn.fused && !ffn2.has_bias) return g.matmul_residual(gated, ffn2.weight_id, res1);  // down projection + residual
     const size_t ffn2_out = ffn2.forward(g, gated);
     return g.add(res1, ffn2_out);

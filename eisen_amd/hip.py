@@ -268,6 +268,11 @@ class Context:
         """C = R + op(A) op(B)."""
         self._call("eisen_hip_gemm_residual", _ptr(A), _ptr(B), _ptr(R), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(M), _sz(N), _sz(K))
 
+    def gemm_swiglu_backward(self, A, B, gate, up, dgate, dup, dtype, trans_a, trans_b, M, N, K):
+        """[dgate, dup] = d(silu(gate) * up) for dH = op(A) op(B)."""
+        self._call("eisen_hip_gemm_swiglu_backward", _ptr(A), _ptr(B), _ptr(gate), _ptr(up), _ptr(dgate), _ptr(dup), _i(dtype), _i(trans_a), _i(trans_b),
+                   _sz(M), _sz(N), _sz(K))
+
     def gemm_ksegments(self, As, Bs, Ks, Cbuf, dtype_ab, dtype_c, trans_a, trans_b, M, N, accumulate=0):
         """C (+)= sum_s op(A_s) op(B_s) over up to three (A, B, K) segments."""
         n = len(Ks)

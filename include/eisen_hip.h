@@ -213,6 +213,14 @@ int eisen_hip_gemm_strided_batched(eisen_ctx* ctx, const void* A, const void* B,
  * `g.add(res1_out, ffn2_out)`) as one kernel: the product is added to the residual in f32 and rounded once. */
 int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void* B, const void* R, void* C, int dtype_ab, int dtype_c,
                             int trans_a, int trans_b, size_t M, size_t N, size_t K);
+
+/* [dgate, dup] = d(silu(gate) * up) for dH = op(A) * op(B): the input gradient of the down projection
+ * (src/graph/ops/linear.rs:269-277, dA = dC B^T) followed by the backward of `g.mul(g.silu(gate), up)`
+ * (src/nn/transformer.rs:44-46; src/graph/ops/elementwise.rs:442-455 silu, :294-331 mul) in one kernel: dH is
+ * never stored, the two gradients are formed from the f32 accumulators.  gate, up, dgate, dup are [M, N] of
+ * `dtype`; the results are assigned (no accumulation). */
+int eisen_hip_gemm_swiglu_backward(eisen_ctx* ctx, const void* A, const void* B, const void* gate, const void* up, void* dgate,
+                                   void* dup, int dtype, int trans_a, int trans_b, size_t M, size_t N, size_t K);
 /* C (+)= sum over up to three segments s of op(A_s) * op(B_s), each segment with its own operands and
  * contraction length K_s (A_s is [M,K_s] or, transposed, [K_s,M]; B_s is [K_s,N] or [N,K_s]).  This is the
  * input gradient of several linear layers that read the same tensor (dX = dQ Wq^T + dK Wk^T + dV Wv^T, which

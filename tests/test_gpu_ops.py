@@ -622,6 +622,28 @@ def test_gemm_wide_tile_batched_and_segmented(ctx):
         x.free()
 
 
+@pytest.mark.parametrize("M,N,K,dtype", [(256, 128, 192, BF16), (4096, 1024, 128, BF16), (512, 384, 1024, BF16), (200, 72, 40, BF16), (64, 48, 32, F32)])
+def test_gemm_swiglu_backward(ctx, M, N, K, dtype):
+    # dH = dY W^T (dY [M, K], W [N, K]) never stored; dgate = dH * up * silu'(gate), dup = dH * silu(gate)
+    dy, w = prep(gen.normal(520, (M, K)), dtype), prep(gen.normal(521, (N, K), 0.2), dtype)
+    gate, up_ = prep(gen.normal(522, (M, N)), dtype), prep(gen.normal(523, (M, N)), dtype)
+    dh = dy.astype(np.float64) @ w.astype(np.float64).T
+    g64 = gate.astype(np.float64)
+    sig = 1.0 / (1.0 + np.exp(-g64))
+    silu = g64 * sig
+    exp_dgate = dh * up_ * (silu + sig * (1.0 - silu))
+    exp_dup = dh * silu
+    d = [up(ctx, x, dtype) for x in (dy, w, gate, up_)]
+    es = 2 if dtype == BF16 else 4
+    dgate, dup = ctx.malloc(M * N * es), ctx.malloc(M * N * es)
+    ctx.gemm_swiglu_backward(d[0], d[1], d[2], d[3], dgate, dup, dtype, 0, 1, M, N, K)
+    tol = 2e-2 if dtype == BF16 else 2e-4
+    assert_close(dn(ctx, dgate, (M, N), dtype), exp_dgate, tol, "dgate")
+    assert_close(dn(ctx, dup, (M, N), dtype), exp_dup, tol, "dup")
+    for x in d + [dgate, dup]:
+        x.free()
+
+
 def test_gemm_f32_matches_oracle_order_tolerance(ctx):
     # config-1 sized linear against the sequential-order f32 oracle, rtol 1e-4
     a, b, go = gen.normal(410, (64, 64)), gen.normal(411, (64, 256), 0.02), gen.normal(412, (64, 256))
