@@ -39,6 +39,9 @@ struct AttnArgs {
     float scale, scale_log2e;
     int causal;
     int paired;  // query-stationary kernels: a block runs a long query block and its short mirror image
+    // backward only: when set ([S][hd/2] cos/sin), Q and K are rotary-embedded projections and dQ, dK are the
+    // gradients of the projections before the rotation (the inverse rotation is applied as the gradients are stored)
+    const float2* rope;
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -59,6 +62,19 @@ __device__ __forceinline__ bf16x8 concat4(bf16x4 lo, bf16x4 hi) {
 }
 // Row index inside a 32x32 MFMA accumulator tile held by register v of a lane in half g.
 __device__ __forceinline__ int acc_row(int v, int g) { return 8 * (v >> 2) + 4 * g + (v & 3); }
+
+// Backward of the rotary embedding on NP interleaved pairs: dx0 = g0 c + g1 s, dx1 = -g0 s + g1 c
+// (src/graph/ops/transform.rs:592-595); cs points at the (cos, sin) of the first pair.
+template <int NP>
+__device__ __forceinline__ void unrotate_pairs(float* x, const float2* cs) {
+#pragma unroll
+    for (int j = 0; j < NP; j++) {
+        const float2 t = cs[j];
+        const float g0 = x[2 * j], g1 = x[2 * j + 1];
+        x[2 * j] = g0 * t.x + g1 * t.y;
+        x[2 * j + 1] = -g0 * t.y + g1 * t.x;
+    }
+}
 
 // K-operand (8 values along the contraction) for contraction step t of a [32-row k-dim] x
 // [32-col] block of a row-major LDS tile, in the order the accumulator registers 8t..8t+7 use.
@@ -447,9 +463,13 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int vg = 0; vg < 4; vg++) {
+                    float x[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[e] = dq[dt][vg * 4 + e] * a.scale;
+                    if (a.rope) unrotate_pairs<2>(x, a.rope + (size_t)q * (HD / 2) + (dt * 32 + 8 * vg + 4 * g) / 2);
                     bf16x4 w;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) w[e] = (bf16_t)(dq[dt][vg * 4 + e] * a.scale);
+                    for (int e = 0; e < 4; e++) w[e] = (bf16_t)x[e];
                     *reinterpret_cast<bf16x4*>(dQp + dt * 32 + 8 * vg + 4 * g) = w;
                 }
         }
@@ -629,6 +649,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dkv_kernel(AttnArgs a) {
                 }
                 const int kr = k0 + e0 / HD;
                 if (kr < a.S) {
+                    if (which == 0 && a.rope) unrotate_pairs<4>(acc8, a.rope + (size_t)kr * (HD / 2) + (e0 % HD) / 2);
                     bf16x8 o8;
 #pragma unroll
                     for (int e = 0; e < 8; e++) o8[e] = (bf16_t)acc8[e];
@@ -861,11 +882,11 @@ extern "C" int eisen_hip_attention_forward(eisen_ctx* ctx, const void* q, const 
     return 0;
 }
 
-extern "C" int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
-                                            const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype,
-                                            size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
-                                            const long long* q_strides, const long long* kv_strides, float scale,
-                                            int causal) {
+static int attention_backward_common(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                     const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype,
+                                     size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
+                                     const long long* q_strides, const long long* kv_strides, float scale,
+                                     int causal, bool rope) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, q && k && v && out && dout && lse && dq && dk && dv, EISEN_E_ARG, "attention_backward: null pointer");
     AttnArgs a{};
@@ -877,6 +898,10 @@ extern "C" int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const
     rc = eisen_workspace(ctx, B * Hq * S * sizeof(float), &ws);
     if (rc) return rc;
     a.D = static_cast<float*>(ws);
+    if (rope) {
+        rc = eisen_rope_table_get(ctx, S, hd, &a.rope);
+        if (rc) return rc;
+    }
     if (dtype == EISEN_BF16) {
         EISEN_REQUIRE(ctx, eisen_aligned(q, 16) && eisen_aligned(k, 16) && eisen_aligned(v, 16) && eisen_aligned(out, 16) &&
                                eisen_aligned(dout, 16) && eisen_aligned(dq, 16) && eisen_aligned(dk, 16) && eisen_aligned(dv, 16),
@@ -893,4 +918,25 @@ extern "C" int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const
     }
     EISEN_LAUNCH_CHECK(ctx, "attention backward");
     return 0;
+}
+
+extern "C" int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                            const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype,
+                                            size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
+                                            const long long* q_strides, const long long* kv_strides, float scale,
+                                            int causal) {
+    return attention_backward_common(ctx, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, q_strides, kv_strides, scale, causal, false);
+}
+
+extern "C" int eisen_hip_attention_rope_backward(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                                 const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype,
+                                                 size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd, float scale, int causal) {
+    EISEN_CHECK_CTX(ctx);
+    if (dtype == EISEN_BF16)  // the MFMA kernels rotate dQ and dK back as they store them
+        return attention_backward_common(ctx, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, nullptr, nullptr, scale, causal, true);
+    // f32 path: the plain backward, then the rotary backward in place
+    int rc = attention_backward_common(ctx, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, nullptr, nullptr, scale, causal, false);
+    if (!rc) rc = eisen_hip_rope_backward(ctx, dq, dq, dtype, B, S, Hq * hd, hd, 0);
+    if (!rc) rc = eisen_hip_rope_backward(ctx, dk, dk, dtype, B, S, Hkv * hd, hd, 0);
+    return rc;
 }

@@ -888,6 +888,40 @@ size_t Graph::attention_gqa(size_t q, size_t k, size_t v, size_t heads, size_t k
     return attention_impl(q, k, v, sq[0], sq[1], heads, kv_heads, hd, nullptr, nullptr, scale, causal, sq);
 }
 
+// `g.rope(q)`, `g.rope(k)` and the attention chain (src/nn/attention.rs:316-375) as one node.  Forward: the two
+// rotary kernels into internal tensors, then the fused attention.  Backward: one attention backward whose
+// kernels un-rotate dQ and dK as they store them, so the gradients land directly on the projections.
+size_t Graph::attention_gqa_rope(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal) {
+    const std::vector<size_t> sq = at(q).shape, sk = at(k).shape;
+    if (sq.size() != 3 || sk.size() != 3 || at(v).shape != sk) throw Error("attention_gqa_rope: expects q [B,S,Hq*hd], k/v [B,S,Hkv*hd]");
+    if (heads == 0 || kv_heads == 0 || sq[2] % heads || heads % kv_heads) throw Error("attention_gqa_rope: bad head counts");
+    const size_t hd = sq[2] / heads, B = sq[0], S = sq[1];
+    if (sk[2] != kv_heads * hd || sk[0] != B || sk[1] != S) throw Error("attention_gqa_rope: k/v shape does not match q");
+    const Storage dq = compute_data(q), dk = compute_data(k), dv = compute_data(v);
+    if (dq.dtype != dk.dtype || dq.dtype != dv.dtype) throw Error("attention_gqa_rope: q, k, v must share an element type");
+    const size_t q_rot = push_tensor(sq, dq.dtype, true), k_rot = push_tensor(sk, dk.dtype, true);  // kept for backward
+    check(eisen_hip_rope(ctx_, dq.ptr, at(q_rot).data.ptr, dq.dtype, B, S, sq[2], hd), "rope");
+    check(eisen_hip_rope(ctx_, dk.ptr, at(k_rot).data.ptr, dk.dtype, B, S, sk[2], hd), "rope");
+    const size_t out = alloc_pooled_dtype(sq, dq.dtype);
+    const size_t lse = alloc_pooled_dtype({B, heads, S}, EISEN_F32);
+    check(eisen_hip_attention_forward(ctx_, at(q_rot).data.ptr, at(k_rot).data.ptr, dv.ptr, at(out).data.ptr, (float*)at(lse).data.ptr, dq.dtype, B, S,
+                                      heads, kv_heads, hd, nullptr, nullptr, scale, causal ? 1 : 0),
+          "attention forward");
+    record({q, k, v}, out, [=](Graph& gg) {
+        const Storage& go = gg.grad_for_read(out);
+        int aq = 0, ak = 0, av = 0;
+        Storage& gq = gg.grad_for_write(q, &aq);
+        Storage& gk = gg.grad_for_write(k, &ak);
+        Storage& gv = gg.grad_for_write(v, &av);
+        if (aq || ak || av) throw Error("attention backward: q, k, v must not have other consumers");
+        gg.check(eisen_hip_attention_rope_backward(gg.ctx(), gg.at(q_rot).data.ptr, gg.at(k_rot).data.ptr, gg.compute_data(v).ptr, gg.at(out).data.ptr, go.ptr,
+                                                   (const float*)gg.at(lse).data.ptr, gq.ptr, gk.ptr, gv.ptr, go.dtype, B, S, heads, kv_heads, hd, scale,
+                                                   causal ? 1 : 0),
+                 "attention backward");
+    });
+    return out;
+}
+
 size_t Graph::flash_attention(size_t q, size_t k, size_t v, float scale, bool causal) {
     const std::vector<size_t> sq = at(q).shape, sk = at(k).shape, sv = at(v).shape;
     if (sq.size() != 3) throw Error("flash_attention expects q=[B,M,D]");

@@ -127,6 +127,8 @@ class Graph {
     size_t flash_attention(size_t q, size_t k, size_t v, float scale, bool causal);
     // q [B,S,Hq*hd], k/v [B,S,Hkv*hd] straight from the projections -> [B,S,Hq*hd].
     size_t attention_gqa(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal);
+    // the same with the rotary embedding of q and k inside: rope(q), rope(k) -> attention; backward stores d q, d k un-rotated
+    size_t attention_gqa_rope(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal);
 
     // src/graph/mod.rs:670-796
     void backward(size_t loss_id);

@@ -99,14 +99,14 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
         k = k_proj.forward(g, x_id);
         v = v_proj.forward(g, x_id);
     }
-    const size_t q_rope = g.rope(q, head_dim), k_rope = g.rope(k, head_dim);
     const float scale = 1.0f / std::sqrt((float)head_dim);
     if (fused) {
-        // one op for steps 3-11: head split, GQA repeat, scores, scale, mask, softmax, P V, merge
-        const size_t ctx = g.attention_gqa(q_rope, k_rope, v, num_heads, num_kv_heads, scale, causal);
+        // one op for the rotary embedding and steps 3-11: head split, GQA repeat, scores, scale, mask, softmax, P V, merge
+        const size_t ctx = g.attention_gqa_rope(q, k, v, num_heads, num_kv_heads, scale, causal);
         if (residual != (size_t)-1 && !out_proj.has_bias) return g.matmul_residual(ctx, out_proj.weight_id, residual);
         return out_proj.forward(g, ctx);
     }
+    const size_t q_rope = g.rope(q, head_dim), k_rope = g.rope(k, head_dim);
     const size_t q4 = g.reshape(q_rope, {batch, seq, num_heads, head_dim});
     const size_t k4 = g.reshape(k_rope, {batch, seq, num_kv_heads, head_dim});
     const size_t v4 = g.reshape(v, {batch, seq, num_kv_heads, head_dim});

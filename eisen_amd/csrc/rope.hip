@@ -5,14 +5,10 @@
 #include "device_utils.cuh"
 #include "runtime.h"
 
-namespace {
-
-constexpr int kThreads = 256;
-
 // cos/sin table [seq][head_dim/2] as float2, built on the host with the libm routines the CPU
 // arm uses (theta = pos / 10000^(2p/hd); src/graph/ops/transform.rs:559-561), so the device
 // rotates by exactly the same angles.
-int get_rope_table(eisen_ctx* ctx, size_t seq, size_t head_dim, const float2** out) {
+int eisen_rope_table_get(eisen_ctx* ctx, size_t seq, size_t head_dim, const float2** out) {
     for (auto& t : ctx->rope_tables)
         if (t.head_dim == head_dim && t.seq >= seq) {
             *out = reinterpret_cast<const float2*>(t.cos_sin);
@@ -38,6 +34,10 @@ int get_rope_table(eisen_ctx* ctx, size_t seq, size_t head_dim, const float2** o
     *out = reinterpret_cast<const float2*>(dev);
     return 0;
 }
+
+namespace {
+
+constexpr int kThreads = 256;
 
 // fwd: y0 = x0 c - x1 s, y1 = x0 s + x1 c;  bwd: dx0 = g0 c + g1 s, dx1 = -g0 s + g1 c
 // (src/graph/ops/transform.rs:562-566, :592-595).  One packet = N/2 pairs of one head.
@@ -80,7 +80,7 @@ int launch_rope(eisen_ctx* ctx, const void* in, void* out, size_t batch, size_t 
                 int accumulate) {
     constexpr int N = Pack<T>::N;
     const float2* table = nullptr;
-    int rc = get_rope_table(ctx, seq, head_dim, &table);
+    int rc = eisen_rope_table_get(ctx, seq, head_dim, &table);
     if (rc) return rc;
     const size_t n_packets = batch * seq * hidden / N;
     const unsigned blocks = (unsigned)std::min<size_t>(256 * 16, eisen_ceil_div(n_packets, kThreads));

@@ -61,6 +61,9 @@ struct eisen_ctx {
     char last_error[512] = {0};
 };
 
+// cos/sin table of the rotary embedding, [seq][head_dim/2] float2 on the device, cached in the context (rope.hip)
+int eisen_rope_table_get(eisen_ctx* ctx, size_t seq, size_t head_dim, const float2** out);
+
 // Brackets the launches issued during its lifetime when profiling is on; free when it is off.
 int eisen_prof_begin(eisen_ctx* ctx, const char* name, double work, bool is_flops);
 void eisen_prof_end(eisen_ctx* ctx, int rec);

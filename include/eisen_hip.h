@@ -251,6 +251,15 @@ int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const void* k, c
                                  size_t S, size_t Hq, size_t Hkv, size_t hd, const long long* q_strides,
                                  const long long* kv_strides, float scale, int causal);
 
+/* eisen_hip_attention_backward for q and k that are rotary-embedded projections, q = rope(q0), k = rope(k0)
+ * (src/nn/attention.rs:316-317 applies `g.rope` to both before the attention chain): dq and dk receive the
+ * gradients of q0 and k0, i.e. the rotary backward (src/graph/ops/transform.rs:592-595) is applied to the f32
+ * results as they are stored instead of in two further passes over dq and dk.  Contiguous [B, S, H, hd]
+ * layouts only; positions are the sequence index. */
+int eisen_hip_attention_rope_backward(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                      const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype,
+                                      size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd, float scale, int causal);
+
 /* ---- embedding ------------------------------------------------------------------------- */
 
 /* gather_f32 (kernels/ops_f32.cu:513; Graph::gather, src/graph/ops/transform.rs:132-324).

@@ -758,6 +758,37 @@ def test_attention_bf16_layout_bhsd_and_non_causal(ctx):
     _attn_case(ctx, BF16, 1, 70, 2, 1, 128, causal=False)
 
 
+@pytest.mark.parametrize("dtype,B,S,Hq,Hkv,hd", [(BF16, 2, 96, 4, 2, 64), (BF16, 1, 100, 8, 2, 64), (BF16, 2, 160, 8, 2, 32), (BF16, 1, 130, 2, 1, 128),
+                                                 (F32, 2, 37, 4, 2, 16)])
+def test_attention_rope_backward(ctx, dtype, B, S, Hq, Hkv, hd):
+    """q = rope(q0), k = rope(k0): the fused backward must return the oracle's attention gradients passed through
+    the oracle's rotary backward (gradients of q0 and k0)."""
+    sd = 1.0 / np.sqrt(hd)
+    q0, do = prep(gen.normal(540, (B, S, Hq * hd), sd), dtype), prep(gen.normal(541, (B, S, Hq, hd), sd), dtype)
+    k0, v = prep(gen.normal(542, (B, S, Hkv * hd), sd), dtype), prep(gen.normal(543, (B, S, Hkv, hd), sd), dtype)
+    scale = np.float32(1.0) / np.sqrt(np.float32(hd))
+    dq0, dk0, dv_, ddo = up(ctx, q0, dtype), up(ctx, k0, dtype), up(ctx, v, dtype), up(ctx, do, dtype)
+    es = 2 if dtype == BF16 else 4
+    dq_, dk_ = ctx.malloc(q0.size * es), ctx.malloc(k0.size * es)
+    ctx.rope(dq0, dq_, dtype, B, S, Hq * hd, hd)
+    ctx.rope(dk0, dk_, dtype, B, S, Hkv * hd, hd)
+    q = dn(ctx, dq_, (B, S, Hq, hd), dtype)   # the rotated inputs exactly as the kernels see them
+    k = dn(ctx, dk_, (B, S, Hkv, hd), dtype)
+    _, edq, edk, edv = oracle_attention(q, k, v, do, scale, True)
+    edq0 = R.rope_bwd(edq.reshape(B, S, Hq * hd), hd)
+    edk0 = R.rope_bwd(edk.reshape(B, S, Hkv * hd), hd)
+    out, lse = ctx.malloc(q.size * 4), ctx.malloc(B * Hq * S * 4)
+    ctx.attention_forward(dq_, dk_, dv_, out, lse, dtype, B, S, Hq, Hkv, hd, float(scale), True)
+    gq, gk, gv = ctx.malloc(q.size * 4), ctx.malloc(k.size * 4), ctx.malloc(k.size * 4)
+    ctx.attention_rope_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, dtype, B, S, Hq, Hkv, hd, float(scale), True)
+    tol = tol_for(dtype)
+    assert_close(dn(ctx, gq, (B, S, Hq * hd), dtype), edq0, tol, "dQ0")
+    assert_close(dn(ctx, gk, (B, S, Hkv * hd), dtype), edk0, tol, "dK0")
+    assert_close(dn(ctx, gv, (B, S, Hkv, hd), dtype), edv, tol, "dV")
+    for x in (dq0, dk0, dv_, ddo, dq_, dk_, out, lse, gq, gk, gv):
+        x.free()
+
+
 def test_attention_config3_full_size_properties(ctx):
     """B8 S1024 Hq16 Hkv4 hd64 bf16 (config 3): too large for the unfused oracle in seconds, so check
     one batch element's heads of one KV group against the oracle (S=1024 is kept), and size-independent
