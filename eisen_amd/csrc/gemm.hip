@@ -412,7 +412,7 @@ __device__ __forceinline__ void barrier_no_fence() {
 }
 
 // For shapes that are whole multiples of the tile in M, N and K (no bounds checks anywhere).
-// PIPE: the operand registers of contraction step st+1 are read while the MFMAs of step st run.
+// PIPE: the operand registers of contraction step st+1 are read between the MFMAs of step st.
 template <int BM, int BN, int BK, int WGM, int WGN, bool A_KC, bool B_KC, typename TC, bool PIPE>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmArgs g) {
     constexpr int WAVES = WGM * WGN, STAGES = 3;
@@ -525,6 +525,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
             for (int i = 0; i < TM; i++) a[0][i] = TA::fragment(As, wm * WM + i * 32, 0, lane);
 #pragma unroll
             for (int j = 0; j < TN; j++) b[0][j] = TB::fragment(Bs, wn * WN + j * 32, 0, lane);
+            constexpr int kReadsStep = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);
+            __builtin_amdgcn_sched_group_barrier(0x100, kReadsStep, 0);  // step 0's reads, so that the read groups below are the next step's
             static_for<KSTEPS>([&](auto st_c) {
                 constexpr int st = decltype(st_c)::value;
                 if (st + 1 < KSTEPS) {
@@ -539,9 +541,15 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
                     for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[st & 1][i], b[st & 1][j], acc[i][j], 0, 0, 0);
                 if (REFILL)
                     issue(next, std::integral_constant<int, st * NLOADS / KSTEPS>{}, std::integral_constant<int, (st + 1) * NLOADS / KSTEPS>{});
+                // pin the order: each MFMA of this step is followed by its share of the next step's operand reads
                 if (st + 1 < KSTEPS) {
-                    constexpr int kReadsStep = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);
-                    __builtin_amdgcn_sched_group_barrier(0x100, kReadsStep, 0);
+                    static_for<TM * TN>([&](auto m_c) {
+                        constexpr int mi = decltype(m_c)::value;
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        constexpr int r_lo = mi * kReadsStep / (TM * TN), r_hi = (mi + 1) * kReadsStep / (TM * TN);
+                        if (r_hi > r_lo) __builtin_amdgcn_sched_group_barrier(0x100, r_hi - r_lo, 0);
+                    });
+                } else {
                     __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
                 }
             });
@@ -669,9 +677,9 @@ void launch_mfma_direct(eisen_ctx* ctx, GemmArgs g, bool a_kc, bool b_kc, int ba
     // grids many N tiles wide walk C in groups of 32 N tiles (measured on the 32000-column lm_head GEMMs: 4 % and
     // 10 % faster than row-major order); narrower grids are a few rounds of workgroups anyway
     g.tile_group = g.N / BN >= 64 ? 32 : 0;
-    // reading step st+1's operand registers under step st's MFMAs gains ~2 % when an operand is k-contiguous and
-    // nothing or less when both take the transposing reads
-    const bool pipe = a_kc || b_kc;
+    // reading step st+1's operand registers between step st's MFMAs gains 2-4 % except in the slab-32 kernels of the
+    // dW shapes (two steps per slab, two or three workgroups per CU already overlapping), where it loses
+    const bool pipe = a_kc || b_kc || BK == 64;
     dim3 grid((unsigned)(g.N / BN), (unsigned)(g.M / BM), (unsigned)(batch * (g.split > 1 ? g.split : 1)));
     constexpr int T = 64 * WGM * WGN;
 #define EISEN_DIRECT(AK, BKC, TC) do { if (pipe) gemm_mfma_direct_kernel<BM, BN, BK, WGM, WGN, AK, BKC, TC, true><<<grid, T, 0, ctx->stream>>>(g); else gemm_mfma_direct_kernel<BM, BN, BK, WGM, WGN, AK, BKC, TC, false><<<grid, T, 0, ctx->stream>>>(g); } while (0)
