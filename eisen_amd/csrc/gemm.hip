@@ -515,6 +515,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
         if (REFILL || kt + 1 < nk) wait_loads_but<NLOADS>();
         else wait_loads_but<0>();
         barrier_no_fence();  // slab kt is complete in LDS; every wave is done with slab kt-1
+        __builtin_amdgcn_s_setprio(2);  // a wave multiplying a slab goes ahead of one still waiting for its loads (worth ~0.3 % of the step)
         const SlabSource next = locate(REFILL ? kt + 2 : kt, stage == 0 ? 2 : stage - 1);
         const bf16_t* As = lds[stage];
         const bf16_t* Bs = lds[stage] + TA::ELEMS;
@@ -568,6 +569,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
             if (REFILL)
                 issue(next, std::integral_constant<int, st * NLOADS / KSTEPS>{}, std::integral_constant<int, (st + 1) * NLOADS / KSTEPS>{});
         });
+        __builtin_amdgcn_s_setprio(0);
         stage = stage == 2 ? 0 : stage + 1;
     };
     int kt = 0;
