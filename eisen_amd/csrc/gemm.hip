@@ -50,6 +50,14 @@ struct GemmArgs {
     const void* gate;
     const void* up;
     void* C2;
+    // Grouped launch (direct kernel, ngroup > 0): blockIdx.x enumerates the tiles of up to 4 products that share M, K and the
+    // operand orders but have their own A, B, C and N; grp_tile_end[p] = number of tiles of products 0..p
+    int ngroup;
+    const void* grp_A[4];
+    const void* grp_B[4];
+    void* grp_C[4];
+    int grp_N[4];
+    int grp_tile_end[4];
     int tile_group;                    // direct kernel: > 0 = N tiles per group of the tile order (see the kernel), 0 = row-major order
     int vec_c;                         // C rows are 16-byte aligned at every 8th column: the epilogue may use 16-byte accesses
     // K made of up to three segments with their own operands, C (+)= sum_s op(A_s) op(B_s): segment 0 is A/B/lda/ldb,
@@ -438,6 +446,22 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
         const int width = min(g.tile_group, n_tiles - grp * g.tile_group);
         mt = within / width;
         nt = grp * g.tile_group + within % width;
+    }
+    if (g.ngroup > 0) {  // which product this tile belongs to (uniform); static indices keep the tables in scalar registers
+        const int t = blockIdx.x;
+        int first = 0;
+        g.A = g.grp_A[0]; g.B = g.grp_B[0]; g.C = g.grp_C[0]; g.N = g.grp_N[0];
+#pragma unroll
+        for (int q = 1; q < 4; q++)
+            if (q < g.ngroup && t >= g.grp_tile_end[q - 1]) {
+                first = g.grp_tile_end[q - 1];
+                g.A = g.grp_A[q]; g.B = g.grp_B[q]; g.C = g.grp_C[q]; g.N = g.grp_N[q];
+            }
+        const int n_tiles = g.N / BN;
+        mt = (t - first) / n_tiles;
+        nt = (t - first) % n_tiles;
+        g.ldc = g.N;
+        if (!B_KC) g.ldb = g.N;
     }
     const int m0 = mt * BM, n0 = nt * BN;
     const int split = g.split > 1 ? g.split : 1;
@@ -919,6 +943,48 @@ extern "C" int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void
         return 0;
     }
     return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, 1, 0, 0, 0, 0, "eisen_hip_gemm_residual", nullptr, R);
+}
+
+extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* const* A, const void* const* B, void* const* C, const size_t* N,
+                                      int dtype_ab, int dtype_c, int trans_a, int trans_b, size_t M, size_t K, int accumulate) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, n >= 1 && n <= 4 && A && B && C && N, EISEN_E_ARG, "eisen_hip_gemm_grouped: 1 to 4 products, no null pointers");
+    // One launch when every product is a whole number of 128x128 tiles of the dW form (bf16 operands stored [K][M] and
+    // [K][N], f32 result) and together they give every CU at least two tiles; otherwise one launch per product.
+    bool grouped = n >= 2 && dtype_ab == EISEN_BF16 && dtype_c == EISEN_F32 && trans_a && !trans_b && M % 128 == 0 && K % 64 == 0 && K > 0 &&
+                   M < (size_t(1) << 30) && K < (size_t(1) << 30);
+    long long tiles = 0;
+    for (size_t p = 0; p < n && grouped; p++) {
+        grouped = A[p] && B[p] && C[p] && N[p] > 0 && N[p] % 128 == 0 && N[p] < (size_t(1) << 30) && eisen_aligned(A[p], 16) && eisen_aligned(B[p], 16) &&
+                  eisen_aligned(C[p], 16);
+        tiles += (long long)(M / 128) * (long long)(N[p] / 128);
+    }
+    if (grouped && tiles >= 512 && tiles < (1ll << 30)) {
+        GemmArgs g{};
+        g.M = (int)M; g.K = (int)K;
+        g.lda = (int)M;
+        g.accumulate = accumulate;
+        g.vec_c = 1;
+        g.ngroup = (int)n;
+        int end = 0;
+        double flops = 0.0;
+        for (size_t p = 0; p < n; p++) {
+            g.grp_A[p] = A[p]; g.grp_B[p] = B[p]; g.grp_C[p] = C[p];
+            g.grp_N[p] = (int)N[p];
+            end += (int)((M / 128) * (N[p] / 128));
+            g.grp_tile_end[p] = end;
+            flops += 2.0 * (double)M * (double)N[p] * (double)K;
+        }
+        EisenProfScope prof(ctx, "gemm_tn_bf16_f32out_128x128x32_grouped", flops, true);
+        gemm_mfma_direct_kernel<128, 128, 32, 2, 2, false, false, float, false><<<dim3((unsigned)end, 1, 1), 256, 0, ctx->stream>>>(g);
+        EISEN_LAUNCH_CHECK(ctx, "eisen_hip_gemm_grouped");
+        return 0;
+    }
+    for (size_t p = 0; p < n; p++) {
+        const int rc = gemm_common(ctx, A[p], B[p], C[p], dtype_ab, dtype_c, trans_a, trans_b, M, N[p], K, 1, 0, 0, 0, accumulate, "eisen_hip_gemm_grouped");
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 extern "C" int eisen_hip_gemm_swiglu_backward(eisen_ctx* ctx, const void* A, const void* B, const void* gate, const void* up, void* dgate,

@@ -259,6 +259,10 @@ void Graph::backward(size_t loss_id) {
         node.backward_fn(*this);
     }
     backward_root_ = (size_t)-1;
+    if (!pending_dw.empty()) {
+        pending_dw.clear();
+        throw Error("backward: a deferred weight gradient was not collected by a matmul_group");
+    }
 }
 
 // ---- elementwise ---------------------------------------------------------------------------------
@@ -380,7 +384,7 @@ size_t Graph::matmul(size_t a, size_t b) {
 // Graph::matmul followed by Graph::add of a residual (src/nn/transformer.rs:36, :47) as one kernel:
 // out = r + a b, with r and out [.., N].  Backward is that of the two ops: dR += dOut, dA += dOut B^T,
 // dB += A^T dOut.
-size_t Graph::matmul_residual(size_t a, size_t b, size_t r) {
+size_t Graph::matmul_residual(size_t a, size_t b, size_t r, bool defer_dw) {
     const std::vector<size_t> sa = at(a).shape, sb = at(b).shape, sr = at(r).shape;
     if (sb.size() != 2 || sa.empty() || sr.empty()) throw Error("matmul_residual: expects a [..,K], b [K,N], r [..,N]");
     const size_t K = sa.back(), M = numel_of(sa) / std::max<size_t>(K, 1), N = sb[1];
@@ -409,8 +413,13 @@ size_t Graph::matmul_residual(size_t a, size_t b, size_t r) {
         }
         Storage& ga = g.grad_for_write(a, &acc);
         g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc), "matmul_residual backward dA");
-        Storage& gb = g.grad_for_write(b, &acc);
-        g.check(eisen_hip_gemm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul_residual backward dB");
+        if (defer_dw && go.dtype == EISEN_BF16 && g.at(b).is_param) {
+            // dOut's buffer (now also dR's) is only added to by nodes that run after the collecting group
+            g.pending_dw.push_back(PendingDW{b, g.compute_data(a).ptr, go.ptr, M, K, N});
+        } else {
+            Storage& gb = g.grad_for_write(b, &acc);
+            g.check(eisen_hip_gemm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul_residual backward dB");
+        }
     });
     return out;
 }
@@ -471,7 +480,7 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r)
 // fewer launches: equally shaped neighbours (K and V, gate and up) run as a batch of two whose "stride" is the
 // distance between the two tensors, forward and for dW; the input gradient of the whole group is one GEMM
 // whose contraction runs over the outputs of all members, written once.
-std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws) {
+std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws, size_t collect_dw) {
     const std::vector<size_t> sa = at(a).shape;
     const size_t n = ws.size();
     const Storage da = compute_data(a);
@@ -536,9 +545,62 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws)
             if (m > 0)
                 g.check(eisen_hip_gemm_ksegments(g.ctx(), m, As, Bs, Ks, ga.ptr, EISEN_BF16, ga.dtype, 0, 1, M, K, acc), "matmul_group backward dA");
         }
-        // dW_i (+)= A^T dY_i, pairs as one launch when both halves exist and are in the same accumulate state
+        // dW_i (+)= A^T dY_i.  First choice: every member, and the deferred gradient this group collects, as one grouped
+        // launch (same rows, same input width, same accumulate state, f32 gradients).
         const Storage xa = g.compute_data(a);
-        for (size_t i = 0; i < n; i++) {
+        PendingDW extra{};
+        bool have_extra = false;
+        for (size_t e = 0; e < g.pending_dw.size(); e++)
+            if (g.pending_dw[e].weight == collect_dw) {
+                extra = g.pending_dw[e];
+                have_extra = true;
+                g.pending_dw.erase(g.pending_dw.begin() + (ptrdiff_t)e);
+                break;
+            }
+        bool done = false;
+        // (a plain pair of equal shapes stays with the batched launch below: the 256x128 tile serves it better)
+        if (all && n + (have_extra ? 1 : 0) >= 3 && n + (have_extra ? 1 : 0) <= 4 && (!have_extra || (extra.rows == M && extra.in == K))) {
+            const void* As[4];
+            const void* Bs[4];
+            void* Cs[4];
+            size_t Ns[4];
+            int accs[4];
+            size_t m = 0;
+            bool same = true;
+            for (size_t i = 0; i < n; i++) {
+                As[m] = xa.ptr;
+                Bs[m] = g.grad_for_read(outs[i]).ptr;
+                Storage& gw = g.grad_for_write(ws[i], &accs[m]);
+                same = same && gw.dtype == EISEN_F32;
+                Cs[m] = gw.ptr;
+                Ns[m] = N[i];
+                m++;
+            }
+            if (have_extra) {
+                As[m] = extra.x;
+                Bs[m] = extra.dy;
+                Storage& gw = g.grad_for_write(extra.weight, &accs[m]);
+                same = same && gw.dtype == EISEN_F32;
+                Cs[m] = gw.ptr;
+                Ns[m] = extra.out;
+                m++;
+            }
+            for (size_t i = 1; i < m; i++) same = same && accs[i] == accs[0];
+            if (same) {
+                g.check(eisen_hip_gemm_grouped(g.ctx(), m, As, Bs, Cs, Ns, EISEN_BF16, EISEN_F32, 1, 0, K, M, accs[0]), "matmul_group backward dW");
+            } else {  // same work, one launch per product (grad_for_write has already been consumed above)
+                for (size_t i = 0; i < m; i++)
+                    g.check(eisen_hip_gemm(g.ctx(), As[i], Bs[i], Cs[i], EISEN_BF16, i < n ? g.at(ws[i]).grad.dtype : g.at(extra.weight).grad.dtype, 1, 0, K,
+                                           Ns[i], M, accs[i]),
+                            "matmul_group backward dW");
+            }
+            done = true;
+        } else if (have_extra) {
+            int acc = 0;
+            Storage& gw = g.grad_for_write(extra.weight, &acc);
+            g.check(eisen_hip_gemm(g.ctx(), extra.x, extra.dy, gw.ptr, EISEN_BF16, gw.dtype, 1, 0, extra.in, extra.out, extra.rows, acc), "deferred dW");
+        }
+        for (size_t i = 0; i < n && !done; i++) {
             if (pair[i] && has[i] && has[i + 1]) {
                 const Storage& go1 = g.grad_for_read(outs[i]);
                 const Storage& go2 = g.grad_for_read(outs[i + 1]);

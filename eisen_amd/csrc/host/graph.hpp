@@ -106,10 +106,13 @@ class Graph {
     size_t silu(size_t a);
     size_t swiglu(size_t gate, size_t up);                      // fused silu(gate) * up
     size_t matmul(size_t a, size_t b);
-    size_t matmul_residual(size_t a, size_t b, size_t r);  // r + a b in one kernel
+    // r + a b in one kernel.  defer_dw: the weight gradient is left for the matmul_group whose `collect_dw` names b (it
+    // runs later in backward and puts b's gradient GEMM into the same launch as its own); backward() fails loudly if
+    // nobody collects it
+    size_t matmul_residual(size_t a, size_t b, size_t r, bool defer_dw = false);
     size_t swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r);  // r + (silu(gate) * up) b; backward forms dgate, dup in the dX GEMM
     // matmuls of one input against 2-3 weights with fewer launches (bf16 graphs; otherwise plain matmuls)
-    std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights);
+    std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights, size_t collect_dw = (size_t)-1);
     size_t matmul_bf16(size_t a, size_t b) { return matmul(a, b); }
     size_t matmul_trans_b(size_t a, size_t b);
     size_t bmm(size_t a, size_t b, bool trans_b);
@@ -147,6 +150,14 @@ class Graph {
     size_t backward_root() const { return backward_root_; }
     size_t backward_epoch() const { return backward_epoch_; }  // counts backward() calls
     bool has_grad(size_t id) { const Tensor& t = at(id); return t.is_param || (t.grad.valid() && t.grad_written); }
+    // A weight-gradient GEMM dW (+)= x^T dy left for a later node of the same backward pass (see matmul_residual)
+    struct PendingDW {
+        size_t weight;
+        const void* x;    // [rows, in] activations the weight multiplied
+        const void* dy;   // [rows, out] gradient of the product
+        size_t rows, in, out;
+    };
+    std::vector<PendingDW> pending_dw;
 
    private:
     eisen_ctx* ctx_;

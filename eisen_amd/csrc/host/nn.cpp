@@ -91,7 +91,9 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
     size_t q, k, v;
     if (fused && !q_proj.has_bias && !k_proj.has_bias && !v_proj.has_bias) {
         // the three projections read the same input: K and V as one launch, one input-gradient GEMM for all
-        const std::vector<size_t> qkv = g.matmul_group(x_id, {q_proj.weight_id, k_proj.weight_id, v_proj.weight_id});
+        // (the group also collects the output projection's weight gradient when that projection defers it: four dW GEMMs, one launch)
+        const bool defer_out = residual != (size_t)-1 && !out_proj.has_bias;
+        const std::vector<size_t> qkv = g.matmul_group(x_id, {q_proj.weight_id, k_proj.weight_id, v_proj.weight_id}, defer_out ? out_proj.weight_id : (size_t)-1);
         q = qkv[0]; k = qkv[1]; v = qkv[2];
         for (size_t t : qkv) g.reinterpret_shape(t, {batch, seq, g.at(t).shape.back()});
     } else {
@@ -103,7 +105,8 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
     if (fused) {
         // one op for the rotary embedding and steps 3-11: head split, GQA repeat, scores, scale, mask, softmax, P V, merge
         const size_t ctx = g.attention_gqa_rope(q, k, v, num_heads, num_kv_heads, scale, causal);
-        if (residual != (size_t)-1 && !out_proj.has_bias) return g.matmul_residual(ctx, out_proj.weight_id, residual);
+        if (residual != (size_t)-1 && !out_proj.has_bias)
+            return g.matmul_residual(ctx, out_proj.weight_id, residual, /*defer_dw=*/!q_proj.has_bias && !k_proj.has_bias && !v_proj.has_bias);
         return out_proj.forward(g, ctx);
     }
     const size_t q_rope = g.rope(q, head_dim), k_rope = g.rope(k, head_dim);

@@ -268,6 +268,15 @@ class Context:
         """C = R + op(A) op(B)."""
         self._call("eisen_hip_gemm_residual", _ptr(A), _ptr(B), _ptr(R), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(M), _sz(N), _sz(K))
 
+    def gemm_grouped(self, As, Bs, Cs, Ns, dtype_ab, dtype_c, trans_a, trans_b, M, K, accumulate=0):
+        """C_p (+)= op(A_p) op(B_p) for up to four products sharing M and K."""
+        n = len(Ns)
+        pa = (_vp * n)(*[_ptr(a) for a in As])
+        pb = (_vp * n)(*[_ptr(b) for b in Bs])
+        pc = (_vp * n)(*[_ptr(c) for c in Cs])
+        pn = (C.c_size_t * n)(*Ns)
+        self._call("eisen_hip_gemm_grouped", _sz(n), pa, pb, pc, pn, _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(M), _sz(K), _i(accumulate))
+
     def gemm_swiglu_backward(self, A, B, gate, up, dgate, dup, dtype, trans_a, trans_b, M, N, K):
         """[dgate, dup] = d(silu(gate) * up) for dH = op(A) op(B)."""
         self._call("eisen_hip_gemm_swiglu_backward", _ptr(A), _ptr(B), _ptr(gate), _ptr(up), _ptr(dgate), _ptr(dup), _i(dtype), _i(trans_a), _i(trans_b),

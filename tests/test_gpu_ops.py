@@ -644,6 +644,23 @@ def test_gemm_swiglu_backward(ctx, M, N, K, dtype):
         x.free()
 
 
+@pytest.mark.parametrize("M,K,Ns", [(2048, 128, (2048, 512, 512, 2048)), (2048, 192, (1024, 3072)), (256, 64, (128, 256, 128))])
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_gemm_grouped_weight_gradients(ctx, M, K, Ns, accumulate):
+    # dW_p (+)= X_p^T dY_p with X_p [K, M] and dY_p [K, N_p] (here K is the token count): the first two shapes run as one
+    # grid of 128x128 tiles, the last one falls back to one launch per product
+    xs = [prep(gen.normal(550 + i, (K, M)), BF16) for i in range(len(Ns))]
+    dys = [prep(gen.normal(560 + i, (K, n)), BF16) for i, n in enumerate(Ns)]
+    c0 = [gen.normal(570 + i, (M, n)).astype(np.float32) for i, n in enumerate(Ns)]
+    dA, dB, dC = [up(ctx, x, BF16) for x in xs], [up(ctx, d, BF16) for d in dys], [up(ctx, c, F32) for c in c0]
+    ctx.gemm_grouped(dA, dB, dC, list(Ns), BF16, F32, 1, 0, M, K, accumulate)
+    for i, n in enumerate(Ns):
+        exp = xs[i].astype(np.float64).T @ dys[i].astype(np.float64) + (c0[i] if accumulate else 0)
+        assert_close(dn(ctx, dC[i], (M, n), F32), exp, 1e-3, f"product {i}")
+    for x in dA + dB + dC:
+        x.free()
+
+
 def test_gemm_f32_matches_oracle_order_tolerance(ctx):
     # config-1 sized linear against the sequential-order f32 oracle, rtol 1e-4
     a, b, go = gen.normal(410, (64, 64)), gen.normal(411, (64, 256), 0.02), gen.normal(412, (64, 256))
