@@ -849,7 +849,9 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     const long long wide_tiles = (long long)(M / 256) * (N / 128) * batch;
     const bool wide = mfma_ok && split == 1 && big_tile && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && wide_tiles >= 256 &&
                       (double)wide_tiles / (double)(256 * ((wide_tiles + 255) / 256)) >= 0.85;
-    const char* tile = !mfma_ok ? "fma64x64" : wide ? (!a_kc && !b_kc && wide_tiles >= 512 ? "256x128x32" : "256x128x64") : (big_tile || split128) ? (K % 64 == 0 && !(!a_kc && !b_kc && M % 128 == 0 && N % 128 == 0 && tiles128 * split >= 512) ? "128x128x64" : "128x128x32") : "64x64x32";
+    const bool wide32 = mfma_ok && split == 1 && n_more == 0 && !a_kc && !b_kc && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 &&
+                        (wide_tiles >= 512 || (wide_tiles >= 300 && !wide));
+    const char* tile = !mfma_ok ? "fma64x64" : wide32 ? "256x128x32" : wide ? "256x128x64" : (big_tile || split128) ? (K % 64 == 0 && !(!a_kc && !b_kc && M % 128 == 0 && N % 128 == 0 && tiles128 * split >= 512) ? "128x128x64" : "128x128x32") : "64x64x32";
     snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
              dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : "");
     EisenProfScope prof(ctx, pname, 2.0 * (double)M * (double)N * (double)K * (double)batch, true);
@@ -866,9 +868,10 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         // straight into three LDS stages is the fastest kernel whenever the shape is a whole number of such tiles
         // and they fill the CUs evenly (it is 5-13 % ahead of the same tile staged through registers); other
         // large shapes run 128x128 with 4 waves, two workgroups per CU.  64x64 is for problems with few tiles.
-        if (wide && !a_kc && !b_kc && wide_tiles >= 512) {
-            // both operands through the (slower) transposing LDS reads and at least two tiles per CU: slabs of 32 need
-            // half the LDS, so two workgroups share a CU and cover each other's barrier waits and epilogues (6-7 % faster)
+        if (wide32) {
+            // both operands through the (slower) transposing LDS reads and more than one tile per CU: slabs of 32 need
+            // half the LDS, so two workgroups share a CU and cover each other's barrier waits and epilogues (6-7 % faster
+            // than slabs of 64; at 352 tiles, the down projection's dW, still 11 % faster than 704 tiles of 128x128x32)
             launch_mfma_direct<256, 128, 32, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else if (wide) {
             launch_mfma_direct<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
@@ -959,7 +962,9 @@ extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* cons
                   eisen_aligned(C[p], 16);
         tiles += (long long)(M / 128) * (long long)(N[p] / 128);
     }
-    if (grouped && tiles >= 512 && tiles < (1ll << 30)) {
+    const bool wide = grouped && M % 256 == 0 && tiles / 2 >= 300;  // 256x128x32 tiles, two workgroups per CU
+    if (grouped && (wide || tiles >= 512) && tiles < (1ll << 30)) {
+        const size_t bm = wide ? 256 : 128;
         GemmArgs g{};
         g.M = (int)M; g.K = (int)K;
         g.lda = (int)M;
@@ -971,12 +976,13 @@ extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* cons
         for (size_t p = 0; p < n; p++) {
             g.grp_A[p] = A[p]; g.grp_B[p] = B[p]; g.grp_C[p] = C[p];
             g.grp_N[p] = (int)N[p];
-            end += (int)((M / 128) * (N[p] / 128));
+            end += (int)((M / bm) * (N[p] / 128));
             g.grp_tile_end[p] = end;
             flops += 2.0 * (double)M * (double)N[p] * (double)K;
         }
-        EisenProfScope prof(ctx, "gemm_tn_bf16_f32out_128x128x32_grouped", flops, true);
-        gemm_mfma_direct_kernel<128, 128, 32, 2, 2, false, false, float, false><<<dim3((unsigned)end, 1, 1), 256, 0, ctx->stream>>>(g);
+        EisenProfScope prof(ctx, wide ? "gemm_tn_bf16_f32out_256x128x32_grouped" : "gemm_tn_bf16_f32out_128x128x32_grouped", flops, true);
+        if (wide) gemm_mfma_direct_kernel<256, 128, 32, 4, 2, false, false, float, false><<<dim3((unsigned)end, 1, 1), 512, 0, ctx->stream>>>(g);
+        else gemm_mfma_direct_kernel<128, 128, 32, 2, 2, false, false, float, false><<<dim3((unsigned)end, 1, 1), 256, 0, ctx->stream>>>(g);
         EISEN_LAUNCH_CHECK(ctx, "eisen_hip_gemm_grouped");
         return 0;
     }
