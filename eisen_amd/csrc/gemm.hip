@@ -604,6 +604,157 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
                                                               m0, n0, wave, wm, wn, lane);
 }
 
+// ---- gate and up projections with the SwiGLU in the epilogue ----------------------------------------
+// G = X Wg, U = X Wu, H = silu(G) * U (src/nn/transformer.rs:41-46) as one kernel: a workgroup multiplies its 256 rows of
+// X against the same 128 columns of both weights, so every A operand register feeds twice as many MFMAs (a 64 x 128
+// wave tile in effect: a sixth fewer LDS reads per MFMA than two separate products), and H is formed from the f32
+// accumulators.  Same machinery as gemm_mfma_direct_kernel: direct-to-LDS loads, three stages, slabs of 32.
+struct SwigluForwardArgs {
+    const bf16_t* X;   // [M, K]
+    const bf16_t* Wg;  // [K, N]
+    const bf16_t* Wu;  // [K, N]
+    bf16_t* G;         // [M, N]
+    bf16_t* U;
+    bf16_t* H;
+    int M, N, K;
+};
+__global__ __launch_bounds__(512) void gemm_swiglu_forward_kernel(SwigluForwardArgs g) {
+    constexpr int BM = 256, BN = 128, BK = 32, WGN = 2, WAVES = 8, STAGES = 3;
+    constexpr int WM = 64, WN = 64, TM = 2, TN = 2, KSTEPS = BK / 16;
+    using TA = DirectOperandTile<BM, true, BK, WAVES>;
+    using TB = DirectOperandTile<BN, false, BK, WAVES>;
+    constexpr int NLOADS = TA::LOADS + 2 * TB::LOADS, STAGE_ELEMS = TA::ELEMS + 2 * TB::ELEMS;
+    __shared__ __attribute__((aligned(1024))) bf16_t lds[STAGES][STAGE_ELEMS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    f32x16 accg[TM][TN], accu[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) { accg[i][j][v] = 0.f; accu[i][j][v] = 0.f; }
+
+    int a_row[TA::LOADS], a_chunk[TA::LOADS], b_row[TB::LOADS], b_chunk[TB::LOADS];
+#pragma unroll
+    for (int i = 0; i < TA::LOADS; i++) TA::lane_chunk(i, wave, lane, a_row[i], a_chunk[i]);
+#pragma unroll
+    for (int i = 0; i < TB::LOADS; i++) TB::lane_chunk(i, wave, lane, b_row[i], b_chunk[i]);
+    // loads h_lo..h_hi-1 of the NLOADS this wave issues per slab: X rows, then the Wg and Wu slabs
+    auto issue = [&](int slab, int stage, auto h_lo_c, auto h_hi_c) {
+        constexpr int h_lo = decltype(h_lo_c)::value, h_hi = decltype(h_hi_c)::value;
+        const int k0 = slab * BK;
+        bf16_t* st = lds[stage];
+#pragma unroll
+        for (int h = h_lo; h < h_hi; h++) {
+            if (h < TA::LOADS) {
+                load_to_lds_16(g.X + (long long)(m0 + a_row[h]) * g.K + k0 + a_chunk[h] * 8, st + TA::lds_block(h, wave));
+            } else {
+                const int hb = (h - TA::LOADS) % TB::LOADS;
+                const bool second = h - TA::LOADS >= TB::LOADS;
+                const bf16_t* W = second ? g.Wu : g.Wg;
+                load_to_lds_16(W + (long long)(k0 + b_row[hb]) * g.N + n0 + b_chunk[hb] * 8, st + TA::ELEMS + (second ? TB::ELEMS : 0) + TB::lds_block(hb, wave));
+            }
+        }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using IN = std::integral_constant<int, NLOADS>;
+    const int nk = g.K / BK;
+    issue(0, 0, I0{}, IN{});
+    if (nk > 1) issue(1, 1, I0{}, IN{});
+    int stage = 0;
+    auto slab = [&](int kt, auto refill_c) {
+        constexpr bool REFILL = decltype(refill_c)::value;
+        if (REFILL || kt + 1 < nk) wait_loads_but<NLOADS>();
+        else wait_loads_but<0>();
+        barrier_no_fence();
+        __builtin_amdgcn_s_setprio(2);
+        const int refill_stage = stage == 0 ? 2 : stage - 1;
+        const bf16_t* As = lds[stage];
+        const bf16_t* Bg = lds[stage] + TA::ELEMS;
+        const bf16_t* Bu = Bg + TB::ELEMS;
+        static_for<KSTEPS>([&](auto st_c) {
+            constexpr int st = decltype(st_c)::value;
+            bf16x8 a[TM], bg[TN], bu[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) a[i] = TA::fragment(As, wm * WM + i * 32, st * 16, lane);
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                bg[j] = TB::fragment(Bg, wn * WN + j * 32, st * 16, lane);
+                bu[j] = TB::fragment(Bu, wn * WN + j * 32, st * 16, lane);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    accg[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], bg[j], accg[i][j], 0, 0, 0);
+                    accu[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], bu[j], accu[i][j], 0, 0, 0);
+                }
+            if (REFILL) issue(kt + 2, refill_stage, std::integral_constant<int, st * NLOADS / KSTEPS>{}, std::integral_constant<int, (st + 1) * NLOADS / KSTEPS>{});
+        });
+        __builtin_amdgcn_s_setprio(0);
+        stage = stage == 2 ? 0 : stage + 1;
+    };
+    int kt = 0;
+    for (; kt + 2 < nk; kt++) slab(kt, std::true_type{});
+    for (; kt < nk; kt++) slab(kt, std::false_type{});
+    barrier_no_fence();  // the staging epilogue reuses the operand LDS
+
+    // Epilogue: as in gemm_store_tile, each wave turns a 32-row band of its accumulators through its private LDS
+    // area so that a lane ends up with 8 consecutive columns of one row; here twice (G, then U) before H is formed.
+    constexpr int SP = WN + 4, LPR = WN / 8, PASSES = 32 * LPR / 64;
+    static_assert(sizeof(lds) >= (size_t)WAVES * 32 * SP * sizeof(float), "staging area does not fit the operand LDS");
+    float* stage_f = reinterpret_cast<float*>(&lds[0][0]) + wave * (32 * SP);
+    const int c = lane & 31, gh = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        float vg[PASSES][8], vu[PASSES][8];
+#pragma unroll
+        for (int which = 0; which < 2; which++) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    stage_f[(8 * (v / 4) + 4 * gh + (v % 4)) * SP + j * 32 + c] = which == 0 ? accg[i][j][v] : accu[i][j][v];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ps++) {
+                const int idx = ps * 64 + lane, r = idx / LPR, cg = idx % LPR;
+                const float4 lo = *reinterpret_cast<const float4*>(stage_f + r * SP + cg * 8);
+                const float4 hi = *reinterpret_cast<const float4*>(stage_f + r * SP + cg * 8 + 4);
+                float* dst = which == 0 ? vg[ps] : vu[ps];
+                dst[0] = lo.x; dst[1] = lo.y; dst[2] = lo.z; dst[3] = lo.w;
+                dst[4] = hi.x; dst[5] = hi.y; dst[6] = hi.z; dst[7] = hi.w;
+            }
+        }
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ps++) {
+            const int idx = ps * 64 + lane, r = idx / LPR, cg = idx % LPR;
+            const long long at = (long long)(m0 + wm * WM + i * 32 + r) * g.N + n0 + wn * WN + cg * 8;
+            bf16x8 og, ou, oh;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                // the outputs the backward pass reads are the rounded ones, so H is formed from them as the separate kernel would
+                og[e] = (bf16_t)vg[ps][e];
+                ou[e] = (bf16_t)vu[ps][e];
+                const float gv = (float)og[e], uv = (float)ou[e];
+                oh[e] = (bf16_t)(gv * (1.0f / (1.0f + __expf(-gv))) * uv);
+            }
+            *reinterpret_cast<bf16x8*>(g.G + at) = og;
+            *reinterpret_cast<bf16x8*>(g.U + at) = ou;
+            *reinterpret_cast<bf16x8*>(g.H + at) = oh;
+        }
+    }
+}
+
 // C += partial[0] + partial[1] + ... in that order, one thread per 4 consecutive elements of a row.
 template <typename TC>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs g, int batch) {
@@ -946,6 +1097,29 @@ extern "C" int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void
         return 0;
     }
     return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, 1, 0, 0, 0, 0, "eisen_hip_gemm_residual", nullptr, R);
+}
+
+extern "C" int eisen_hip_gemm_swiglu_forward(eisen_ctx* ctx, const void* X, const void* Wg, const void* Wu, void* G, void* U, void* H, int dtype,
+                                             size_t M, size_t N, size_t K) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, X && Wg && Wu && G && U && H, EISEN_E_ARG, "eisen_hip_gemm_swiglu_forward: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_gemm_swiglu_forward: unknown dtype %d", dtype);
+    if (M * N == 0) return 0;
+    const bool fused = dtype == EISEN_BF16 && M % 256 == 0 && N % 128 == 0 && K % 32 == 0 && K >= 32 && (M / 256) * (N / 128) >= 256 &&
+                       M < (size_t(1) << 30) && N < (size_t(1) << 30) && K < (size_t(1) << 30) && eisen_aligned(X, 16) && eisen_aligned(Wg, 16) &&
+                       eisen_aligned(Wu, 16) && eisen_aligned(G, 16) && eisen_aligned(U, 16) && eisen_aligned(H, 16);
+    if (fused) {
+        SwigluForwardArgs a{static_cast<const bf16_t*>(X), static_cast<const bf16_t*>(Wg), static_cast<const bf16_t*>(Wu), static_cast<bf16_t*>(G),
+                            static_cast<bf16_t*>(U),       static_cast<bf16_t*>(H),        (int)M,                          (int)N, (int)K};
+        EisenProfScope prof(ctx, "gemm_nn_bf16_swiglu_256x128x32", 4.0 * (double)M * (double)N * (double)K, true);
+        gemm_swiglu_forward_kernel<<<dim3((unsigned)(N / 128), (unsigned)(M / 256), 1), 512, 0, ctx->stream>>>(a);
+        EISEN_LAUNCH_CHECK(ctx, "eisen_hip_gemm_swiglu_forward");
+        return 0;
+    }
+    int rc = gemm_common(ctx, X, Wg, G, dtype, dtype, 0, 0, M, N, K, 1, 0, 0, 0, 0, "eisen_hip_gemm_swiglu_forward");
+    if (!rc) rc = gemm_common(ctx, X, Wu, U, dtype, dtype, 0, 0, M, N, K, 1, 0, 0, 0, 0, "eisen_hip_gemm_swiglu_forward");
+    if (!rc) rc = eisen_hip_swiglu(ctx, G, U, H, dtype, M * N);
+    return rc;
 }
 
 extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* const* A, const void* const* B, void* const* C, const size_t* N,

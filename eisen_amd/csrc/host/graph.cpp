@@ -428,15 +428,20 @@ size_t Graph::matmul_residual(size_t a, size_t b, size_t r, bool defer_dw) {
 // as one node: forward = the SwiGLU kernel + the residual GEMM; backward = dR (buffer hand-over as in
 // matmul_residual), dW += h^T dOut, and one GEMM whose epilogue turns dH = dOut W^T straight into dgate and dup
 // (dH itself is never stored).
-size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r) {
+size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r, size_t h_in) {
     const std::vector<size_t> sg = at(gate).shape, sb = at(b).shape, sr = at(r).shape;
     if (sb.size() != 2 || sg.empty() || sr.empty() || at(up).shape != sg) throw Error("swiglu_matmul_residual: expects gate/up [..,K], b [K,N], r [..,N]");
     const size_t K = sg.back(), M = numel_of(sg) / std::max<size_t>(K, 1), N = sb[1];
     if (sb[0] != K || sr.back() != N || numel_of(sr) != M * N) throw Error("swiglu_matmul_residual: shapes do not match: " + shape_str(sg) + " x " + shape_str(sb) + " + " + shape_str(sr));
     const Storage dg = compute_data(gate), du = compute_data(up), db = compute_data(b), dr = compute_data(r);
     if (dg.dtype != du.dtype || dg.dtype != db.dtype || dr.dtype != dg.dtype) throw Error("swiglu_matmul_residual: operands have different element types");
-    const size_t h = push_tensor(sg, dg.dtype, true);  // kept for dW
-    check(eisen_hip_swiglu(ctx_, dg.ptr, du.ptr, at(h).data.ptr, dg.dtype, dg.numel), "swiglu");
+    size_t h = h_in;  // kept for dW
+    if (h == (size_t)-1) {
+        h = push_tensor(sg, dg.dtype, true);
+        check(eisen_hip_swiglu(ctx_, dg.ptr, du.ptr, at(h).data.ptr, dg.dtype, dg.numel), "swiglu");
+    } else if (numel_of(at(h).shape) != dg.numel || at(h).data.dtype != dg.dtype) {
+        throw Error("swiglu_matmul_residual: h does not match gate and up");
+    }
     const size_t out = push_tensor(sr, dg.dtype, true);
     check(eisen_hip_gemm_residual(ctx_, at(h).data.ptr, db.ptr, dr.ptr, at(out).data.ptr, dg.dtype, dg.dtype, 0, 0, M, N, K), "swiglu_matmul_residual");
     record({gate, up, b, r}, out, [=](Graph& g) {
@@ -480,7 +485,7 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r)
 // fewer launches: equally shaped neighbours (K and V, gate and up) run as a batch of two whose "stride" is the
 // distance between the two tensors, forward and for dW; the input gradient of the whole group is one GEMM
 // whose contraction runs over the outputs of all members, written once.
-std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws, size_t collect_dw) {
+std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws, size_t collect_dw, size_t* swiglu_h) {
     const std::vector<size_t> sa = at(a).shape;
     const size_t n = ws.size();
     const Storage da = compute_data(a);
@@ -491,6 +496,7 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
     if (!ok) {
         std::vector<size_t> outs;
         for (size_t w : ws) outs.push_back(matmul(a, w));
+        if (swiglu_h) *swiglu_h = (size_t)-1;
         return outs;
     }
     const size_t K = sa.back(), M = numel_of(sa) / std::max<size_t>(K, 1);
@@ -506,7 +512,15 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
         if (!(i > 0 && pair[i - 1]) && at(ws[i]).shape == at(ws[i + 1]).shape &&
             congruent(compute_data(ws[i]).ptr, compute_data(ws[i + 1]).ptr, 2) && congruent(at(outs[i]).data.ptr, at(outs[i + 1]).data.ptr, 2))
             pair[i] = 1;
-    for (size_t i = 0; i < n; i++) {
+    // shapes whose gate|up + SwiGLU kernel exists (eisen_hip_gemm_swiglu_forward would otherwise run three launches
+    // where the batched pair below and the SwiGLU kernel are two)
+    const bool with_h = swiglu_h && n == 2 && N[0] == N[1] && M % 256 == 0 && N[0] % 128 == 0 && K % 32 == 0 && (M / 256) * (N[0] / 128) >= 256;
+    if (swiglu_h) *swiglu_h = with_h ? push_tensor({M, N[0]}, da.dtype, true) : (size_t)-1;
+    if (with_h)
+        check(eisen_hip_gemm_swiglu_forward(ctx_, da.ptr, compute_data(ws[0]).ptr, compute_data(ws[1]).ptr, at(outs[0]).data.ptr, at(outs[1]).data.ptr,
+                                            at(*swiglu_h).data.ptr, da.dtype, M, N[0], K),
+              "matmul_group");
+    for (size_t i = 0; i < n && !with_h; i++) {
         const Storage w = compute_data(ws[i]);
         if (pair[i]) {
             const ptrdiff_t wd = ((const char*)compute_data(ws[i + 1]).ptr - (const char*)w.ptr) / 2;

@@ -110,9 +110,11 @@ class Graph {
     // runs later in backward and puts b's gradient GEMM into the same launch as its own); backward() fails loudly if
     // nobody collects it
     size_t matmul_residual(size_t a, size_t b, size_t r, bool defer_dw = false);
-    size_t swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r);  // r + (silu(gate) * up) b; backward forms dgate, dup in the dX GEMM
+    // r + (silu(gate) * up) b; backward forms dgate, dup in the dX GEMM.  h: silu(gate) * up where a matmul_group has
+    // already formed it.
+    size_t swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r, size_t h = (size_t)-1);
     // matmuls of one input against 2-3 weights with fewer launches (bf16 graphs; otherwise plain matmuls)
-    std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights, size_t collect_dw = (size_t)-1);
+    std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights, size_t collect_dw = (size_t)-1, size_t* swiglu_h = nullptr);
     size_t matmul_bf16(size_t a, size_t b) { return matmul(a, b); }
     size_t matmul_trans_b(size_t a, size_t b);
     size_t bmm(size_t a, size_t b, bool trans_b);

@@ -170,10 +170,10 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
     }
     const size_t norm2_out = norm2.forward(g, res1);
     size_t gated;
-    size_t gate_id = (size_t)-1, up_id = (size_t)-1;  // set when gate and up are available unfused-multiplied (SwiGLU folded into the down projection node)
+    size_t gate_id = (size_t)-1, up_id = (size_t)-1, h_id = (size_t)-1;  // set when gate and up are available unfused-multiplied (SwiGLU folded into the down projection node)
     if (attn.fused && !ffn_gate.has_bias && !ffn1.has_bias) {
-        // gate and up projections as one launch, then the fused SwiGLU
-        const std::vector<size_t> guv = g.matmul_group(norm2_out, {ffn_gate.weight_id, ffn1.weight_id});
+        // gate and up projections as one launch that also forms silu(gate) * up where the down projection consumes it
+        const std::vector<size_t> guv = g.matmul_group(norm2_out, {ffn_gate.weight_id, ffn1.weight_id}, (size_t)-1, !ffn2.has_bias ? &h_id : nullptr);
         const std::pair<size_t, size_t> gu{guv[0], guv[1]};
         const std::vector<size_t> ns = g.at(norm2_out).shape;
         if (ns.size() == 3) {
@@ -198,7 +198,7 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
         const size_t up = ffn1.forward(g, norm2_out);
         gated = g.mul(gate, up);
     }
-    if (gate_id != (size_t)-1) return g.swiglu_matmul_residual(gate_id, up_id, ffn2.weight_id, res1);  // SwiGLU + down projection + residual
+    if (gate_id != (size_t)-1) return g.swiglu_matmul_residual(gate_id, up_id, ffn2.weight_id, res1, h_id);  // SwiGLU + down projection + residual
     if (attn.fused && !ffn2.has_bias) return g.matmul_residual(gated, ffn2.weight_id, res1);  // down projection + residual
     const size_t ffn2_out = ffn2.forward(g, gated);
     return g.add(res1, ffn2_out);

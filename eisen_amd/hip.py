@@ -277,6 +277,10 @@ class Context:
         pn = (C.c_size_t * n)(*Ns)
         self._call("eisen_hip_gemm_grouped", _sz(n), pa, pb, pc, pn, _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(M), _sz(K), _i(accumulate))
 
+    def gemm_swiglu_forward(self, X, Wg, Wu, G, U, H, dtype, M, N, K):
+        """G = X Wg, U = X Wu, H = silu(G) * U."""
+        self._call("eisen_hip_gemm_swiglu_forward", _ptr(X), _ptr(Wg), _ptr(Wu), _ptr(G), _ptr(U), _ptr(H), _i(dtype), _sz(M), _sz(N), _sz(K))
+
     def gemm_swiglu_backward(self, A, B, gate, up, dgate, dup, dtype, trans_a, trans_b, M, N, K):
         """[dgate, dup] = d(silu(gate) * up) for dH = op(A) op(B)."""
         self._call("eisen_hip_gemm_swiglu_backward", _ptr(A), _ptr(B), _ptr(gate), _ptr(up), _ptr(dgate), _ptr(dup), _i(dtype), _i(trans_a), _i(trans_b),

@@ -221,6 +221,12 @@ int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void* B, const 
 int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* const* A, const void* const* B, void* const* C, const size_t* N,
                            int dtype_ab, int dtype_c, int trans_a, int trans_b, size_t M, size_t K, int accumulate);
 
+/* G = X Wg, U = X Wu, H = silu(G) * U: the gate and up projections of the feed-forward block and their SwiGLU
+ * (src/nn/transformer.rs:41-46: `ffn_gate.forward`, `g.silu`, `ffn1.forward`, `g.mul`) as one kernel.  X [M, K],
+ * Wg, Wu [K, N], G, U, H [M, N] of `dtype`; G and U are written because the backward pass reads them. */
+int eisen_hip_gemm_swiglu_forward(eisen_ctx* ctx, const void* X, const void* Wg, const void* Wu, void* G, void* U, void* H, int dtype,
+                                  size_t M, size_t N, size_t K);
+
 /* [dgate, dup] = d(silu(gate) * up) for dH = op(A) * op(B): the input gradient of the down projection
  * (src/graph/ops/linear.rs:269-277, dA = dC B^T) followed by the backward of `g.mul(g.silu(gate), up)`
  * (src/nn/transformer.rs:44-46; src/graph/ops/elementwise.rs:442-455 silu, :294-331 mul) in one kernel: dH is

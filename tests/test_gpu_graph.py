@@ -239,6 +239,13 @@ def test_config5_block_shape_bf16_mixed_step(ctx):
     _train_steps(ctx, cfg, G.BF16_MIXED, 2, 128, steps=1, accum=1, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
 
 
+def test_wide_ffn_bf16_mixed_step(ctx):
+    """2048 tokens through a 128 -> 4096 -> 128 feed-forward block: large enough for the kernel that forms gate, up and
+    silu(gate) * up in one launch and for the wide-tile GEMMs behind it; head_dim 64, 2:1 GQA."""
+    cfg = dict(vocab=256, hidden=128, heads=2, kv_heads=1, ffn=4096, layers=1, tie=False)
+    _train_steps(ctx, cfg, G.BF16_MIXED, 4, 512, steps=1, accum=1, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
+
+
 def test_grad_accumulation_invariants_on_gpu(ctx):
     # tests/test_grad_accum.rs: additivity (:59-98), g_accum = N g_full (:108-166), clear_activations keeps
     # parameter gradients, zero_grad, tape emptied, tensor count back at the watermark

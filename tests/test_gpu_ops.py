@@ -644,6 +644,27 @@ def test_gemm_swiglu_backward(ctx, M, N, K, dtype):
         x.free()
 
 
+@pytest.mark.parametrize("M,N,K,dtype", [(4096, 2048, 32, BF16), (4096, 2048, 64, BF16), (2048, 4096, 160, BF16), (512, 384, 96, BF16), (200, 72, 40, BF16),
+                                         (64, 48, 32, F32)])
+def test_gemm_swiglu_forward(ctx, M, N, K, dtype):
+    # G = X Wg, U = X Wu, H = silu(G) * U; the first three shapes take the kernel that forms all three, the others the
+    # separate launches
+    x, wg, wu = prep(gen.normal(530, (M, K)), dtype), prep(gen.normal(531, (K, N), 0.2), dtype), prep(gen.normal(532, (K, N), 0.2), dtype)
+    d = [up(ctx, a, dtype) for a in (x, wg, wu)]
+    es = 2 if dtype == BF16 else 4
+    outs = [ctx.malloc(M * N * es) for _ in range(3)]
+    ctx.gemm_swiglu_forward(d[0], d[1], d[2], outs[0], outs[1], outs[2], dtype, M, N, K)
+    tol = 2e-2 if dtype == BF16 else 2e-4
+    G, U, H = (dn(ctx, o, (M, N), dtype) for o in outs)
+    assert_close(G, x.astype(np.float64) @ wg.astype(np.float64), tol, "gate")
+    assert_close(U, x.astype(np.float64) @ wu.astype(np.float64), tol, "up")
+    # H is formed from the stored (rounded) gate and up, as the separate SwiGLU kernel forms it
+    g64 = G.astype(np.float64)
+    assert_close(H, g64 / (1.0 + np.exp(-g64)) * U.astype(np.float64), 1e-2 if dtype == BF16 else 1e-5, "h")
+    for a in d + outs:
+        a.free()
+
+
 @pytest.mark.parametrize("M,K,Ns", [(2048, 128, (2048, 512, 512, 2048)), (2048, 192, (1024, 3072)), (256, 64, (128, 256, 128))])
 @pytest.mark.parametrize("accumulate", [0, 1])
 def test_gemm_grouped_weight_gradients(ctx, M, K, Ns, accumulate):
