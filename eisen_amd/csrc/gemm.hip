@@ -33,6 +33,7 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+constexpr int kMaxGroup = 8;  // products of one grouped launch
 struct GemmArgs {
     const void* A;
     const void* B;
@@ -50,14 +51,14 @@ struct GemmArgs {
     const void* gate;
     const void* up;
     void* C2;
-    // Grouped launch (direct kernel, ngroup > 0): blockIdx.x enumerates the tiles of up to 4 products that share M, K and the
-    // operand orders but have their own A, B, C and N; grp_tile_end[p] = number of tiles of products 0..p
+    // Grouped launch (direct kernel, ngroup > 0): blockIdx.x enumerates the tiles of up to kMaxGroup products that share M, K
+    // and the operand orders but have their own A, B, C and N; grp_tile_end[p] = number of tiles of products 0..p
     int ngroup;
-    const void* grp_A[4];
-    const void* grp_B[4];
-    void* grp_C[4];
-    int grp_N[4];
-    int grp_tile_end[4];
+    const void* grp_A[kMaxGroup];
+    const void* grp_B[kMaxGroup];
+    void* grp_C[kMaxGroup];
+    int grp_N[kMaxGroup];
+    int grp_tile_end[kMaxGroup];
     int tile_group;                    // direct kernel: > 0 = N tiles per group of the tile order (see the kernel), 0 = row-major order
     int vec_c;                         // C rows are 16-byte aligned at every 8th column: the epilogue may use 16-byte accesses
     // K made of up to three segments with their own operands, C (+)= sum_s op(A_s) op(B_s): segment 0 is A/B/lda/ldb,
@@ -452,7 +453,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
         int first = 0;
         g.A = g.grp_A[0]; g.B = g.grp_B[0]; g.C = g.grp_C[0]; g.N = g.grp_N[0];
 #pragma unroll
-        for (int q = 1; q < 4; q++)
+        for (int q = 1; q < kMaxGroup; q++)
             if (q < g.ngroup && t >= g.grp_tile_end[q - 1]) {
                 first = g.grp_tile_end[q - 1];
                 g.A = g.grp_A[q]; g.B = g.grp_B[q]; g.C = g.grp_C[q]; g.N = g.grp_N[q];
@@ -1125,7 +1126,7 @@ extern "C" int eisen_hip_gemm_swiglu_forward(eisen_ctx* ctx, const void* X, cons
 extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* const* A, const void* const* B, void* const* C, const size_t* N,
                                       int dtype_ab, int dtype_c, int trans_a, int trans_b, size_t M, size_t K, int accumulate) {
     EISEN_CHECK_CTX(ctx);
-    EISEN_REQUIRE(ctx, n >= 1 && n <= 4 && A && B && C && N, EISEN_E_ARG, "eisen_hip_gemm_grouped: 1 to 4 products, no null pointers");
+    EISEN_REQUIRE(ctx, n >= 1 && n <= (size_t)kMaxGroup && A && B && C && N, EISEN_E_ARG, "eisen_hip_gemm_grouped: 1 to 8 products, no null pointers");
     // One launch when every product is a whole number of 128x128 tiles of the dW form (bf16 operands stored [K][M] and
     // [K][N], f32 result) and together they give every CU at least two tiles; otherwise one launch per product.
     bool grouped = n >= 2 && dtype_ab == EISEN_BF16 && dtype_c == EISEN_F32 && trans_a && !trans_b && M % 128 == 0 && K % 64 == 0 && K > 0 &&

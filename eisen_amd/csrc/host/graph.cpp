@@ -485,7 +485,7 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r,
 // fewer launches: equally shaped neighbours (K and V, gate and up) run as a batch of two whose "stride" is the
 // distance between the two tensors, forward and for dW; the input gradient of the whole group is one GEMM
 // whose contraction runs over the outputs of all members, written once.
-std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws, size_t collect_dw, size_t* swiglu_h) {
+std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws, const std::vector<size_t>& collect_dw, size_t* swiglu_h, bool defer_dw) {
     const std::vector<size_t> sa = at(a).shape;
     const size_t n = ws.size();
     const Storage da = compute_data(a);
@@ -559,44 +559,55 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
             if (m > 0)
                 g.check(eisen_hip_gemm_ksegments(g.ctx(), m, As, Bs, Ks, ga.ptr, EISEN_BF16, ga.dtype, 0, 1, M, K, acc), "matmul_group backward dA");
         }
-        // dW_i (+)= A^T dY_i.  First choice: every member, and the deferred gradient this group collects, as one grouped
+        // dW_i (+)= A^T dY_i.  First choice: every member, and the deferred gradients this group collects, as one grouped
         // launch (same rows, same input width, same accumulate state, f32 gradients).
         const Storage xa = g.compute_data(a);
-        PendingDW extra{};
-        bool have_extra = false;
-        for (size_t e = 0; e < g.pending_dw.size(); e++)
-            if (g.pending_dw[e].weight == collect_dw) {
-                extra = g.pending_dw[e];
-                have_extra = true;
-                g.pending_dw.erase(g.pending_dw.begin() + (ptrdiff_t)e);
-                break;
+        if (defer_dw && all && collect_dw.empty()) {
+            // only products that the grouped launch takes as wide tiles are worth the wait: small ones are served better by
+            // the batched pair below
+            bool params = K % 256 == 0 && M % 64 == 0;
+            size_t wide_tiles = 0;
+            for (size_t i = 0; i < n; i++) {
+                params = params && g.at(ws[i]).is_param && N[i] % 128 == 0 && g.at(ws[i]).grad.dtype == EISEN_F32;
+                wide_tiles += (K / 256) * (N[i] / 128);
             }
+            if (params && wide_tiles >= 300) {
+                for (size_t i = 0; i < n; i++) g.pending_dw.push_back(PendingDW{ws[i], xa.ptr, g.grad_for_read(outs[i]).ptr, M, K, N[i]});
+                return;
+            }
+        }
+        std::vector<PendingDW> extras;
+        for (size_t e = 0; e < g.pending_dw.size();) {
+            if (std::find(collect_dw.begin(), collect_dw.end(), g.pending_dw[e].weight) != collect_dw.end()) {
+                extras.push_back(g.pending_dw[e]);
+                g.pending_dw.erase(g.pending_dw.begin() + (ptrdiff_t)e);
+            } else {
+                e++;
+            }
+        }
         bool done = false;
+        bool fits = all && n + extras.size() >= 3 && n + extras.size() <= 8;
+        for (const PendingDW& e : extras) fits = fits && e.rows == M && e.in == K;
         // (a plain pair of equal shapes stays with the batched launch below: the 256x128 tile serves it better)
-        if (all && n + (have_extra ? 1 : 0) >= 3 && n + (have_extra ? 1 : 0) <= 4 && (!have_extra || (extra.rows == M && extra.in == K))) {
-            const void* As[4];
-            const void* Bs[4];
-            void* Cs[4];
-            size_t Ns[4];
-            int accs[4];
+        if (fits) {
+            const void* As[8];
+            const void* Bs[8];
+            void* Cs[8];
+            size_t Ns[8];
+            int accs[8];
+            int dts[8];
             size_t m = 0;
             bool same = true;
-            for (size_t i = 0; i < n; i++) {
-                As[m] = xa.ptr;
-                Bs[m] = g.grad_for_read(outs[i]).ptr;
-                Storage& gw = g.grad_for_write(ws[i], &accs[m]);
+            for (size_t i = 0; i < n + extras.size(); i++) {
+                const bool own = i < n;
+                const size_t w = own ? ws[i] : extras[i - n].weight;
+                As[m] = own ? xa.ptr : extras[i - n].x;
+                Bs[m] = own ? g.grad_for_read(outs[i]).ptr : extras[i - n].dy;
+                Storage& gw = g.grad_for_write(w, &accs[m]);
                 same = same && gw.dtype == EISEN_F32;
+                dts[m] = gw.dtype;
                 Cs[m] = gw.ptr;
-                Ns[m] = N[i];
-                m++;
-            }
-            if (have_extra) {
-                As[m] = extra.x;
-                Bs[m] = extra.dy;
-                Storage& gw = g.grad_for_write(extra.weight, &accs[m]);
-                same = same && gw.dtype == EISEN_F32;
-                Cs[m] = gw.ptr;
-                Ns[m] = extra.out;
+                Ns[m] = own ? N[i] : extras[i - n].out;
                 m++;
             }
             for (size_t i = 1; i < m; i++) same = same && accs[i] == accs[0];
@@ -604,15 +615,15 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
                 g.check(eisen_hip_gemm_grouped(g.ctx(), m, As, Bs, Cs, Ns, EISEN_BF16, EISEN_F32, 1, 0, K, M, accs[0]), "matmul_group backward dW");
             } else {  // same work, one launch per product (grad_for_write has already been consumed above)
                 for (size_t i = 0; i < m; i++)
-                    g.check(eisen_hip_gemm(g.ctx(), As[i], Bs[i], Cs[i], EISEN_BF16, i < n ? g.at(ws[i]).grad.dtype : g.at(extra.weight).grad.dtype, 1, 0, K,
-                                           Ns[i], M, accs[i]),
-                            "matmul_group backward dW");
+                    g.check(eisen_hip_gemm(g.ctx(), As[i], Bs[i], Cs[i], EISEN_BF16, dts[i], 1, 0, K, Ns[i], M, accs[i]), "matmul_group backward dW");
             }
             done = true;
-        } else if (have_extra) {
-            int acc = 0;
-            Storage& gw = g.grad_for_write(extra.weight, &acc);
-            g.check(eisen_hip_gemm(g.ctx(), extra.x, extra.dy, gw.ptr, EISEN_BF16, gw.dtype, 1, 0, extra.in, extra.out, extra.rows, acc), "deferred dW");
+        } else {
+            for (const PendingDW& e : extras) {
+                int acc = 0;
+                Storage& gw = g.grad_for_write(e.weight, &acc);
+                g.check(eisen_hip_gemm(g.ctx(), e.x, e.dy, gw.ptr, EISEN_BF16, gw.dtype, 1, 0, e.in, e.out, e.rows, acc), "deferred dW");
+            }
         }
         for (size_t i = 0; i < n && !done; i++) {
             if (pair[i] && has[i] && has[i + 1]) {

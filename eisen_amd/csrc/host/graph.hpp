@@ -113,8 +113,12 @@ class Graph {
     // r + (silu(gate) * up) b; backward forms dgate, dup in the dX GEMM.  h: silu(gate) * up where a matmul_group has
     // already formed it.
     size_t swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r, size_t h = (size_t)-1);
-    // matmuls of one input against 2-3 weights with fewer launches (bf16 graphs; otherwise plain matmuls)
-    std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights, size_t collect_dw = (size_t)-1, size_t* swiglu_h = nullptr);
+    // matmuls of one input against 2-3 weights with fewer launches (bf16 graphs; otherwise plain matmuls).
+    // collect_dw: weights whose deferred gradient GEMMs join this group's dW launch; defer_dw: this group's own weight
+    // gradients are left for a later group that names them; swiglu_h: receives the id of silu(out0) * out1 when the
+    // kernel that forms it with the two products ran, (size_t)-1 otherwise
+    std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights, const std::vector<size_t>& collect_dw = {}, size_t* swiglu_h = nullptr,
+                                     bool defer_dw = false);
     size_t matmul_bf16(size_t a, size_t b) { return matmul(a, b); }
     size_t matmul_trans_b(size_t a, size_t b);
     size_t bmm(size_t a, size_t b, bool trans_b);

@@ -84,16 +84,18 @@ GroupedQueryAttention::GroupedQueryAttention(Graph& g, size_t hidden, size_t hea
 }
 
 // GroupedQueryAttention::forward_with_mask (src/nn/attention.rs:289-388).
-size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool causal, size_t residual) const {
+size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool causal, size_t residual, const std::vector<size_t>& collect_dw) const {
     const std::vector<size_t> xs = g.at(x_id).shape;
     if (xs.size() != 3) throw Error("GQA requires [Batch, Seq, Dim]");
     const size_t batch = xs[0], seq = xs[1];
     size_t q, k, v;
-    if (fused && !q_proj.has_bias && !k_proj.has_bias && !v_proj.has_bias) {
+    if (collects()) {
         // the three projections read the same input: K and V as one launch, one input-gradient GEMM for all
         // (the group also collects the output projection's weight gradient when that projection defers it: four dW GEMMs, one launch)
         const bool defer_out = residual != (size_t)-1 && !out_proj.has_bias;
-        const std::vector<size_t> qkv = g.matmul_group(x_id, {q_proj.weight_id, k_proj.weight_id, v_proj.weight_id}, defer_out ? out_proj.weight_id : (size_t)-1);
+        std::vector<size_t> collect = collect_dw;
+        if (defer_out) collect.insert(collect.begin(), out_proj.weight_id);
+        const std::vector<size_t> qkv = g.matmul_group(x_id, {q_proj.weight_id, k_proj.weight_id, v_proj.weight_id}, collect);
         q = qkv[0]; k = qkv[1]; v = qkv[2];
         for (size_t t : qkv) g.reinterpret_shape(t, {batch, seq, g.at(t).shape.back()});
     } else {
@@ -162,8 +164,11 @@ TransformerBlock::TransformerBlock(Graph& g, size_t hidden, size_t heads, size_t
 size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) const {
     const size_t norm1_out = norm1.forward(g, x_id);
     size_t res1;
+    bool defer_ffn = false;
     if (attn.fused && !attn.out_proj.has_bias) {
-        res1 = attn.forward_with_mask(g, norm1_out, causal, x_id);  // the output projection adds the residual itself
+        // the output projection adds the residual itself; the weight gradients of gate and up wait for the Q/K/V group
+        defer_ffn = attn.collects() && !ffn_gate.has_bias && !ffn1.has_bias;
+        res1 = attn.forward_with_mask(g, norm1_out, causal, x_id, defer_ffn ? std::vector<size_t>{ffn_gate.weight_id, ffn1.weight_id} : std::vector<size_t>{});
     } else {
         const size_t attn_out = attn.forward_with_mask(g, norm1_out, causal);
         res1 = g.add(x_id, attn_out);
@@ -173,7 +178,7 @@ size_t TransformerBlock::forward_with_mask(Graph& g, size_t x_id, bool causal) c
     size_t gate_id = (size_t)-1, up_id = (size_t)-1, h_id = (size_t)-1;  // set when gate and up are available unfused-multiplied (SwiGLU folded into the down projection node)
     if (attn.fused && !ffn_gate.has_bias && !ffn1.has_bias) {
         // gate and up projections as one launch that also forms silu(gate) * up where the down projection consumes it
-        const std::vector<size_t> guv = g.matmul_group(norm2_out, {ffn_gate.weight_id, ffn1.weight_id}, (size_t)-1, !ffn2.has_bias ? &h_id : nullptr);
+        const std::vector<size_t> guv = g.matmul_group(norm2_out, {ffn_gate.weight_id, ffn1.weight_id}, {}, !ffn2.has_bias ? &h_id : nullptr, defer_ffn);
         const std::pair<size_t, size_t> gu{guv[0], guv[1]};
         const std::vector<size_t> ns = g.at(norm2_out).shape;
         if (ns.size() == 3) {

@@ -57,7 +57,10 @@ struct GroupedQueryAttention : Module {
     GroupedQueryAttention(Graph& g, size_t hidden_dim, size_t num_heads, size_t num_kv_heads);
     // residual != npos (fused path only): the output projection also adds this tensor, i.e. the result is
     // residual + attention(x) as the transformer block computes it
-    size_t forward_with_mask(Graph& g, size_t x_id, bool causal, size_t residual = (size_t)-1) const;
+    // residual: added by the output projection's kernel.  collect_dw: weights of later layers of the same block whose
+    // deferred gradient GEMMs join the Q/K/V group's launch; collects() says whether this call would take them.
+    size_t forward_with_mask(Graph& g, size_t x_id, bool causal, size_t residual = (size_t)-1, const std::vector<size_t>& collect_dw = {}) const;
+    bool collects() const { return fused && !q_proj.has_bias && !k_proj.has_bias && !v_proj.has_bias; }
     size_t forward(Graph& g, size_t x_id) const override { return forward_with_mask(g, x_id, true); }
     std::vector<size_t> params() const override;
 };

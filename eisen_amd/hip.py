@@ -269,7 +269,7 @@ class Context:
         self._call("eisen_hip_gemm_residual", _ptr(A), _ptr(B), _ptr(R), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(M), _sz(N), _sz(K))
 
     def gemm_grouped(self, As, Bs, Cs, Ns, dtype_ab, dtype_c, trans_a, trans_b, M, K, accumulate=0):
-        """C_p (+)= op(A_p) op(B_p) for up to four products sharing M and K."""
+        """C_p (+)= op(A_p) op(B_p) for up to eight products sharing M and K."""
         n = len(Ns)
         pa = (_vp * n)(*[_ptr(a) for a in As])
         pb = (_vp * n)(*[_ptr(b) for b in Bs])

@@ -214,10 +214,10 @@ int eisen_hip_gemm_strided_batched(eisen_ctx* ctx, const void* A, const void* B,
 int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void* B, const void* R, void* C, int dtype_ab, int dtype_c,
                             int trans_a, int trans_b, size_t M, size_t N, size_t K);
 
-/* C_p (+)= op(A_p) * op(B_p) for p < n <= 4: products that share M, K, the operand orders and the element types but
+/* C_p (+)= op(A_p) * op(B_p) for p < n <= 8: products that share M, K, the operand orders and the element types but
  * have their own operands, outputs and N_p.  Stands for n calls of the matmul backward's dB GEMM
- * (src/graph/ops/linear.rs:279-287), e.g. the weight gradients of the Q, K, V and output projections of one
- * attention block; they run as one grid when that fills the chip better than the separate launches. */
+ * (src/graph/ops/linear.rs:279-287), e.g. the weight gradients of the Q, K, V, output, gate and up projections of one
+ * transformer block; they run as one grid when that fills the chip better than the separate launches. */
 int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* const* A, const void* const* B, void* const* C, const size_t* N,
                            int dtype_ab, int dtype_c, int trans_a, int trans_b, size_t M, size_t K, int accumulate);
 

@@ -246,6 +246,14 @@ def test_wide_ffn_bf16_mixed_step(ctx):
     _train_steps(ctx, cfg, G.BF16_MIXED, 4, 512, steps=1, accum=1, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
 
 
+def test_deferred_weight_gradients_bf16_mixed_step(ctx):
+    """Two layers whose gate and up projections are wide enough (256 -> 19200) for their weight gradients to wait for the
+    Q/K/V group of the block and run with the Q, K, V and output projections' as one grouped launch; two accumulated
+    micro-batches, so the launch also runs in its accumulating form."""
+    cfg = dict(vocab=256, hidden=256, heads=4, kv_heads=2, ffn=19200, layers=2, tie=False)
+    _train_steps(ctx, cfg, G.BF16_MIXED, 2, 128, steps=1, accum=2, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
+
+
 def test_grad_accumulation_invariants_on_gpu(ctx):
     # tests/test_grad_accum.rs: additivity (:59-98), g_accum = N g_full (:108-166), clear_activations keeps
     # parameter gradients, zero_grad, tape emptied, tensor count back at the watermark
