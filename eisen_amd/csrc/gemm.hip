@@ -422,8 +422,12 @@ __device__ __forceinline__ void barrier_no_fence() {
 
 // For shapes that are whole multiples of the tile in M, N and K (no bounds checks anywhere).
 // PIPE: the operand registers of contraction step st+1 are read between the MFMAs of step st.
-template <int BM, int BN, int BK, int WGM, int WGN, bool A_KC, bool B_KC, typename TC, bool PIPE>
+// SWIGLU_BWD: an instantiation of its own for the launches with the SwiGLU-backward epilogue (the epilogue itself is
+// chosen by g.gate in every instantiation), so that a kernel trace lists them apart from the plain products: they run
+// beside a weight-gradient GEMM on the side stream, which stretches their durations.
+template <int BM, int BN, int BK, int WGM, int WGN, bool A_KC, bool B_KC, typename TC, bool PIPE, bool SWIGLU_BWD = false>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmArgs g) {
+    if (SWIGLU_BWD && !g.gate) return;
     constexpr int WAVES = WGM * WGN, STAGES = 3;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -1005,7 +1009,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
                         (wide_tiles >= 512 || (wide_tiles >= 300 && !wide));
     const char* tile = !mfma_ok ? "fma64x64" : wide32 ? "256x128x32" : wide ? "256x128x64" : (big_tile || split128) ? (K % 64 == 0 && !(!a_kc && !b_kc && M % 128 == 0 && N % 128 == 0 && tiles128 * split >= 512) ? "128x128x64" : "128x128x32") : "64x64x32";
     snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
-             dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : "");
+             dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : swiglu ? "_swiglu_bwd" : "");
     EisenProfScope prof(ctx, pname, 2.0 * (double)M * (double)N * (double)K * (double)batch, true);
     if (mfma_ok) {
         if (split > 1) {
@@ -1025,6 +1029,9 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
             // half the LDS, so two workgroups share a CU and cover each other's barrier waits and epilogues (6-7 % faster
             // than slabs of 64; at 352 tiles, the down projection's dW, still 11 % faster than 704 tiles of 128x128x32)
             launch_mfma_direct<256, 128, 32, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+        } else if (wide && swiglu && a_kc && b_kc && dtype_c == EISEN_BF16 && batch == 1) {
+            g.tile_group = g.N / 128 >= 64 ? 32 : 0;
+            gemm_mfma_direct_kernel<256, 128, 64, 4, 2, true, true, bf16_t, true, true><<<dim3((unsigned)(g.N / 128), (unsigned)(g.M / 256), 1), 512, 0, ctx->stream>>>(g);
         } else if (wide) {
             launch_mfma_direct<256, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else if (big_tile || split128) {

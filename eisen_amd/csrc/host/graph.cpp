@@ -217,7 +217,13 @@ Storage& Graph::grad_for_write(size_t id, int* accumulate) {
         *accumulate = t.grad_written ? 1 : 0;
     }
     t.grad_written = true;
+    if (!side_guards.empty() && std::find(side_guards.begin(), side_guards.end(), t.grad.ptr) != side_guards.end()) side_join();
     return t.grad;
+}
+
+void Graph::side_join() {
+    check(eisen_hip_side_wait(ctx_), "side stream join");
+    side_guards.clear();
 }
 
 const Storage& Graph::grad_for_read(size_t id) {
@@ -259,6 +265,7 @@ void Graph::backward(size_t loss_id) {
         node.backward_fn(*this);
     }
     backward_root_ = (size_t)-1;
+    side_join();
     if (!pending_dw.empty()) {
         pending_dw.clear();
         throw Error("backward: a deferred weight gradient was not collected by a matmul_group");
@@ -459,6 +466,17 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r,
             if (gr.ptr == go.ptr) throw Error("swiglu_matmul_residual backward: a second backward pass over the same activations is not supported");
             g.check(eisen_hip_accumulate(g.ctx(), gr.ptr, go.ptr, go.dtype, M * N, acc), "swiglu_matmul_residual backward dR");
         }
+        // large products only: a small one gains nothing from running beside the chain
+        const bool side = go.dtype == EISEN_BF16 && g.at(b).is_param && K % 256 == 0 && N % 128 == 0 && M % 64 == 0 && (K / 256) * (N / 128) >= 128;
+        if (side) {
+            // dB beside the input-gradient chain: it reads h and dOut; dOut's buffer (now dR's) is next written by whoever
+            // accumulates into dR, and that write waits (grad_for_write)
+            g.check(eisen_hip_side_begin(g.ctx()), "side stream");
+            Storage& gb = g.grad_for_write(b, &acc);
+            g.check(eisen_hip_gemm(g.ctx(), g.at(h).data.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "swiglu_matmul_residual backward dB");
+            g.check(eisen_hip_side_end(g.ctx()), "side stream");
+            g.side_guards.push_back(go.ptr);
+        }
         int ag = 0, au = 0;
         Storage& gg = g.grad_for_write(gate, &ag);
         Storage& gu = g.grad_for_write(up, &au);
@@ -474,8 +492,10 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r,
                     "swiglu_matmul_residual backward");
             g.device_free(dh);
         }
-        Storage& gb = g.grad_for_write(b, &acc);
-        g.check(eisen_hip_gemm(g.ctx(), g.at(h).data.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "swiglu_matmul_residual backward dB");
+        if (!side) {
+            Storage& gb = g.grad_for_write(b, &acc);
+            g.check(eisen_hip_gemm(g.ctx(), g.at(h).data.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "swiglu_matmul_residual backward dB");
+        }
     });
     return out;
 }

@@ -164,6 +164,10 @@ class Graph {
         size_t rows, in, out;
     };
     std::vector<PendingDW> pending_dw;
+    // buffers that GEMMs on the context's side stream are still reading: the first node that asks to write one of them waits
+    // for those GEMMs
+    std::vector<const void*> side_guards;
+    void side_join();
 
    private:
     eisen_ctx* ctx_;

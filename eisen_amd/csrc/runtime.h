@@ -35,7 +35,10 @@ struct eisen_prof {
 
 struct eisen_ctx {
     int device = 0;
-    hipStream_t stream = nullptr;
+    hipStream_t stream = nullptr;       // the stream every entry point launches on (the side stream between side_begin and side_end)
+    hipStream_t main_stream = nullptr, side_stream = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_side = nullptr;
+    bool side_active = false, side_pending = false;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     bool timer_running = false;
     // size-keyed free lists in front of hipMallocAsync (exact-size buckets, like the

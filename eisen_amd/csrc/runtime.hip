@@ -28,6 +28,10 @@ extern "C" int eisen_hip_init(int device, eisen_ctx** out) {
     ctx->device = device;
     // default priority, non-blocking with respect to the legacy null stream
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    ctx->main_stream = ctx->stream;
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->ev_side, hipEventDisableTiming);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev_start);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev_stop);
     if (e == hipSuccess) {
@@ -60,6 +64,8 @@ extern "C" int eisen_hip_pool_trim(eisen_ctx* ctx) {
 extern "C" int eisen_hip_destroy(eisen_ctx* ctx) {
     EISEN_CHECK_CTX(ctx);
     (void)hipSetDevice(ctx->device);
+    ctx->stream = ctx->main_stream;
+    (void)hipStreamSynchronize(ctx->side_stream);
     (void)hipStreamSynchronize(ctx->stream);
     (void)eisen_hip_pool_trim(ctx);
     for (auto& kv : ctx->live) (void)hipFreeAsync(kv.first, ctx->stream);
@@ -73,14 +79,46 @@ extern "C" int eisen_hip_destroy(eisen_ctx* ctx) {
     for (hipEvent_t e : ctx->prof.pool) (void)hipEventDestroy(e);
     (void)hipEventDestroy(ctx->ev_start);
     (void)hipEventDestroy(ctx->ev_stop);
+    (void)hipEventDestroy(ctx->ev_fork);
+    (void)hipEventDestroy(ctx->ev_side);
+    (void)hipStreamDestroy(ctx->side_stream);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return 0;
 }
 
+// Work issued between side_begin and side_end runs on a second stream, after everything issued before side_begin and
+// concurrently with what the main stream is given next; side_wait makes the main stream wait for it.
+extern "C" int eisen_hip_side_begin(eisen_ctx* ctx) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, !ctx->side_active, EISEN_E_ARG, "eisen_hip_side_begin: already on the side stream");
+    EISEN_HIP_TRY(ctx, hipEventRecord(ctx->ev_fork, ctx->main_stream));
+    EISEN_HIP_TRY(ctx, hipStreamWaitEvent(ctx->side_stream, ctx->ev_fork, 0));
+    ctx->stream = ctx->side_stream;
+    ctx->side_active = true;
+    return 0;
+}
+extern "C" int eisen_hip_side_end(eisen_ctx* ctx) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, ctx->side_active, EISEN_E_ARG, "eisen_hip_side_end: not on the side stream");
+    ctx->stream = ctx->main_stream;
+    ctx->side_active = false;
+    EISEN_HIP_TRY(ctx, hipEventRecord(ctx->ev_side, ctx->side_stream));
+    ctx->side_pending = true;
+    return 0;
+}
+extern "C" int eisen_hip_side_wait(eisen_ctx* ctx) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, !ctx->side_active, EISEN_E_ARG, "eisen_hip_side_wait: still on the side stream");
+    if (ctx->side_pending) EISEN_HIP_TRY(ctx, hipStreamWaitEvent(ctx->main_stream, ctx->ev_side, 0));
+    ctx->side_pending = false;
+    return 0;
+}
+
 extern "C" int eisen_hip_stream_sync(eisen_ctx* ctx) {
     EISEN_CHECK_CTX(ctx);
-    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->side_pending || ctx->side_active) EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->side_stream));
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->main_stream));
     return 0;
 }
 

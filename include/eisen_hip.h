@@ -55,6 +55,14 @@ int eisen_hip_destroy(eisen_ctx* ctx);
 const char* eisen_hip_last_error(eisen_ctx* ctx);
 /* stream.synchronize() (e.g. src/graph/mod.rs:776-788). */
 int eisen_hip_stream_sync(eisen_ctx* ctx);
+/* A second stream of the context for work whose result nothing on the main stream needs soon (a weight-gradient GEMM
+ * beside the input-gradient chain): calls between side_begin and side_end are ordered after everything issued before
+ * side_begin and run concurrently with what is issued after side_end; side_wait orders the main stream after them
+ * (eisen_hip_stream_sync waits for both).  Buffers the side work reads must not be written or freed before side_wait.
+ * No counterpart in the reference, which runs one stream (src/graph/mod.rs:776-788). */
+int eisen_hip_side_begin(eisen_ctx* ctx);
+int eisen_hip_side_end(eisen_ctx* ctx);
+int eisen_hip_side_wait(eisen_ctx* ctx);
 /* The hipStream_t of the context, as void*, for callers that enqueue their own work. */
 void* eisen_hip_stream(eisen_ctx* ctx);
 
