@@ -264,6 +264,10 @@ class Context:
         self._call("eisen_hip_gemm_strided_batched", _ptr(A), _ptr(B), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(batch),
                    _sz(M), _sz(N), _sz(K), C.c_longlong(stride_a), C.c_longlong(stride_b), C.c_longlong(stride_c), _i(accumulate))
 
+    def side_begin(self): self._call("eisen_hip_side_begin")
+    def side_end(self): self._call("eisen_hip_side_end")
+    def side_wait(self): self._call("eisen_hip_side_wait")
+
     def gemm_residual(self, A, B, R, Cbuf, dtype_ab, dtype_c, trans_a, trans_b, M, N, K):
         """C = R + op(A) op(B)."""
         self._call("eisen_hip_gemm_residual", _ptr(A), _ptr(B), _ptr(R), _ptr(Cbuf), _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(M), _sz(N), _sz(K))

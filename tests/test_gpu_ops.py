@@ -665,6 +665,30 @@ def test_gemm_swiglu_forward(ctx, M, N, K, dtype):
         a.free()
 
 
+def test_side_stream_orders_after_fork_and_before_join(ctx):
+    # main: a = x w1; side (after the fork): c = a w2, beside main: b = x w3; after the join main reads c: d = c + b
+    M, K, N = 512, 256, 384
+    x, w1, w2, w3 = (prep(gen.normal(580 + i, s, 0.3), BF16) for i, s in enumerate(((M, K), (K, K), (K, N), (K, N))))
+    dx, dw1, dw2, dw3 = (up(ctx, a, BF16) for a in (x, w1, w2, w3))
+    a, b, c, d = ctx.malloc(M * K * 2), ctx.malloc(M * N * 2), ctx.malloc(M * N * 2), ctx.malloc(M * N * 2)
+    for rep in range(3):
+        ctx.gemm(dx, dw1, a, BF16, BF16, 0, 0, M, K, K)
+        ctx.side_begin()
+        ctx.gemm(a, dw2, c, BF16, BF16, 0, 0, M, N, K)
+        ctx.side_end()
+        ctx.gemm(dx, dw3, b, BF16, BF16, 0, 0, M, N, K)
+        ctx.side_wait()
+        ctx.add(c, b, d, BF16, M * N)
+    got = dn(ctx, d, (M, N), BF16)
+    a64 = hip.round_bf16((x.astype(np.float64) @ w1.astype(np.float64)).astype(np.float32)).astype(np.float64)
+    exp = a64 @ w2.astype(np.float64) + x.astype(np.float64) @ w3.astype(np.float64)
+    assert_close(got, exp, 2e-2, "side stream")
+    with pytest.raises(hip.EisenHipError):
+        ctx.side_end()          # not on the side stream
+    for t in (dx, dw1, dw2, dw3, a, b, c, d):
+        t.free()
+
+
 @pytest.mark.parametrize("M,K,Ns", [(2048, 128, (2048, 512, 512, 2048)), (2048, 192, (1024, 3072)), (256, 64, (128, 256, 128))])
 @pytest.mark.parametrize("accumulate", [0, 1])
 def test_gemm_grouped_weight_gradients(ctx, M, K, Ns, accumulate):
