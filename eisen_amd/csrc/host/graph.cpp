@@ -56,6 +56,7 @@ Graph::Graph(eisen_ctx* ctx, PrecisionMode mode) : precision_mode(mode), ctx_(ct
 }
 
 Graph::~Graph() {
+    (void)eisen_hip_side_wait(ctx_);
     for (auto& t : tensors) release(t);
 }
 
@@ -188,6 +189,7 @@ void Graph::reinterpret_shape(size_t id, const std::vector<size_t>& shape) {
 // Graph::restore_save_point / clear_activations (src/graph/mod.rs:336-365, :432-435): buffers go
 // back to the size-keyed pool inside the runtime.
 void Graph::restore_save_point(size_t save_point) {
+    if (!side_guards.empty()) side_join();  // a backward pass that threw may have left side-stream work reading these buffers
     while (tensors.size() > save_point) {
         release(tensors.back());
         tensors.pop_back();
@@ -471,11 +473,13 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r,
         if (side) {
             // dB beside the input-gradient chain: it reads h and dOut; dOut's buffer (now dR's) is next written by whoever
             // accumulates into dR, and that write waits (grad_for_write)
-            g.check(eisen_hip_side_begin(g.ctx()), "side stream");
             Storage& gb = g.grad_for_write(b, &acc);
-            g.check(eisen_hip_gemm(g.ctx(), g.at(h).data.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "swiglu_matmul_residual backward dB");
-            g.check(eisen_hip_side_end(g.ctx()), "side stream");
+            g.check(eisen_hip_side_begin(g.ctx()), "side stream");
+            const int rc = eisen_hip_gemm(g.ctx(), g.at(h).data.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc);
+            const int rc_end = eisen_hip_side_end(g.ctx());  // back on the main stream whatever the GEMM returned
             g.side_guards.push_back(go.ptr);
+            g.check(rc, "swiglu_matmul_residual backward dB");
+            g.check(rc_end, "side stream");
         }
         int ag = 0, au = 0;
         Storage& gg = g.grad_for_write(gate, &ag);
