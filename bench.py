@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c3|c2]
 
-Default workload c5 = BASELINE config 5: the "~1.1B" Llama-style model (vocab 32000, d 2048,
+Default workload c5 = the headline configuration (config 5): the "~1.1B" Llama-style model (vocab 32000, d 2048,
 16 layers, 32 query / 8 KV heads, head_dim 64, SiLU-gated MLP 5632, untied lm_head), seq 1024,
 micro-batch 4, gradient accumulation 8 (32,768 tokens per optimiser step), bf16 activations and
 matmuls, f32 master weights and AdamW state, synthetic Zipf(1.1) token ids, N(0, 0.02) weights.
