@@ -89,23 +89,26 @@ __global__ __launch_bounds__(kBwdThreads) void rms_norm_bwd_kernel(const T* __re
     }
     // the next row's packets are requested before the current row is reduced, so a wave always has
     // two rows of loads in flight
-    Pack<T> xp[MAXP], gp[MAXP], xn[MAXP], gn[MAXP];
-    auto fetch = [&](size_t row, Pack<T>* xd, Pack<T>* gd) {
+    // (the row of gx an accumulating call adds to travels with them: requested after the row reduction it would cost
+    // every row a second memory latency)
+    Pack<T> xp[MAXP], gp[MAXP], op[MAXP], xn[MAXP], gn[MAXP], on[MAXP];
+    auto fetch = [&](size_t row, Pack<T>* xd, Pack<T>* gd, Pack<T>* od) {
 #pragma unroll
         for (int p = 0; p < MAXP; p++) {
             const int c = (p * kWave + lane) * N;
             if (c < dim) {
                 xd[p] = load_pack(x + row * dim + c);
                 gd[p] = load_pack(go + row * dim + c);
+                if (accumulate_x) od[p] = load_pack(gx + row * dim + c);
             }
         }
     };
-    if (wave_global < rows) fetch(wave_global, xp, gp);
+    if (wave_global < rows) fetch(wave_global, xp, gp, op);
     for (size_t row = wave_global; row < rows; row += wave_stride) {
         T* gxr = gx + row * dim;
         const float rrms = rrms_in[row];
         const size_t next = row + wave_stride;
-        if (next < rows) fetch(next, xn, gn);
+        if (next < rows) fetch(next, xn, gn, on);
         float gdxw = 0.f;
 #pragma unroll
         for (int p = 0; p < MAXP; p++) {
@@ -121,8 +124,7 @@ __global__ __launch_bounds__(kBwdThreads) void rms_norm_bwd_kernel(const T* __re
         for (int p = 0; p < MAXP; p++) {
             const int c = (p * kWave + lane) * N;
             if (c < dim) {
-                Pack<T> o;
-                if (accumulate_x) o = load_pack(gxr + c);
+                Pack<T> o = op[p];
 #pragma unroll
                 for (int j = 0; j < N; j++) {
                     const float xv = xp[p].get(j), gv = gp[p].get(j);
@@ -137,6 +139,7 @@ __global__ __launch_bounds__(kBwdThreads) void rms_norm_bwd_kernel(const T* __re
         for (int p = 0; p < MAXP; p++) {
             xp[p] = xn[p];
             gp[p] = gn[p];
+            op[p] = on[p];
         }
     }
     // combine the block's waves in a fixed order
