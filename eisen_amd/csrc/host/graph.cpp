@@ -190,6 +190,7 @@ void Graph::reinterpret_shape(size_t id, const std::vector<size_t>& shape) {
 // back to the size-keyed pool inside the runtime.
 void Graph::restore_save_point(size_t save_point) {
     if (!side_guards.empty()) side_join();  // a backward pass that threw may have left side-stream work reading these buffers
+    flush_norm_dw(false);                   // ... and partial rows nobody will finish
     while (tensors.size() > save_point) {
         release(tensors.back());
         tensors.pop_back();
@@ -221,6 +222,27 @@ Storage& Graph::grad_for_write(size_t id, int* accumulate) {
     t.grad_written = true;
     if (!side_guards.empty() && std::find(side_guards.begin(), side_guards.end(), t.grad.ptr) != side_guards.end()) side_join();
     return t.grad;
+}
+
+void Graph::flush_norm_dw(bool compute) {
+    if (pending_norm_dw.empty()) return;
+    std::vector<PendingNormDW> list;
+    list.swap(pending_norm_dw);
+    int rc = 0;
+    if (compute) {
+        std::vector<const float*> parts;
+        std::vector<float*> gws;
+        std::vector<size_t> nrows;
+        for (const PendingNormDW& e : list) {
+            if (e.nrows == 0) continue;
+            parts.push_back((const float*)e.partial.ptr);
+            gws.push_back((float*)at(e.weight).grad.ptr);
+            nrows.push_back(e.nrows);
+        }
+        if (!parts.empty()) rc = eisen_hip_rms_norm_dw_finish(ctx_, parts.size(), parts.data(), gws.data(), nrows.data(), list[0].dim);
+    }
+    for (PendingNormDW& e : list) device_free(e.partial);
+    check(rc, "rms_norm gain gradients");
 }
 
 void Graph::side_join() {
@@ -267,6 +289,7 @@ void Graph::backward(size_t loss_id) {
         node.backward_fn(*this);
     }
     backward_root_ = (size_t)-1;
+    flush_norm_dw(true);
     side_join();
     if (!pending_dw.empty()) {
         pending_dw.clear();
@@ -935,9 +958,21 @@ size_t Graph::rms_norm(size_t x, size_t w, float eps) {
         g.materialize_grad(w);
         Tensor& tw = g.at(w);
         if (!tw.grad.valid() || tw.grad.dtype != EISEN_F32) throw Error("rms_norm backward: the gain needs an f32 gradient buffer");
-        g.check(eisen_hip_rms_norm_backward(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr, (const float*)g.at(rr).data.ptr, go.ptr, gx.ptr,
-                                            (float*)tw.grad.ptr, go.dtype, rows, dim, acc),
-                "rms_norm backward");
+        if (tw.is_param) {
+            // the gain gradient stays in partial rows until the end of the backward pass (flush_norm_dw)
+            bool clash = g.pending_norm_dw.size() >= 64;
+            for (const PendingNormDW& e : g.pending_norm_dw) clash = clash || e.weight == w || e.dim != dim;
+            if (clash) g.flush_norm_dw(true);
+            PendingNormDW e{g.device_alloc((size_t)EISEN_RMS_NORM_PARTIAL_ROWS * dim, EISEN_F32, false), w, 0, dim};
+            const int rc = eisen_hip_rms_norm_backward_partial(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr, (const float*)g.at(rr).data.ptr,
+                                                               go.ptr, gx.ptr, (float*)e.partial.ptr, &e.nrows, go.dtype, rows, dim, acc);
+            g.pending_norm_dw.push_back(e);  // before the check: the buffer is released with the list
+            g.check(rc, "rms_norm backward");
+        } else {
+            g.check(eisen_hip_rms_norm_backward(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr, (const float*)g.at(rr).data.ptr, go.ptr, gx.ptr,
+                                                (float*)tw.grad.ptr, go.dtype, rows, dim, acc),
+                    "rms_norm backward");
+        }
     });
     return out;
 }

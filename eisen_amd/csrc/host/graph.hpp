@@ -167,6 +167,13 @@ class Graph {
     // buffers that GEMMs on the context's side stream are still reading: the first node that asks to write one of them waits
     // for those GEMMs
     std::vector<const void*> side_guards;
+    // gain gradients of RMSNorm nodes left as partial rows during a backward pass; one launch finishes them all at its end
+    struct PendingNormDW {
+        Storage partial;
+        size_t weight, nrows, dim;
+    };
+    std::vector<PendingNormDW> pending_norm_dw;
+    void flush_norm_dw(bool compute);
     void side_join();
 
    private:

@@ -161,8 +161,18 @@ __global__ __launch_bounds__(kBwdThreads) void rms_norm_bwd_kernel(const T* __re
 
 // Second stage: gw[c] += sum over the block rows of `partial`, in a fixed order.  A workgroup owns
 // 32 columns; its 8 row groups each add every 8th partial row, then meet in LDS (group 0..7 in order).
-__global__ __launch_bounds__(256) void rms_norm_dw_reduce_kernel(const float* __restrict__ partial, float* __restrict__ gw, int nblocks, int dim) {
+// blockIdx.y picks one of up to kFinishSlots (partial, gw) pairs: the gains of many norms finish in one launch.
+constexpr int kFinishSlots = 64;
+struct FinishSlots {
+    const float* partial[kFinishSlots];
+    float* gw[kFinishSlots];
+    int nrows[kFinishSlots];
+};
+__global__ __launch_bounds__(256) void rms_norm_dw_reduce_kernel(FinishSlots slots, int dim) {
     __shared__ float sh[8][32];
+    const float* __restrict__ partial = slots.partial[blockIdx.y];
+    float* __restrict__ gw = slots.gw[blockIdx.y];
+    const int nblocks = slots.nrows[blockIdx.y];
     const int cl = threadIdx.x & 31, rg = threadIdx.x >> 5;
     const int c = blockIdx.x * 32 + cl;
     float s = 0.f;
@@ -261,41 +271,58 @@ int rms_norm_fwd(eisen_ctx* ctx, const void* x, const float* w, void* out, float
     return 0;
 }
 
+constexpr unsigned kMaxPartialRows = EISEN_RMS_NORM_PARTIAL_ROWS;
+
 template <typename T, int MAXP>
-int rms_norm_bwd_vec(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* gw,
+int rms_norm_bwd_vec(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* partial, unsigned blocks,
                      size_t rows, size_t dim, int accumulate_x) {
-    // enough waves to cover the chip a few times over, few enough that the partial rows stay small
-    unsigned blocks = (unsigned)std::min<size_t>(eisen_ceil_div(rows, kBwdWaves), 256);
-    void* ws = nullptr;
-    int rc = eisen_workspace(ctx, (size_t)blocks * dim * sizeof(float), &ws);
-    if (rc) return rc;
     const size_t lds = (size_t)kBwdWaves * dim * sizeof(float);
-    rms_norm_bwd_kernel<T, MAXP><<<blocks, kBwdThreads, lds, ctx->stream>>>((const T*)x, w, rrms, (const T*)go, (T*)gx,
-                                                                            (float*)ws, rows, (int)dim, accumulate_x);
+    rms_norm_bwd_kernel<T, MAXP><<<blocks, kBwdThreads, lds, ctx->stream>>>((const T*)x, w, rrms, (const T*)go, (T*)gx, partial, rows, (int)dim,
+                                                                            accumulate_x);
     EISEN_LAUNCH_CHECK(ctx, "rms_norm_bwd_kernel");
-    rms_norm_dw_reduce_kernel<<<(unsigned)eisen_ceil_div(dim, 32), 256, 0, ctx->stream>>>((const float*)ws, gw, (int)blocks, (int)dim);
-    EISEN_LAUNCH_CHECK(ctx, "rms_norm_dw_reduce_kernel");
     return 0;
 }
 
+// dx, and the gain gradient as rows of `partial` ([kMaxPartialRows][dim]); *nrows = rows written.
 template <typename T>
-int rms_norm_bwd(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* gw,
-                 size_t rows, size_t dim, int accumulate_x) {
+int rms_norm_bwd_partial(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* partial, size_t* nrows,
+                         size_t rows, size_t dim, int accumulate_x) {
     constexpr int N = Pack<T>::N;
     const bool vec = dim % N == 0 && eisen_aligned(x, 16) && eisen_aligned(go, 16) && eisen_aligned(gx, 16) && eisen_aligned(w, 16) &&
                      dim <= (size_t)kWave * N * 8 && (size_t)kBwdWaves * dim * sizeof(float) <= 64 * 1024;
     if (vec) {
+        // enough waves to cover the chip a few times over, few enough that the partial rows stay small
+        const unsigned blocks = (unsigned)std::min<size_t>(eisen_ceil_div(rows, kBwdWaves), kMaxPartialRows);
+        *nrows = blocks;
         const size_t packs = eisen_ceil_div(dim, (size_t)kWave * N);
-        if (packs <= 1) return rms_norm_bwd_vec<T, 1>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
-        if (packs <= 2) return rms_norm_bwd_vec<T, 2>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
-        if (packs <= 4) return rms_norm_bwd_vec<T, 4>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
-        return rms_norm_bwd_vec<T, 8>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
+        if (packs <= 1) return rms_norm_bwd_vec<T, 1>(ctx, x, w, rrms, go, gx, partial, blocks, rows, dim, accumulate_x);
+        if (packs <= 2) return rms_norm_bwd_vec<T, 2>(ctx, x, w, rrms, go, gx, partial, blocks, rows, dim, accumulate_x);
+        if (packs <= 4) return rms_norm_bwd_vec<T, 4>(ctx, x, w, rrms, go, gx, partial, blocks, rows, dim, accumulate_x);
+        return rms_norm_bwd_vec<T, 8>(ctx, x, w, rrms, go, gx, partial, blocks, rows, dim, accumulate_x);
     }
     rms_norm_bwd_scalar_kernel<T><<<(unsigned)eisen_ceil_div(rows, kRowWaves), kRowThreads, 0, ctx->stream>>>(
         (const T*)x, w, rrms, (const T*)go, (T*)gx, rows, (int)dim, accumulate_x);
     EISEN_LAUNCH_CHECK(ctx, "rms_norm_bwd_scalar_kernel");
-    rms_norm_dw_scalar_kernel<T><<<(unsigned)eisen_ceil_div(dim, 256), 256, 0, ctx->stream>>>((const T*)x, rrms, (const T*)go, gw, rows, (int)dim);
+    *nrows = 1;  // one thread per column adds its rows in order into a zeroed row
+    int rc = eisen_hip_fill(ctx, partial, EISEN_F32, 0.0f, dim);
+    if (rc) return rc;
+    rms_norm_dw_scalar_kernel<T><<<(unsigned)eisen_ceil_div(dim, 256), 256, 0, ctx->stream>>>((const T*)x, rrms, (const T*)go, partial, rows, (int)dim);
     EISEN_LAUNCH_CHECK(ctx, "rms_norm_dw_scalar_kernel");
+    return 0;
+}
+
+int rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim) {
+    for (size_t first = 0; first < n; first += kFinishSlots) {
+        FinishSlots slots{};
+        const size_t m = std::min<size_t>(kFinishSlots, n - first);
+        for (size_t i = 0; i < m; i++) {
+            slots.partial[i] = partial[first + i];
+            slots.gw[i] = gw[first + i];
+            slots.nrows[i] = (int)nrows[first + i];
+        }
+        rms_norm_dw_reduce_kernel<<<dim3((unsigned)eisen_ceil_div(dim, 32), (unsigned)m, 1), 256, 0, ctx->stream>>>(slots, (int)dim);
+        EISEN_LAUNCH_CHECK(ctx, "rms_norm_dw_reduce_kernel");
+    }
     return 0;
 }
 
@@ -320,8 +347,39 @@ extern "C" int eisen_hip_rms_norm_backward(eisen_ctx* ctx, const void* x, const 
     EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_rms_norm_backward: unknown dtype %d", dtype);
     EISEN_REQUIRE(ctx, dim > 0 && dim < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_rms_norm_backward: dim %zu out of range", dim);
     if (rows == 0) return 0;
-    return dtype == EISEN_F32 ? rms_norm_bwd<float>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x)
-                              : rms_norm_bwd<bf16_t>(ctx, x, w, rrms, go, gx, gw, rows, dim, accumulate_x);
+    // the two-part form with the library's workspace in between
+    void* ws = nullptr;
+    int rc = eisen_workspace(ctx, (size_t)kMaxPartialRows * dim * sizeof(float), &ws);
+    if (rc) return rc;
+    size_t nrows = 0;
+    rc = dtype == EISEN_F32 ? rms_norm_bwd_partial<float>(ctx, x, w, rrms, go, gx, (float*)ws, &nrows, rows, dim, accumulate_x)
+                            : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx, (float*)ws, &nrows, rows, dim, accumulate_x);
+    if (rc) return rc;
+    const float* p = (const float*)ws;
+    return rms_norm_dw_finish(ctx, 1, &p, &gw, &nrows, dim);
+}
+
+extern "C" int eisen_hip_rms_norm_backward_partial(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx,
+                                                   float* partial, size_t* nrows_out, int dtype, size_t rows, size_t dim, int accumulate_x) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, x && w && rrms && go && gx && partial && nrows_out, EISEN_E_ARG, "eisen_hip_rms_norm_backward_partial: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_rms_norm_backward_partial: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, dim > 0 && dim < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_rms_norm_backward_partial: dim %zu out of range", dim);
+    *nrows_out = 0;
+    if (rows == 0) return 0;
+    return dtype == EISEN_F32 ? rms_norm_bwd_partial<float>(ctx, x, w, rrms, go, gx, partial, nrows_out, rows, dim, accumulate_x)
+                              : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx, partial, nrows_out, rows, dim, accumulate_x);
+}
+
+extern "C" int eisen_hip_rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, n == 0 || (partial && gw && nrows), EISEN_E_ARG, "eisen_hip_rms_norm_dw_finish: null pointer");
+    EISEN_REQUIRE(ctx, dim > 0 && dim < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_rms_norm_dw_finish: dim %zu out of range", dim);
+    for (size_t i = 0; i < n; i++) {
+        EISEN_REQUIRE(ctx, partial[i] && gw[i] && nrows[i] <= kMaxPartialRows, EISEN_E_ARG, "eisen_hip_rms_norm_dw_finish: entry %zu is null or has too many rows", i);
+        for (size_t j = 0; j < i; j++) EISEN_REQUIRE(ctx, gw[i] != gw[j], EISEN_E_ARG, "eisen_hip_rms_norm_dw_finish: entries %zu and %zu add to the same gradient", j, i);
+    }
+    return rms_norm_dw_finish(ctx, n, partial, gw, nrows, dim);
 }
 
 extern "C" int eisen_hip_softmax(eisen_ctx* ctx, const void* x, void* out, int dtype, size_t rows, size_t n) {

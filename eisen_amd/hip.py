@@ -232,6 +232,23 @@ class Context:
     def rms_norm_backward(self, x, w, rrms, go, gx, gw, dtype, rows, dim, accumulate_x=0):
         self._call("eisen_hip_rms_norm_backward", _ptr(x), _ptr(w), _ptr(rrms), _ptr(go), _ptr(gx), _ptr(gw), _i(dtype), _sz(rows), _sz(dim), _i(accumulate_x))
 
+    RMS_NORM_PARTIAL_ROWS = 256
+
+    def rms_norm_backward_partial(self, x, w, rrms, go, gx, partial, dtype, rows, dim, accumulate_x=0):
+        """dx, and the gain gradient as rows of `partial` ([RMS_NORM_PARTIAL_ROWS, dim] f32); returns the rows written."""
+        n = C.c_size_t(0)
+        self._call("eisen_hip_rms_norm_backward_partial", _ptr(x), _ptr(w), _ptr(rrms), _ptr(go), _ptr(gx), _ptr(partial), C.byref(n), _i(dtype),
+                   _sz(rows), _sz(dim), _i(accumulate_x))
+        return n.value
+
+    def rms_norm_dw_finish(self, partials, gws, nrows, dim):
+        """gw_i += column sums of the first nrows_i rows of partial_i, all in one launch."""
+        n = len(partials)
+        pp = (_vp * n)(*[_ptr(p) for p in partials])
+        pg = (_vp * n)(*[_ptr(g) for g in gws])
+        pn = (C.c_size_t * n)(*nrows)
+        self._call("eisen_hip_rms_norm_dw_finish", _sz(n), pp, pg, pn, _sz(dim))
+
     def rope(self, x, out, dtype, batch, seq, hidden, head_dim):
         self._call("eisen_hip_rope", _ptr(x), _ptr(out), _i(dtype), _sz(batch), _sz(seq), _sz(hidden), _sz(head_dim))
 

@@ -205,6 +205,35 @@ def test_rms_norm(ctx, dtype, rows, dim):
     assert np.array_equal(dn(ctx, gw2, (dim,), F32), dn(ctx, gw3, (dim,), F32))
 
 
+@pytest.mark.parametrize("dtype,dim", [(BF16, 2048), (F32, 256), (BF16, 100)], ids=["bf16-2048", "f32-256", "bf16-scalar-path"])
+def test_rms_norm_backward_in_two_parts(ctx, dtype, dim):
+    # three norms of different row counts leave their gain gradients as partial rows; one launch finishes them all
+    row_counts = (4096, 300, 7)
+    parts, gws, nrows, exp = [], [], [], []
+    keep = []
+    for i, rows in enumerate(row_counts):
+        x, go = prep(gen.normal(600 + i, (rows, dim), 1.5), dtype), prep(gen.normal(610 + i, (rows, dim)), dtype)
+        w = (1.0 + gen.normal(620 + i, (dim,), 0.2)).astype(np.float32)
+        _, er = R.rms_norm_fwd(x, w, 1e-5)
+        egx, egw = R.rms_norm_bwd(x, w, er, go)
+        dx, dw, dgo, rr = up(ctx, x, dtype), up(ctx, w, F32), up(ctx, go, dtype), ctx.upload(er.astype(np.float32))
+        gx, part = ctx.malloc(x.nbytes), ctx.malloc(ctx.RMS_NORM_PARTIAL_ROWS * dim * 4)
+        gw0 = gen.normal(630 + i, (dim,))
+        gw = ctx.upload(gw0)
+        n = ctx.rms_norm_backward_partial(dx, dw, rr, dgo, gx, part, dtype, rows, dim, 0)
+        assert 1 <= n <= ctx.RMS_NORM_PARTIAL_ROWS
+        assert_close(dn(ctx, gx, x.shape, dtype), egx, tol_for(dtype), f"dx {i}")
+        parts.append(part); gws.append(gw); nrows.append(n); exp.append(gw0 + egw)
+        keep += [dx, dw, dgo, rr, gx]
+    ctx.rms_norm_dw_finish(parts, gws, nrows, dim)
+    for i in range(len(row_counts)):
+        assert_close(dn(ctx, gws[i], (dim,), F32), exp[i], tol_for(dtype) if dtype == BF16 else 2e-4, f"dw {i}")
+    with pytest.raises(hip.EisenHipError):
+        ctx.rms_norm_dw_finish([parts[0], parts[1]], [gws[0], gws[0]], nrows[:2], dim)   # two entries, one gradient
+    for t in keep + parts + gws:
+        t.free()
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
 @pytest.mark.parametrize("b,s,hidden,hd", [(1, 2, 8, 8), (2, 33, 64, 16), (2, 128, 256, 64)])
 def test_rope(ctx, dtype, b, s, hidden, hd):
