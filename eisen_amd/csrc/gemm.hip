@@ -1114,7 +1114,7 @@ extern "C" int eisen_hip_gemm_swiglu_forward(eisen_ctx* ctx, const void* X, cons
     EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_gemm_swiglu_forward: unknown dtype %d", dtype);
     if (M * N == 0) return 0;
     const bool fused = dtype == EISEN_BF16 && M % 256 == 0 && N % 128 == 0 && K % 32 == 0 && K >= 32 && (M / 256) * (N / 128) >= 256 &&
-                       M < (size_t(1) << 30) && N < (size_t(1) << 30) && K < (size_t(1) << 30) && eisen_aligned(X, 16) && eisen_aligned(Wg, 16) &&
+                       M / 256 <= 65535 && M < (size_t(1) << 30) && N < (size_t(1) << 30) && K < (size_t(1) << 30) && eisen_aligned(X, 16) && eisen_aligned(Wg, 16) &&
                        eisen_aligned(Wu, 16) && eisen_aligned(G, 16) && eisen_aligned(U, 16) && eisen_aligned(H, 16);
     if (fused) {
         SwigluForwardArgs a{static_cast<const bf16_t*>(X), static_cast<const bf16_t*>(Wg), static_cast<const bf16_t*>(Wu), static_cast<bf16_t*>(G),
