@@ -1046,8 +1046,7 @@ size_t Graph::attention_gqa_rope(size_t q, size_t k, size_t v, size_t heads, siz
     const Storage dq = compute_data(q), dk = compute_data(k), dv = compute_data(v);
     if (dq.dtype != dk.dtype || dq.dtype != dv.dtype) throw Error("attention_gqa_rope: q, k, v must share an element type");
     const size_t q_rot = push_tensor(sq, dq.dtype, true), k_rot = push_tensor(sk, dk.dtype, true);  // kept for backward
-    check(eisen_hip_rope(ctx_, dq.ptr, at(q_rot).data.ptr, dq.dtype, B, S, sq[2], hd), "rope");
-    check(eisen_hip_rope(ctx_, dk.ptr, at(k_rot).data.ptr, dk.dtype, B, S, sk[2], hd), "rope");
+    check(eisen_hip_rope_pair(ctx_, dq.ptr, at(q_rot).data.ptr, sq[2], dk.ptr, at(k_rot).data.ptr, sk[2], dq.dtype, B, S, hd), "rope");
     const size_t out = alloc_pooled_dtype(sq, dq.dtype);
     const size_t lse = alloc_pooled_dtype({B, heads, S}, EISEN_F32);
     check(eisen_hip_attention_forward(ctx_, at(q_rot).data.ptr, at(k_rot).data.ptr, dv.ptr, at(out).data.ptr, (float*)at(lse).data.ptr, dq.dtype, B, S,

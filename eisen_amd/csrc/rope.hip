@@ -75,6 +75,37 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ in
     }
 }
 
+// The forward rotation of two tensors that share batch, seq and head_dim (the q and k projections of an attention block)
+// as one launch: packets [0, n0) belong to the first tensor, the rest to the second.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void rope_pair_kernel(const T* __restrict__ in0, T* __restrict__ out0, size_t n0, int hidden0,
+                                                             const T* __restrict__ in1, T* __restrict__ out1, size_t n1, int hidden1,
+                                                             const float2* __restrict__ table, int seq, int head_dim) {
+    constexpr int N = Pack<T>::N;
+    const int half = head_dim / 2;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n0 + n1; i += (size_t)gridDim.x * blockDim.x) {
+        const bool second = i >= n0;
+        const size_t pk = second ? i - n0 : i;
+        const T* in = second ? in1 : in0;
+        T* out = second ? out1 : out0;
+        const int packets_per_row = (second ? hidden1 : hidden0) / N;
+        const size_t row = pk / packets_per_row;
+        const int col = (int)(pk % packets_per_row) * N;
+        const int pos = (int)(row % seq);
+        const int pair0 = (col % head_dim) / 2;
+        const Pack<T> v = load_pack(in + pk * N);
+        Pack<T> o;
+#pragma unroll
+        for (int j = 0; j < N / 2; j++) {
+            const float2 cs = table[(size_t)pos * half + pair0 + j];
+            const float a = v.get(2 * j), b = v.get(2 * j + 1);
+            o.set(2 * j, a * cs.x - b * cs.y);
+            o.set(2 * j + 1, a * cs.y + b * cs.x);
+        }
+        store_pack(out + pk * N, o);
+    }
+}
+
 template <typename T, bool BWD>
 int launch_rope(eisen_ctx* ctx, const void* in, void* out, size_t batch, size_t seq, size_t hidden, size_t head_dim,
                 int accumulate) {
@@ -172,6 +203,34 @@ extern "C" int eisen_hip_rope(eisen_ctx* ctx, const void* x, void* out, int dtyp
                               size_t head_dim) {
     return rope_common(ctx, x, out, dtype, batch, seq, hidden, head_dim, 0, false);
 }
+extern "C" int eisen_hip_rope_pair(eisen_ctx* ctx, const void* q, void* q_out, size_t hidden_q, const void* k, void* k_out, size_t hidden_k, int dtype,
+                                   size_t batch, size_t seq, size_t head_dim) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, q && q_out && k && k_out, EISEN_E_ARG, "rope_pair: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "rope_pair: unknown dtype %d", dtype);
+    const size_t n = dtype == EISEN_F32 ? 4 : 8;
+    const bool one_launch = head_dim >= 2 && head_dim % n == 0 && hidden_q % head_dim == 0 && hidden_k % head_dim == 0 && hidden_q > 0 && hidden_k > 0 &&
+                            batch * seq > 0 && seq < (size_t(1) << 24) && hidden_q < (size_t(1) << 24) && hidden_k < (size_t(1) << 24) &&
+                            eisen_aligned(q, 16) && eisen_aligned(q_out, 16) && eisen_aligned(k, 16) && eisen_aligned(k_out, 16);
+    if (!one_launch) {  // the single-tensor entry point validates and reports
+        const int rc = eisen_hip_rope(ctx, q, q_out, dtype, batch, seq, hidden_q, head_dim);
+        return rc ? rc : eisen_hip_rope(ctx, k, k_out, dtype, batch, seq, hidden_k, head_dim);
+    }
+    const float2* table = nullptr;
+    const int rc = eisen_rope_table_get(ctx, seq, head_dim, &table);
+    if (rc) return rc;
+    const size_t n0 = batch * seq * hidden_q / n, n1 = batch * seq * hidden_k / n;
+    const unsigned blocks = (unsigned)std::min<size_t>(256 * 16, eisen_ceil_div(n0 + n1, kThreads));
+    if (dtype == EISEN_F32)
+        rope_pair_kernel<float><<<blocks, kThreads, 0, ctx->stream>>>((const float*)q, (float*)q_out, n0, (int)hidden_q, (const float*)k, (float*)k_out, n1,
+                                                                      (int)hidden_k, table, (int)seq, (int)head_dim);
+    else
+        rope_pair_kernel<bf16_t><<<blocks, kThreads, 0, ctx->stream>>>((const bf16_t*)q, (bf16_t*)q_out, n0, (int)hidden_q, (const bf16_t*)k, (bf16_t*)k_out,
+                                                                       n1, (int)hidden_k, table, (int)seq, (int)head_dim);
+    EISEN_LAUNCH_CHECK(ctx, "rope_pair_kernel");
+    return 0;
+}
+
 extern "C" int eisen_hip_rope_backward(eisen_ctx* ctx, const void* go, void* gx, int dtype, size_t batch, size_t seq,
                                        size_t hidden, size_t head_dim, int accumulate) {
     return rope_common(ctx, go, gx, dtype, batch, seq, hidden, head_dim, accumulate, true);

@@ -252,6 +252,9 @@ class Context:
     def rope(self, x, out, dtype, batch, seq, hidden, head_dim):
         self._call("eisen_hip_rope", _ptr(x), _ptr(out), _i(dtype), _sz(batch), _sz(seq), _sz(hidden), _sz(head_dim))
 
+    def rope_pair(self, q, q_out, hidden_q, k, k_out, hidden_k, dtype, batch, seq, head_dim):
+        self._call("eisen_hip_rope_pair", _ptr(q), _ptr(q_out), _sz(hidden_q), _ptr(k), _ptr(k_out), _sz(hidden_k), _i(dtype), _sz(batch), _sz(seq), _sz(head_dim))
+
     def rope_backward(self, go, gx, dtype, batch, seq, hidden, head_dim, accumulate=0):
         self._call("eisen_hip_rope_backward", _ptr(go), _ptr(gx), _i(dtype), _sz(batch), _sz(seq), _sz(hidden), _sz(head_dim), _i(accumulate))
 

@@ -186,6 +186,11 @@ int eisen_hip_rope(eisen_ctx* ctx, const void* x, void* out, int dtype, size_t b
                    size_t head_dim);
 int eisen_hip_rope_backward(eisen_ctx* ctx, const void* go, void* gx, int dtype, size_t batch, size_t seq,
                             size_t hidden, size_t head_dim, int accumulate);
+
+/* eisen_hip_rope of two tensors that share batch, seq and head_dim in one launch: the q and k projections of
+ * GroupedQueryAttention::forward_with_mask (src/nn/attention.rs:304-305, two `g.rope` calls). */
+int eisen_hip_rope_pair(eisen_ctx* ctx, const void* q, void* q_out, size_t hidden_q, const void* k, void* k_out, size_t hidden_k, int dtype,
+                        size_t batch, size_t seq, size_t head_dim);
 /* transpose_0213_f32 / _backward (kernels/ops_f32.cu:694,709; src/graph/ops/transform.rs:7-127):
  * [b, s, h, d] -> [b, h, s, d]; the backward is the same permutation applied to the grad. */
 int eisen_hip_transpose_0213(eisen_ctx* ctx, const void* in, void* out, int dtype, size_t b, size_t s, size_t h,

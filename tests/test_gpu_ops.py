@@ -253,6 +253,23 @@ def test_rope(ctx, dtype, b, s, hidden, hd):
     assert_close(dn(ctx, gx, x.shape, dtype), 2 * R.rope_bwd(go, hd), tol, "rope bwd +=")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=_ids.get)
+def test_rope_pair(ctx, dtype):
+    # q [B, S, 8*32] and k [B, S, 2*32] rotated in one launch = the two separate calls, bit for bit
+    b, s, hd = 2, 48, 32
+    q, k = prep(gen.normal(640, (b, s, 8 * hd)), dtype), prep(gen.normal(641, (b, s, 2 * hd)), dtype)
+    dq, dk = up(ctx, q, dtype), up(ctx, k, dtype)
+    oq, ok, rq, rk = (ctx.malloc(a.nbytes) for a in (q, k, q, k))
+    ctx.rope_pair(dq, oq, 8 * hd, dk, ok, 2 * hd, dtype, b, s, hd)
+    ctx.rope(dq, rq, dtype, b, s, 8 * hd, hd)
+    ctx.rope(dk, rk, dtype, b, s, 2 * hd, hd)
+    assert np.array_equal(dn(ctx, oq, q.shape, dtype), dn(ctx, rq, q.shape, dtype))
+    assert np.array_equal(dn(ctx, ok, k.shape, dtype), dn(ctx, rk, k.shape, dtype))
+    assert_close(dn(ctx, ok, k.shape, dtype), R.rope_fwd(k, hd), tol_for(dtype), "rope pair k")
+    for t in (dq, dk, oq, ok, rq, rk):
+        t.free()
+
+
 def test_rope_reference_vector(ctx):
     # tests/gpu_kernels.rs:485-513
     x = np.ones((1, 2, 4), np.float32)
