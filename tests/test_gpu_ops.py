@@ -752,6 +752,90 @@ def test_gemm_grouped_weight_gradients(ctx, M, K, Ns, accumulate):
         x.free()
 
 
+def _rand_bf16(seed, shape, scale=1.0):
+    """bf16-representable normal values, generated fast enough for the config-5 operand sizes."""
+    return hip.round_bf16(np.random.default_rng(seed).standard_normal(shape, dtype=np.float32) * np.float32(scale))
+
+
+def _check_product(name, C, A, B, rtol, base=None, rows_per_block=256):
+    """C == A @ B (+ base) without forming the product on the host: both checksums (C r against A (B r), s^T C against
+    (s^T A) B, with random +-1 vectors: any wrong, missing or misplaced tile moves one of them by far more than the
+    rounding of C) and one exactly recomputed row per block of `rows_per_block` rows, to the usual element bound."""
+    M, N = C.shape
+    rng = np.random.default_rng(99)
+    r, sgn = rng.choice([-1.0, 1.0], N), rng.choice([-1.0, 1.0], M)
+    C64, A64, B64 = C.astype(np.float64), A.astype(np.float64), B.astype(np.float64)
+    b0 = np.zeros((M, N)) if base is None else base.astype(np.float64)
+    # rounding of C: independent errors of relative size eps per element -> eps * ||row|| on a row checksum
+    eps = 2.0 ** -8 if rtol >= 1e-2 else 1e-5
+    right = A64 @ (B64 @ r) + b0 @ r
+    bound = 8 * eps * np.linalg.norm(C64, axis=1) + 1e-6
+    bad = np.abs(C64 @ r - right) > bound
+    assert not bad.any(), f"{name}: row checksum off in rows {np.nonzero(bad)[0][:8]}"
+    left = (sgn @ A64) @ B64 + sgn @ b0
+    bound = 8 * eps * np.linalg.norm(C64, axis=0) + 1e-6
+    bad = np.abs(sgn @ C64 - left) > bound
+    assert not bad.any(), f"{name}: column checksum off in columns {np.nonzero(bad)[0][:8]}"
+    rows = np.array([lo + rng.integers(min(rows_per_block, M - lo)) for lo in range(0, M, rows_per_block)])
+    assert_close(C64[rows], A64[rows] @ B64 + b0[rows], rtol, f"{name}: sampled rows")
+
+
+def test_gemm_config5_full_size_properties(ctx):
+    """The products of one config-5 transformer block at their real shapes (4096 tokens, d 2048, KV width 512, ffn 5632),
+    each through the entry point and tile the training step uses: checksums and sampled rows instead of a full host product."""
+    T, d, dkv, f = 4096, 2048, 512, 5632
+    x, wq, w2 = _rand_bf16(700, (T, d)), _rand_bf16(701, (d, d), 0.05), _rand_bf16(702, (f, d), 0.05)
+    wg, wu = _rand_bf16(703, (d, f), 0.05), _rand_bf16(704, (d, f), 0.05)
+    dx, dwq, dw2, dwg, dwu = (up(ctx, a, BF16) for a in (x, wq, w2, wg, wu))
+    # forward projection (NN, 256 tiles of 256x128x64) and its input gradient form (NT)
+    c = ctx.malloc(T * d * 2)
+    ctx.gemm(dx, dwq, c, BF16, BF16, 0, 0, T, d, d)
+    _check_product("q projection", dn(ctx, c, (T, d), BF16), x, wq, 2e-2)
+    ctx.gemm(dx, dwq, c, BF16, BF16, 0, 1, T, d, d)
+    _check_product("dX of a projection", dn(ctx, c, (T, d), BF16), x, wq.T, 2e-2)
+    # gate, up and h = silu(gate) * up in one kernel (704 tiles)
+    g_, u_, h_ = (ctx.malloc(T * f * 2) for _ in range(3))
+    ctx.gemm_swiglu_forward(dx, dwg, dwu, g_, u_, h_, BF16, T, f, d)
+    G, U, H = (dn(ctx, t, (T, f), BF16) for t in (g_, u_, h_))
+    _check_product("gate", G, x, wg, 2e-2)
+    _check_product("up", U, x, wu, 2e-2)
+    g64 = G.astype(np.float64)
+    assert_close(H, g64 / (1.0 + np.exp(-g64)) * U.astype(np.float64), 1e-2, "h")
+    # down projection + residual (K = 5632)
+    res = _rand_bf16(705, (T, d))
+    dres, o = up(ctx, res, BF16), ctx.malloc(T * d * 2)
+    ctx.gemm_residual(h_, dw2, dres, o, BF16, BF16, 0, 0, T, d, f)
+    _check_product("down projection + residual", dn(ctx, o, (T, d), BF16), H, w2, 2e-2, base=res)
+    # its input gradient with the SwiGLU backward in the epilogue: dgate, dup against dH = dOut W2^T through the
+    # exactly recomputed rows (dgate and dup are not linear in the operands, so no checksum)
+    dout = _rand_bf16(706, (T, d))
+    ddout, dgate, dup_ = up(ctx, dout, BF16), ctx.malloc(T * f * 2), ctx.malloc(T * f * 2)
+    ctx.gemm_swiglu_backward(ddout, dw2, g_, u_, dgate, dup_, BF16, 0, 1, T, f, d)
+    rows = np.arange(0, T, 64) + np.random.default_rng(5).integers(0, 64, T // 64)
+    dh = dout[rows].astype(np.float64) @ w2.astype(np.float64).T
+    gs, us = G[rows].astype(np.float64), U[rows].astype(np.float64)
+    sig = 1.0 / (1.0 + np.exp(-gs))
+    silu = gs * sig
+    assert_close(dn(ctx, dgate, (T, f), BF16)[rows], dh * us * (silu + sig * (1.0 - silu)), 2e-2, "dgate rows")
+    assert_close(dn(ctx, dup_, (T, f), BF16)[rows], dh * silu, 2e-2, "dup rows")
+    # weight gradients, f32 +=: the down projection's (352 tiles of 256x128x32) and the six-product grouped launch
+    c0 = np.random.default_rng(707).standard_normal((f, d), dtype=np.float32)
+    dc = up(ctx, c0, F32)
+    ctx.gemm(h_, ddout, dc, BF16, F32, 1, 0, f, d, T, 1)
+    _check_product("down projection dW", dn(ctx, dc, (f, d), F32), H.T, dout, 1e-3, base=c0)
+    dys = [_rand_bf16(710 + i, (T, n)) for i, n in enumerate((d, dkv, dkv, d, f, f))]
+    xs = [x, x, x, _rand_bf16(720, (T, d)), res, res]
+    dxs = {id(a): up(ctx, a, BF16) for a in (x, xs[3], res)}
+    ddys = [up(ctx, a, BF16) for a in dys]
+    c0s = [np.random.default_rng(730 + i).standard_normal((d, a.shape[1]), dtype=np.float32) for i, a in enumerate(dys)]
+    dcs = [up(ctx, a, F32) for a in c0s]
+    ctx.gemm_grouped([dxs[id(a)] for a in xs], ddys, dcs, [a.shape[1] for a in dys], BF16, F32, 1, 0, d, T, 1)
+    for i in range(6):
+        _check_product(f"grouped dW {i}", dn(ctx, dcs[i], c0s[i].shape, F32), xs[i].T, dys[i], 1e-3, base=c0s[i])
+    for t in [dx, dwq, dw2, dwg, dwu, c, g_, u_, h_, dres, o, ddout, dgate, dup_, dc] + list(dxs.values()) + ddys + dcs:
+        t.free()
+
+
 def test_gemm_f32_matches_oracle_order_tolerance(ctx):
     # config-1 sized linear against the sequential-order f32 oracle, rtol 1e-4
     a, b, go = gen.normal(410, (64, 64)), gen.normal(411, (64, 256), 0.02), gen.normal(412, (64, 256))
