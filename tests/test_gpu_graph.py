@@ -254,6 +254,36 @@ def test_deferred_weight_gradients_bf16_mixed_step(ctx):
     _train_steps(ctx, cfg, G.BF16_MIXED, 2, 128, steps=1, accum=2, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
 
 
+def test_config5_layer_fused_path_matches_the_reference_chain(ctx):
+    """One layer at config 5's real width and tokens per micro-batch (d 2048, 32 q / 8 kv heads, ffn 5632, 4096 tokens as
+    32 x 128: every GEMM has its config-5 shape, while the chain's materialised [B*H, S, S] scores stay small): the fused
+    path (grouped and deferred weight gradients, SwiGLU inside the GEMMs, side stream, rotary embedding inside attention)
+    against the reference's op-by-op chain built from the individually oracle-checked kernels, same weights, two
+    accumulated micro-batches.  The oracle itself would need minutes at this size."""
+    from eisen_amd import hip
+    cfg = dict(vocab=1024, hidden=2048, heads=32, kv_heads=8, ffn=5632, layers=1, tie=False)
+    weights = [(n, hip.round_bf16(w) if w.ndim == 2 else w) for n, w in gen.lm_weights(3, std=0.02, perturb_norm=0.05, **cfg)]
+    grads, losses = [], []
+    for fused in (True, False):
+        gg = G.Graph(ctx, G.BF16_MIXED)
+        lm = G.TransformerLM(gg, **cfg)
+        for pid, (_, w) in enumerate(weights):
+            gg.load_tensor_data(pid, w)
+        gg.mark_params()
+        lm.set_fused(fused)
+        ls = []
+        for micro in range(2):
+            x, y = gen.lm_batch(3000 + micro, 32, 128, cfg["vocab"], "zipf")
+            ls.append(lm.micro_step(x, y))
+        losses.append(ls)
+        grads.append([gg.sync_grad_to_cpu(pid) for pid in range(len(weights))])
+        gg.close()
+    for a, b in zip(*losses):
+        assert abs(a - b) <= 2e-3 * abs(b), losses
+    for pid, (name, _) in enumerate(weights):
+        assert_close(grads[0][pid], grads[1][pid], 2e-2, f"grad {name}", row_scale=(name == "embed"), step=True)
+
+
 def test_grad_accumulation_invariants_on_gpu(ctx):
     # tests/test_grad_accum.rs: additivity (:59-98), g_accum = N g_full (:108-166), clear_activations keeps
     # parameter gradients, zero_grad, tape emptied, tensor count back at the watermark
