@@ -622,7 +622,11 @@ struct SwigluForwardArgs {
     bf16_t* U;
     bf16_t* H;
     int M, N, K;
+    int tile_group;    // PLAIN: N tiles per group of the tile order (see gemm_mfma_direct_kernel), 0 = row-major
 };
+// PLAIN: no SwiGLU; the same main loop as one 256 x 256 tile of C = X W (Wg = W, Wu = W + 128 columns, G = C, U = C + 128
+// columns, N = row length of W and C; blockIdx.x enumerates the (M / 256) * (N / 256) tiles).
+template <bool PLAIN>
 __global__ __launch_bounds__(512) void gemm_swiglu_forward_kernel(SwigluForwardArgs g) {
     constexpr int BM = 256, BN = 128, BK = 32, WGN = 2, WAVES = 8, STAGES = 3;
     constexpr int WM = 64, WN = 64, TM = 2, TN = 2, KSTEPS = BK / 16;
@@ -634,7 +638,19 @@ __global__ __launch_bounds__(512) void gemm_swiglu_forward_kernel(SwigluForwardA
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    int mt = blockIdx.y, nt = blockIdx.x;
+    if (PLAIN) {
+        const int n_tiles = g.N / (2 * BN), m_tiles = g.M / BM, lin = blockIdx.x;
+        mt = lin / n_tiles;
+        nt = lin % n_tiles;
+        if (g.tile_group > 0) {
+            const int per_group = g.tile_group * m_tiles, grp = lin / per_group, within = lin % per_group;
+            const int width = min(g.tile_group, n_tiles - grp * g.tile_group);
+            mt = within / width;
+            nt = grp * g.tile_group + within % width;
+        }
+    }
+    const int m0 = mt * BM, n0 = nt * (PLAIN ? 2 * BN : BN);
 
     f32x16 accg[TM][TN], accu[TM][TN];
 #pragma unroll
@@ -750,12 +766,14 @@ __global__ __launch_bounds__(512) void gemm_swiglu_forward_kernel(SwigluForwardA
                 // the outputs the backward pass reads are the rounded ones, so H is formed from them as the separate kernel would
                 og[e] = (bf16_t)vg[ps][e];
                 ou[e] = (bf16_t)vu[ps][e];
-                const float gv = (float)og[e], uv = (float)ou[e];
-                oh[e] = (bf16_t)(gv * (1.0f / (1.0f + __expf(-gv))) * uv);
+                if (!PLAIN) {
+                    const float gv = (float)og[e], uv = (float)ou[e];
+                    oh[e] = (bf16_t)(gv * (1.0f / (1.0f + __expf(-gv))) * uv);
+                }
             }
             *reinterpret_cast<bf16x8*>(g.G + at) = og;
             *reinterpret_cast<bf16x8*>(g.U + at) = ou;
-            *reinterpret_cast<bf16x8*>(g.H + at) = oh;
+            if (!PLAIN) *reinterpret_cast<bf16x8*>(g.H + at) = oh;
         }
     }
 }
@@ -1007,6 +1025,19 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
                       (double)wide_tiles / (double)(256 * ((wide_tiles + 255) / 256)) >= 0.85;
     const bool wide32 = mfma_ok && split == 1 && n_more == 0 && !a_kc && !b_kc && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 &&
                         (wide_tiles >= 512 || (wide_tiles >= 300 && !wide));
+    // 256 x 256 tiles (the gate/up kernel's main loop: an A operand register feeds twice the MFMAs) where the grid still
+    // has three rounds of them: the lm_head forward (1035 against 980 TFLOP/s at 4096 x 32000 x 2048)
+    const bool wide256 = mfma_ok && split == 1 && n_more == 0 && a_kc && !b_kc && batch == 1 && dtype_c == EISEN_BF16 && !residual && !swiglu &&
+                         !accumulate && M % 256 == 0 && N % 256 == 0 && K % 32 == 0 && (M / 256) * (N / 256) >= 768 && eisen_aligned(C, 16);
+    if (wide256) {
+        SwigluForwardArgs a{static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(B), static_cast<const bf16_t*>(B) + 128, static_cast<bf16_t*>(C),
+                            static_cast<bf16_t*>(C) + 128,  nullptr,                        (int)M,                             (int)N, (int)K,
+                            N / 256 >= 32 ? 16 : 0};
+        EisenProfScope prof(ctx, "gemm_nn_bf16_bf16out_256x256x32", 2.0 * (double)M * (double)N * (double)K, true);
+        gemm_swiglu_forward_kernel<true><<<dim3((unsigned)((M / 256) * (N / 256)), 1, 1), 512, 0, ctx->stream>>>(a);
+        EISEN_LAUNCH_CHECK(ctx, who);
+        return 0;
+    }
     const char* tile = !mfma_ok ? "fma64x64" : wide32 ? "256x128x32" : wide ? "256x128x64" : (big_tile || split128) ? (K % 64 == 0 && !(!a_kc && !b_kc && M % 128 == 0 && N % 128 == 0 && tiles128 * split >= 512) ? "128x128x64" : "128x128x32") : "64x64x32";
     snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
              dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : swiglu ? "_swiglu_bwd" : "");
@@ -1118,9 +1149,9 @@ extern "C" int eisen_hip_gemm_swiglu_forward(eisen_ctx* ctx, const void* X, cons
                        eisen_aligned(Wu, 16) && eisen_aligned(G, 16) && eisen_aligned(U, 16) && eisen_aligned(H, 16);
     if (fused) {
         SwigluForwardArgs a{static_cast<const bf16_t*>(X), static_cast<const bf16_t*>(Wg), static_cast<const bf16_t*>(Wu), static_cast<bf16_t*>(G),
-                            static_cast<bf16_t*>(U),       static_cast<bf16_t*>(H),        (int)M,                          (int)N, (int)K};
+                            static_cast<bf16_t*>(U),       static_cast<bf16_t*>(H),        (int)M,                          (int)N, (int)K, 0};
         EisenProfScope prof(ctx, "gemm_nn_bf16_swiglu_256x128x32", 4.0 * (double)M * (double)N * (double)K, true);
-        gemm_swiglu_forward_kernel<<<dim3((unsigned)(N / 128), (unsigned)(M / 256), 1), 512, 0, ctx->stream>>>(a);
+        gemm_swiglu_forward_kernel<false><<<dim3((unsigned)(N / 128), (unsigned)(M / 256), 1), 512, 0, ctx->stream>>>(a);
         EISEN_LAUNCH_CHECK(ctx, "eisen_hip_gemm_swiglu_forward");
         return 0;
     }

@@ -836,6 +836,17 @@ def test_gemm_config5_full_size_properties(ctx):
         t.free()
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 32000, 96), (4096, 12288, 32), (12288, 4096, 160)])
+def test_gemm_forward_256x256_tiles(ctx, M, N, K):
+    # forward products with at least three rounds of 256 x 256 tiles (the lm_head: 125 tile columns, walked in groups of 16)
+    a, b = _rand_bf16(740, (M, K)), _rand_bf16(741, (K, N), 0.1)
+    da, db, dc = up(ctx, a, BF16), up(ctx, b, BF16), ctx.malloc(M * N * 2)
+    ctx.gemm(da, db, dc, BF16, BF16, 0, 0, M, N, K)
+    _check_product("256x256 tiles", dn(ctx, dc, (M, N), BF16), a, b, 2e-2)
+    for t in (da, db, dc):
+        t.free()
+
+
 def test_gemm_f32_matches_oracle_order_tolerance(ctx):
     # config-1 sized linear against the sequential-order f32 oracle, rtol 1e-4
     a, b, go = gen.normal(410, (64, 64)), gen.normal(411, (64, 256), 0.02), gen.normal(412, (64, 256))
