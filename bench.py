@@ -36,10 +36,10 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # (fetch x 1.997, write x 1.000 after calibration on the library's copy kernel), per workload and per profile
 # name the library reports.  The config-5 GEMM figures are averages over that entry's launches in the step.
 MEASURED_TRAFFIC = {
-    "c5": {"gemm_nn_bf16_bf16out_256x128x64": 253.7e6, "gemm_nt_bf16_bf16out_256x128x64": 438.2e6,
+    "c5": {"gemm_nn_bf16_bf16out_256x128x64": 253.7e6, "gemm_nt_bf16_bf16out_256x128x64": 437.4e6,
            "gemm_nt_bf16_bf16out_256x128x64_swiglu_bwd": 473.7e6, "gemm_nn_bf16_swiglu_256x128x32": 565.8e6,
-           "gemm_tn_bf16_f32out_256x128x32": 576.1e6, "gemm_tn_bf16_f32out_256x128x32_grouped": 1254.0e6,
-           "gemm_nn_bf16_bf16out_128x128x64": 84.1e6, "gemm_nn_bf16_bf16out_256x256x32": None, "ce_fused_bf16": 524.6e6},
+           "gemm_tn_bf16_f32out_256x128x32": 576.6e6, "gemm_tn_bf16_f32out_256x128x32_grouped": 1252.8e6,
+           "gemm_nn_bf16_bf16out_128x128x64": 84.1e6, "gemm_nn_bf16_bf16out_256x256x32": 1561.1e6, "ce_fused_bf16": 524.6e6},
     "c4": {},
     "c3": {"attn_bwd": 78.0e6 + 51.7e6},
     "c2": {"ce_fused_bf16": 1048.9e6},
