@@ -178,9 +178,13 @@ struct BcastBwdArgs {
     size_t dst_numel;
 };
 
+// chunks == 1: as described.  chunks > 1 (few dst elements, long reductions: the gradient of a broadcast scalar): the walk
+// of one dst element is cut into `chunks` consecutive ranges, one thread each, whose sums go to partial[e * chunks + c];
+// bcast_bwd_finish_kernel adds them in ascending order.  Deterministic either way; the chunked form associates the sum
+// differently from the single walk.
 template <typename T>
 __global__ __launch_bounds__(kEwThreads) void bcast_bwd_kernel(T* dst, const T* go, const T* other, BcastBwdArgs g,
-                                                                int accumulate) {
+                                                                int accumulate, size_t chunks, float* partial) {
     size_t fixed_shape[4], red_shape[4];
     size_t out_strides[4];
     size_t cur = 1;
@@ -195,7 +199,10 @@ __global__ __launch_bounds__(kEwThreads) void bcast_bwd_kernel(T* dst, const T* 
         red_shape[d] = is_red ? g.shape[d] : 1;
         nred *= red_shape[d];
     }
-    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < g.dst_numel; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t per_chunk = (nred + chunks - 1) / chunks;
+    for (size_t w = (size_t)blockIdx.x * blockDim.x + threadIdx.x; w < g.dst_numel * chunks; w += (size_t)gridDim.x * blockDim.x) {
+        const size_t e = w / chunks, chunk = w % chunks;
+        const size_t t_lo = chunk * per_chunk, t_hi = t_lo + per_chunk < nred ? t_lo + per_chunk : nred;
         // decode e over the non-reduced dims (dst is contiguous over them in order)
         size_t rem = e, base_out = 0, base_other = 0, dst_idx = 0;
         for (int d = g.rank - 1; d >= 0; d--) {
@@ -205,8 +212,8 @@ __global__ __launch_bounds__(kEwThreads) void bcast_bwd_kernel(T* dst, const T* 
             base_other += c * g.so[d];
             dst_idx += c * g.sd[d];
         }
-        float acc = accumulate ? to_f32(dst[dst_idx]) : 0.f;
-        for (size_t t = 0; t < nred; t++) {
+        float acc = accumulate && chunks == 1 ? to_f32(dst[dst_idx]) : 0.f;
+        for (size_t t = t_lo; t < t_hi; t++) {
             size_t r = t, io = base_out, ioth = base_other;
             for (int d = g.rank - 1; d >= 0; d--) {
                 const size_t c = r % red_shape[d];
@@ -217,6 +224,23 @@ __global__ __launch_bounds__(kEwThreads) void bcast_bwd_kernel(T* dst, const T* 
             const float gv = to_f32(go[io]);
             acc += other ? to_f32(other[ioth]) * gv : gv;
         }
+        if (chunks == 1) dst[dst_idx] = from_f32<T>(acc);
+        else partial[w] = acc;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kEwThreads) void bcast_bwd_finish_kernel(T* dst, const float* partial, BcastBwdArgs g, int accumulate, size_t chunks) {
+    size_t fixed_shape[4];
+    for (int d = 0; d < g.rank; d++) fixed_shape[d] = g.sd[d] == 0 && g.shape[d] > 1 ? 1 : g.shape[d];
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < g.dst_numel; e += (size_t)gridDim.x * blockDim.x) {
+        size_t rem = e, dst_idx = 0;
+        for (int d = g.rank - 1; d >= 0; d--) {
+            dst_idx += (rem % fixed_shape[d]) * g.sd[d];
+            rem /= fixed_shape[d];
+        }
+        float acc = accumulate ? to_f32(dst[dst_idx]) : 0.f;
+        for (size_t c = 0; c < chunks; c++) acc += partial[e * chunks + c];
         dst[dst_idx] = from_f32<T>(acc);
     }
 }
@@ -366,11 +390,31 @@ extern "C" int eisen_hip_bcast_backward(eisen_ctx* ctx, void* dst, const void* g
     }
     EISEN_REQUIRE(ctx, fixed == dst_numel, EISEN_E_SHAPE, "bcast_backward: dst_numel %zu does not match the non-broadcast dims (%zu)", dst_numel, fixed);
     if (dst_numel == 0) return 0;
-    const unsigned blocks = (unsigned)std::min<size_t>(4096, eisen_ceil_div(dst_numel, kEwThreads));
-    if (dtype == EISEN_F32)
-        bcast_bwd_kernel<float><<<blocks, kEwThreads, 0, ctx->stream>>>((float*)dst, (const float*)grad_out, (const float*)other, g, accumulate);
-    else
-        bcast_bwd_kernel<bf16_t><<<blocks, kEwThreads, 0, ctx->stream>>>((bf16_t*)dst, (const bf16_t*)grad_out, (const bf16_t*)other, g, accumulate);
+    // one thread per dst element walks its whole reduction; when that leaves most of the chip idle (a handful of dst
+    // elements, millions of terms each) the walk is cut into chunks of at least 1024 terms
+    size_t total = 1;
+    for (int d = 0; d < rank; d++) total *= out_shape[d];
+    const size_t nred = total / dst_numel;
+    size_t chunks = 1;
+    if (dst_numel < 16384 && nred >= 8192) chunks = std::min<size_t>(nred / 1024, std::max<size_t>(1, 65536 / dst_numel));
+    float* partial = nullptr;
+    if (chunks > 1) {
+        void* ws = nullptr;
+        const int rc = eisen_workspace(ctx, dst_numel * chunks * sizeof(float), &ws);
+        if (rc) return rc;
+        partial = static_cast<float*>(ws);
+    } else {
+        chunks = 1;
+    }
+    const unsigned blocks = (unsigned)std::min<size_t>(4096, eisen_ceil_div(dst_numel * chunks, kEwThreads));
+    const unsigned fin_blocks = (unsigned)std::min<size_t>(4096, eisen_ceil_div(dst_numel, kEwThreads));
+    if (dtype == EISEN_F32) {
+        bcast_bwd_kernel<float><<<blocks, kEwThreads, 0, ctx->stream>>>((float*)dst, (const float*)grad_out, (const float*)other, g, accumulate, chunks, partial);
+        if (chunks > 1) bcast_bwd_finish_kernel<float><<<fin_blocks, kEwThreads, 0, ctx->stream>>>((float*)dst, partial, g, accumulate, chunks);
+    } else {
+        bcast_bwd_kernel<bf16_t><<<blocks, kEwThreads, 0, ctx->stream>>>((bf16_t*)dst, (const bf16_t*)grad_out, (const bf16_t*)other, g, accumulate, chunks, partial);
+        if (chunks > 1) bcast_bwd_finish_kernel<bf16_t><<<fin_blocks, kEwThreads, 0, ctx->stream>>>((bf16_t*)dst, partial, g, accumulate, chunks);
+    }
     EISEN_LAUNCH_CHECK(ctx, "bcast_bwd_kernel");
     return 0;
 }

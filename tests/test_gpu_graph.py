@@ -255,8 +255,7 @@ def test_deferred_weight_gradients_bf16_mixed_step(ctx):
 
 
 def test_config5_layer_fused_path_matches_the_reference_chain(ctx):
-    """One layer at config 5's real width and tokens per micro-batch (d 2048, 32 q / 8 kv heads, ffn 5632, 4096 tokens as
-    32 x 128: every GEMM has its config-5 shape, while the chain's materialised [B*H, S, S] scores stay small): the fused
+    """One layer at config 5's real width and micro-batch (d 2048, 32 q / 8 kv heads, ffn 5632, 4 x 1024 tokens): the fused
     path (grouped and deferred weight gradients, SwiGLU inside the GEMMs, side stream, rotary embedding inside attention)
     against the reference's op-by-op chain built from the individually oracle-checked kernels, same weights, two
     accumulated micro-batches.  The oracle itself would need minutes at this size."""
@@ -273,7 +272,7 @@ def test_config5_layer_fused_path_matches_the_reference_chain(ctx):
         lm.set_fused(fused)
         ls = []
         for micro in range(2):
-            x, y = gen.lm_batch(3000 + micro, 32, 128, cfg["vocab"], "zipf")
+            x, y = gen.lm_batch(3000 + micro, 4, 1024, cfg["vocab"], "zipf")
             ls.append(lm.micro_step(x, y))
         losses.append(ls)
         grads.append([gg.sync_grad_to_cpu(pid) for pid in range(len(weights))])

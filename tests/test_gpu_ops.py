@@ -167,6 +167,26 @@ def test_broadcast_add_mul_and_backward(ctx):
     assert_close(dn(ctx, gm, m.shape, F32), go.sum(0, keepdims=True), 1e-5, "add bcast bwd")
 
 
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_broadcast_backward_long_reductions(ctx, accumulate):
+    # few dst elements, many terms each (the gradient of a broadcast scalar or row): the walk is cut into chunks summed in order
+    shape = (64, 128, 128)
+    go, other = gen.normal(20, shape), gen.normal(21, shape)
+    dgo, doth = up(ctx, go, F32), up(ctx, other, F32)
+    for dst_shape, strides, axes in (((1,), (0, 0, 0), (0, 1, 2)), ((128,), (0, 0, 1), (0, 1))):
+        d0 = gen.normal(22, dst_shape)
+        for oth, exp in ((doth, (go.astype(np.float64) * other).sum(axes)), (None, go.astype(np.float64).sum(axes))):
+            dst = up(ctx, d0, F32)
+            ctx.bcast_backward(dst, dgo, oth, F32, shape, strides, (128 * 128, 128, 1) if oth else None, d0.size, accumulate)
+            got = dn(ctx, dst, dst_shape, F32)
+            assert_close(got, exp.reshape(dst_shape) + (d0 if accumulate else 0), 1e-4, f"dst {dst_shape} other={oth is not None}")
+            dst2 = up(ctx, d0, F32)
+            ctx.bcast_backward(dst2, dgo, oth, F32, shape, strides, (128 * 128, 128, 1) if oth else None, d0.size, accumulate)
+            assert np.array_equal(dn(ctx, dst2, dst_shape, F32), got)       # same bits on a second run
+            dst.free(); dst2.free()
+    dgo.free(); doth.free()
+
+
 # ---------------------------------------------------------------------------
 # rmsnorm, rope, softmax, layout
 # ---------------------------------------------------------------------------
