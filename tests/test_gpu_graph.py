@@ -254,13 +254,13 @@ def test_deferred_weight_gradients_bf16_mixed_step(ctx):
     _train_steps(ctx, cfg, G.BF16_MIXED, 2, 128, steps=1, accum=2, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
 
 
-def test_config5_layer_fused_path_matches_the_reference_chain(ctx):
-    """One layer at config 5's real width and micro-batch (d 2048, 32 q / 8 kv heads, ffn 5632, 4 x 1024 tokens): the fused
+def test_config5_layers_fused_path_matches_the_reference_chain(ctx):
+    """Two layers at config 5's real width and micro-batch (d 2048, 32 q / 8 kv heads, ffn 5632, 4 x 1024 tokens): the fused
     path (grouped and deferred weight gradients, SwiGLU inside the GEMMs, side stream, rotary embedding inside attention)
     against the reference's op-by-op chain built from the individually oracle-checked kernels, same weights, two
     accumulated micro-batches.  The oracle itself would need minutes at this size."""
     from eisen_amd import hip
-    cfg = dict(vocab=1024, hidden=2048, heads=32, kv_heads=8, ffn=5632, layers=1, tie=False)
+    cfg = dict(vocab=1024, hidden=2048, heads=32, kv_heads=8, ffn=5632, layers=2, tie=False)
     weights = [(n, hip.round_bf16(w) if w.ndim == 2 else w) for n, w in gen.lm_weights(3, std=0.02, perturb_norm=0.05, **cfg)]
     grads, losses = [], []
     for fused in (True, True, False):  # the fused path twice: the same bits both times (no atomics, ordered streams)
