@@ -27,7 +27,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-from tests import gen  # noqa: E402  (seeded synthetic inputs shared with the tests)
+from eisen_amd import synth as gen  # noqa: E402  (seeded synthetic inputs, the same the tests use)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E

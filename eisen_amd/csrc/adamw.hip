@@ -206,7 +206,10 @@ int upload_slots(eisen_ctx* ctx, const eisen_param_slot* slots, size_t n_slots, 
     int rc = eisen_hip_malloc(ctx, n_slots * sizeof(SlotDev), &dev);
     if (rc) return rc;
     rc = eisen_hip_htod(ctx, dev, host.data(), n_slots * sizeof(SlotDev));
-    if (rc) return rc;
+    if (rc) {
+        (void)eisen_hip_free(ctx, dev);
+        return rc;
+    }
     *dev_out = (SlotDev*)dev;
     *blocks_out = blocks;
     return 0;
@@ -249,7 +252,10 @@ extern "C" int eisen_hip_grad_norm(eisen_ctx* ctx, const eisen_param_slot* slots
     if (rc) return rc;
     void* ws = nullptr;
     rc = eisen_workspace(ctx, blocks * sizeof(double), &ws);
-    if (rc) return rc;
+    if (rc) {
+        (void)eisen_hip_free(ctx, dev);
+        return rc;
+    }
     sumsq_kernel<<<(unsigned)blocks, kThreads, 0, ctx->stream>>>(dev, (int)n_slots, (double*)ws);
     EISEN_LAUNCH_CHECK(ctx, "sumsq_kernel");
     norm_finish_kernel<<<1, 1024, 0, ctx->stream>>>((const double*)ws, blocks, max_norm, out_device);

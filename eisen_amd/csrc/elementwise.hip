@@ -182,8 +182,8 @@ struct BcastBwdArgs {
 // of one dst element is cut into `chunks` consecutive ranges, one thread each, whose sums go to partial[e * chunks + c];
 // bcast_bwd_finish_kernel adds them in ascending order.  Deterministic either way; the chunked form associates the sum
 // differently from the single walk.
-template <typename T>
-__global__ __launch_bounds__(kEwThreads) void bcast_bwd_kernel(T* dst, const T* go, const T* other, BcastBwdArgs g,
+template <typename T, typename TD>
+__global__ __launch_bounds__(kEwThreads) void bcast_bwd_kernel(TD* dst, const T* go, const T* other, BcastBwdArgs g,
                                                                 int accumulate, size_t chunks, float* partial) {
     size_t fixed_shape[4], red_shape[4];
     size_t out_strides[4];
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(kEwThreads) void bcast_bwd_kernel(T* dst, const T* 
             const float gv = to_f32(go[io]);
             acc += other ? to_f32(other[ioth]) * gv : gv;
         }
-        if (chunks == 1) dst[dst_idx] = from_f32<T>(acc);
+        if (chunks == 1) dst[dst_idx] = from_f32<TD>(acc);
         else partial[w] = acc;
     }
 }
@@ -370,9 +370,9 @@ extern "C" int eisen_hip_mul_bcast(eisen_ctx* ctx, const void* a, const void* b,
     return bcast_common(ctx, a, b, out, dtype, rank, out_shape, a_strides, b_strides, true);
 }
 
-extern "C" int eisen_hip_bcast_backward(eisen_ctx* ctx, void* dst, const void* grad_out, const void* other, int dtype,
-                                        int rank, const size_t* out_shape, const size_t* dst_strides,
-                                        const size_t* other_strides, size_t dst_numel, int accumulate) {
+static int bcast_backward_common(eisen_ctx* ctx, void* dst, const void* grad_out, const void* other, int dtype, bool dst_f32,
+                                 int rank, const size_t* out_shape, const size_t* dst_strides,
+                                 const size_t* other_strides, size_t dst_numel, int accumulate) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, dst && grad_out && out_shape && dst_strides, EISEN_E_ARG, "bcast_backward: null pointer");
     EISEN_REQUIRE(ctx, rank >= 1 && rank <= 4, EISEN_E_SHAPE, "bcast_backward: rank %d not in 1..4", rank);
@@ -409,14 +409,29 @@ extern "C" int eisen_hip_bcast_backward(eisen_ctx* ctx, void* dst, const void* g
     const unsigned blocks = (unsigned)std::min<size_t>(4096, eisen_ceil_div(dst_numel * chunks, kEwThreads));
     const unsigned fin_blocks = (unsigned)std::min<size_t>(4096, eisen_ceil_div(dst_numel, kEwThreads));
     if (dtype == EISEN_F32) {
-        bcast_bwd_kernel<float><<<blocks, kEwThreads, 0, ctx->stream>>>((float*)dst, (const float*)grad_out, (const float*)other, g, accumulate, chunks, partial);
+        bcast_bwd_kernel<float, float><<<blocks, kEwThreads, 0, ctx->stream>>>((float*)dst, (const float*)grad_out, (const float*)other, g, accumulate, chunks, partial);
+        if (chunks > 1) bcast_bwd_finish_kernel<float><<<fin_blocks, kEwThreads, 0, ctx->stream>>>((float*)dst, partial, g, accumulate, chunks);
+    } else if (dst_f32) {
+        bcast_bwd_kernel<bf16_t, float><<<blocks, kEwThreads, 0, ctx->stream>>>((float*)dst, (const bf16_t*)grad_out, (const bf16_t*)other, g, accumulate, chunks, partial);
         if (chunks > 1) bcast_bwd_finish_kernel<float><<<fin_blocks, kEwThreads, 0, ctx->stream>>>((float*)dst, partial, g, accumulate, chunks);
     } else {
-        bcast_bwd_kernel<bf16_t><<<blocks, kEwThreads, 0, ctx->stream>>>((bf16_t*)dst, (const bf16_t*)grad_out, (const bf16_t*)other, g, accumulate, chunks, partial);
+        bcast_bwd_kernel<bf16_t, bf16_t><<<blocks, kEwThreads, 0, ctx->stream>>>((bf16_t*)dst, (const bf16_t*)grad_out, (const bf16_t*)other, g, accumulate, chunks, partial);
         if (chunks > 1) bcast_bwd_finish_kernel<bf16_t><<<fin_blocks, kEwThreads, 0, ctx->stream>>>((bf16_t*)dst, partial, g, accumulate, chunks);
     }
     EISEN_LAUNCH_CHECK(ctx, "bcast_bwd_kernel");
     return 0;
+}
+
+extern "C" int eisen_hip_bcast_backward(eisen_ctx* ctx, void* dst, const void* grad_out, const void* other, int dtype,
+                                        int rank, const size_t* out_shape, const size_t* dst_strides,
+                                        const size_t* other_strides, size_t dst_numel, int accumulate) {
+    return bcast_backward_common(ctx, dst, grad_out, other, dtype, false, rank, out_shape, dst_strides, other_strides, dst_numel, accumulate);
+}
+
+extern "C" int eisen_hip_bcast_backward_f32(eisen_ctx* ctx, float* dst, const void* grad_out, const void* other, int dtype,
+                                            int rank, const size_t* out_shape, const size_t* dst_strides,
+                                            const size_t* other_strides, size_t dst_numel, int accumulate) {
+    return bcast_backward_common(ctx, dst, grad_out, other, dtype, true, rank, out_shape, dst_strides, other_strides, dst_numel, accumulate);
 }
 
 extern "C" int eisen_hip_mul_backward(eisen_ctx* ctx, const void* x, const void* y, const void* go, void* ga, void* gb,

@@ -145,7 +145,10 @@ extern "C" int eisen_hip_gather_backward(eisen_ctx* ctx, const int32_t* ids_host
     int rc = eisen_hip_malloc(ctx, total * sizeof(int32_t), &dev);
     if (rc) return rc;
     rc = eisen_hip_htod(ctx, dev, blob.data(), total * sizeof(int32_t));
-    if (rc) return rc;
+    if (rc) {
+        (void)eisen_hip_free(ctx, dev);
+        return rc;
+    }
     const int32_t* d_order = (const int32_t*)dev;
     const int32_t* d_row = d_order + n_ids;
     const int32_t* d_begin = d_row + n_seg;

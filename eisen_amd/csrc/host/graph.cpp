@@ -328,8 +328,18 @@ size_t Graph::elementwise_binary(size_t a, size_t b, bool is_mul) {
                             const std::vector<size_t>& other_st) {
             int acc = 0;
             Storage& gs = g.grad_for_write(self, &acc);
-            if (gs.dtype != go.dtype) throw Error("add/mul backward: gradient element types differ (parameter operand in mixed precision)");
             const Storage od = g.compute_data(other);
+            if (gs.dtype != go.dtype) {
+                // a parameter operand in mixed precision (a Linear bias): bf16 dOut, f32 parameter gradient
+                if (gs.dtype != EISEN_F32) throw Error("add/mul backward: gradient element types differ");
+                const std::vector<size_t> osv = os.empty() ? std::vector<size_t>{1} : os;
+                std::vector<size_t> st_self = self_st, st_other = other_st;
+                if (os.empty()) { st_self = {1}; st_other = {0}; }
+                g.check(eisen_hip_bcast_backward_f32(g.ctx(), (float*)gs.ptr, go.ptr, is_mul ? od.ptr : nullptr, dtype, (int)osv.size(), osv.data(), st_self.data(),
+                                                     is_mul ? st_other.data() : nullptr, numel_of(self_shape), acc),
+                        "add/mul backward (f32 parameter gradient)");
+                return;
+            }
             if (self_shape == os) {
                 if (is_mul) {
                     // ga (+)= other * go, expressed through mul_backward with the other side disabled

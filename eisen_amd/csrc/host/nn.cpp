@@ -104,46 +104,51 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
         v = v_proj.forward(g, x_id);
     }
     const float scale = 1.0f / std::sqrt((float)head_dim);
-    if (fused) {
+    // the bf16 MFMA attention kernels exist for head_dim 32, 64 and 128; other head dims in mixed precision take the
+    // reference's materialised chain below (any head_dim), like every f32 graph may
+    const bool kernel_head_dim = !g.uses_bf16_mixed_precision() || head_dim == 32 || head_dim == 64 || head_dim == 128;
+    const bool fused_attention = fused && kernel_head_dim;
+    size_t ctx_flat;
+    if (fused_attention) {
         // one op for the rotary embedding and steps 3-11: head split, GQA repeat, scores, scale, mask, softmax, P V, merge
-        const size_t ctx = g.attention_gqa_rope(q, k, v, num_heads, num_kv_heads, scale, causal);
-        if (residual != (size_t)-1 && !out_proj.has_bias)
-            return g.matmul_residual(ctx, out_proj.weight_id, residual, /*defer_dw=*/!q_proj.has_bias && !k_proj.has_bias && !v_proj.has_bias);
-        return out_proj.forward(g, ctx);
-    }
-    const size_t q_rope = g.rope(q, head_dim), k_rope = g.rope(k, head_dim);
-    const size_t q4 = g.reshape(q_rope, {batch, seq, num_heads, head_dim});
-    const size_t k4 = g.reshape(k_rope, {batch, seq, num_kv_heads, head_dim});
-    const size_t v4 = g.reshape(v, {batch, seq, num_kv_heads, head_dim});
-    const size_t qt = g.transpose_0213(q4), kt = g.transpose_0213(k4), vt = g.transpose_0213(v4);
-    const size_t repeats = num_heads / num_kv_heads;
-    const size_t kr = g.repeat_kv(kt, repeats), vr = g.repeat_kv(vt, repeats);
-    const size_t bh = batch * num_heads;
-    g.reinterpret_shape(qt, {bh, seq, head_dim});
-    g.reinterpret_shape(kr, {bh, seq, head_dim});
-    g.reinterpret_shape(vr, {bh, seq, head_dim});
-    size_t ctx;
-    if (g.no_grad) {
-        ctx = g.flash_attention(qt, kr, vr, scale, causal);
+        ctx_flat = g.attention_gqa_rope(q, k, v, num_heads, num_kv_heads, scale, causal);
     } else {
-        const size_t scores = g.bmm(qt, kr, true);
-        // the reference uploads a full [bh, seq, seq] tensor of `scale`; a broadcast scalar is the same product
-        const size_t scale_id = g.alloc_pooled({1});
-        g.load_tensor_data(scale_id, &scale, 1);
-        size_t scaled = g.mul(scores, scale_id);
-        if (causal) {
-            std::vector<float> mask(seq * seq, 0.0f);
-            for (size_t r = 0; r < seq; r++)
-                for (size_t c = r + 1; c < seq; c++) mask[r * seq + c] = -1e20f;
-            const size_t mask_id = g.alloc_pooled({1, seq, seq});
-            g.load_tensor_data(mask_id, mask.data(), mask.size());
-            scaled = g.add(scaled, mask_id);
+        const size_t q_rope = g.rope(q, head_dim), k_rope = g.rope(k, head_dim);
+        const size_t q4 = g.reshape(q_rope, {batch, seq, num_heads, head_dim});
+        const size_t k4 = g.reshape(k_rope, {batch, seq, num_kv_heads, head_dim});
+        const size_t v4 = g.reshape(v, {batch, seq, num_kv_heads, head_dim});
+        const size_t qt = g.transpose_0213(q4), kt = g.transpose_0213(k4), vt = g.transpose_0213(v4);
+        const size_t repeats = num_heads / num_kv_heads;
+        const size_t kr = g.repeat_kv(kt, repeats), vr = g.repeat_kv(vt, repeats);
+        const size_t bh = batch * num_heads;
+        g.reinterpret_shape(qt, {bh, seq, head_dim});
+        g.reinterpret_shape(kr, {bh, seq, head_dim});
+        g.reinterpret_shape(vr, {bh, seq, head_dim});
+        size_t ctx;
+        if (g.no_grad && kernel_head_dim) {
+            ctx = g.flash_attention(qt, kr, vr, scale, causal);
+        } else {
+            const size_t scores = g.bmm(qt, kr, true);
+            // the reference uploads a full [bh, seq, seq] tensor of `scale`; a broadcast scalar is the same product
+            const size_t scale_id = g.alloc_pooled({1});
+            g.load_tensor_data(scale_id, &scale, 1);
+            size_t scaled = g.mul(scores, scale_id);
+            if (causal) {
+                std::vector<float> mask(seq * seq, 0.0f);
+                for (size_t r = 0; r < seq; r++)
+                    for (size_t c = r + 1; c < seq; c++) mask[r * seq + c] = -1e20f;
+                const size_t mask_id = g.alloc_pooled({1, seq, seq});
+                g.load_tensor_data(mask_id, mask.data(), mask.size());
+                scaled = g.add(scaled, mask_id);
+            }
+            ctx = g.bmm(g.softmax(scaled), vr, false);
         }
-        ctx = g.bmm(g.softmax(scaled), vr, false);
+        g.reinterpret_shape(ctx, {batch, num_heads, seq, head_dim});
+        const size_t ctx_t = g.transpose_0213(ctx);
+        ctx_flat = g.reshape(ctx_t, {batch, seq, hidden_dim});
     }
-    g.reinterpret_shape(ctx, {batch, num_heads, seq, head_dim});
-    const size_t ctx_t = g.transpose_0213(ctx);
-    const size_t ctx_flat = g.reshape(ctx_t, {batch, seq, hidden_dim});
+    if (fused && residual != (size_t)-1 && !out_proj.has_bias)
+        return g.matmul_residual(ctx_flat, out_proj.weight_id, residual, /*defer_dw=*/collects());
     return out_proj.forward(g, ctx_flat);
 }
 std::vector<size_t> GroupedQueryAttention::params() const {

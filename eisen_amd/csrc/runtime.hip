@@ -54,10 +54,23 @@ extern "C" int eisen_hip_init(int device, eisen_ctx** out) {
 extern "C" int eisen_hip_pool_trim(eisen_ctx* ctx) {
     EISEN_CHECK_CTX(ctx);
     EISEN_HIP_TRY(ctx, hipSetDevice(ctx->device));
-    for (auto& kv : ctx->free_lists)
-        for (void* p : kv.second) EISEN_HIP_TRY(ctx, hipFreeAsync(p, ctx->stream));
+    // every block leaves the lists before it is freed, so a failing hipFreeAsync cannot leave a freed pointer behind
+    hipError_t first = hipSuccess;
+    for (auto& kv : ctx->free_lists) {
+        while (!kv.second.empty()) {
+            void* p = kv.second.back();
+            kv.second.pop_back();
+            ctx->cached_bytes -= kv.first;
+            const hipError_t e = hipFreeAsync(p, ctx->stream);
+            if (e != hipSuccess && first == hipSuccess) first = e;
+        }
+    }
     ctx->free_lists.clear();
     ctx->cached_bytes = 0;
+    if (first != hipSuccess) {
+        (void)hipGetLastError();
+        return eisen_set_error(ctx, (int)first, "eisen_hip_pool_trim: hipFreeAsync failed: %s", hipGetErrorString(first));
+    }
     return 0;
 }
 
@@ -157,8 +170,7 @@ extern "C" int eisen_hip_malloc(eisen_ctx* ctx, size_t bytes, void** out) {
 extern "C" int eisen_hip_malloc_zeroed(eisen_ctx* ctx, size_t bytes, void** out) {
     int rc = eisen_hip_malloc(ctx, bytes, out);
     if (rc) return rc;
-    EISEN_HIP_TRY(ctx, hipMemsetAsync(*out, 0, ctx->live[*out], ctx->stream));
-    return 0;
+    return eisen_hip_memset_zero(ctx, *out, ctx->live[*out]);
 }
 
 extern "C" int eisen_hip_free(eisen_ctx* ctx, void* ptr) {
@@ -269,6 +281,9 @@ extern "C" int eisen_hip_memset_zero(eisen_ctx* ctx, void* dst, size_t bytes) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, dst != nullptr, EISEN_E_ARG, "eisen_hip_memset_zero: null pointer");
     if (bytes == 0) return 0;
+    // a fill kernel, not hipMemsetAsync: a memset node recorded into a captured graph has replayed wrongly on this
+    // hardware generation, and callers may capture the step
+    if (bytes % 4 == 0 && eisen_aligned(dst, 4)) return eisen_hip_fill(ctx, dst, EISEN_F32, 0.0f, bytes / 4);
     EISEN_HIP_TRY(ctx, hipMemsetAsync(dst, 0, bytes, ctx->stream));
     return 0;
 }

@@ -146,6 +146,12 @@ int eisen_hip_mul_bcast(eisen_ctx* ctx, const void* a, const void* b, void* out,
 int eisen_hip_bcast_backward(eisen_ctx* ctx, void* dst, const void* grad_out, const void* other, int dtype,
                              int rank, const size_t* out_shape, const size_t* dst_strides,
                              const size_t* other_strides, size_t dst_numel, int accumulate);
+/* The same with an f32 destination whatever `dtype` the operands have: the gradient of a parameter operand (a Linear
+ * bias, src/nn/linear.rs:88-93 `g.add(out, bias)`) in mixed precision, where gradients of activations are bf16 and
+ * gradients of parameters f32.  Also covers an operand of the full output shape (no reduced dimension). */
+int eisen_hip_bcast_backward_f32(eisen_ctx* ctx, float* dst, const void* grad_out, const void* other, int dtype,
+                                 int rank, const size_t* out_shape, const size_t* dst_strides,
+                                 const size_t* other_strides, size_t dst_numel, int accumulate);
 /* mul_backward_f32 same-shape (kernels/ops_f32.cu:119): ga (+)= b*go, gb (+)= a*go.
  * ga or gb may be NULL (constant operand). */
 int eisen_hip_mul_backward(eisen_ctx* ctx, const void* a, const void* b, const void* go, void* ga, void* gb,

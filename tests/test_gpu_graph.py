@@ -254,6 +254,37 @@ def test_deferred_weight_gradients_bf16_mixed_step(ctx):
     _train_steps(ctx, cfg, G.BF16_MIXED, 2, 128, steps=1, accum=2, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
 
 
+def test_biased_linear_and_parameter_operands_bf16_mixed(ctx):
+    """Linear::forward with a bias (src/nn/linear.rs:88-93: matmul, then `g.add(out, bias)`), a product with a parameter
+    vector and a sum with a parameter of the full shape, in mixed precision: the activations' gradients are bf16, the
+    parameters' f32, and every parameter gradient is checked against the oracle."""
+    from eisen_amd import hip
+    M, K, N = 96, 64, 48
+    vals = dict(x=hip.round_bf16(gen.normal(41, (M, K))), w=hip.round_bf16(gen.normal(42, (K, N), 0.2)), b=hip.round_bf16(gen.normal(43, (N,), 0.3)),
+                gain=hip.round_bf16(1.0 + gen.normal(44, (N,), 0.2)), full=hip.round_bf16(gen.normal(45, (M, N), 0.3)))
+    targets = gen.uniform_ids(46, (M,), N)
+    grads = []
+    for graph in (G.Graph(ctx, G.BF16_MIXED), R.Graph()):
+        ids = {k: graph.alloc(v.shape, v) for k, v in vals.items()}
+        for accum in range(2):  # the second pass adds into the f32 gradients
+            h = graph.add(graph.matmul(ids["x"], ids["w"]), ids["b"])
+            h = graph.mul(h, ids["gain"])
+            h = graph.add(ids["full"], h)
+            graph.backward(graph.cross_entropy(h, targets))
+        grads.append({k: (graph.sync_grad_to_cpu(i) if isinstance(graph, G.Graph) else graph.grad(i)) for k, i in ids.items()})
+        if isinstance(graph, G.Graph):
+            graph.close()
+    for k in vals:
+        assert_close(grads[0][k], grads[1][k], 2e-2, f"grad {k}")
+
+
+def test_head_dim_without_a_fused_kernel_bf16_mixed_step(ctx):
+    """head_dim 96 in mixed precision: the bf16 attention kernels cover 32, 64 and 128, so the block takes the reference's
+    materialised chain (rope, transposes, repeat_kv, bmm, scale, mask, softmax, bmm) while everything around it stays fused."""
+    cfg = dict(vocab=128, hidden=192, heads=2, kv_heads=1, ffn=256, layers=1, tie=False)
+    _train_steps(ctx, cfg, G.BF16_MIXED, 2, 64, steps=1, accum=2, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
+
+
 def test_config5_layers_fused_path_matches_the_reference_chain(ctx):
     """Two layers at config 5's real width and micro-batch (d 2048, 32 q / 8 kv heads, ffn 5632, 4 x 1024 tokens): the fused
     path (grouped and deferred weight gradients, SwiGLU inside the GEMMs, side stream, rotary embedding inside attention)
