@@ -266,16 +266,18 @@ def test_biased_linear_and_parameter_operands_bf16_mixed(ctx):
     grads = []
     for graph in (G.Graph(ctx, G.BF16_MIXED), R.Graph()):
         ids = {k: graph.alloc(v.shape, v) for k, v in vals.items()}
+        graph.mark_params()
         for accum in range(2):  # the second pass adds into the f32 gradients
             h = graph.add(graph.matmul(ids["x"], ids["w"]), ids["b"])
             h = graph.mul(h, ids["gain"])
             h = graph.add(ids["full"], h)
             graph.backward(graph.cross_entropy(h, targets))
+            graph.clear_activations()
         grads.append({k: (graph.sync_grad_to_cpu(i) if isinstance(graph, G.Graph) else graph.grad(i)) for k, i in ids.items()})
         if isinstance(graph, G.Graph):
             graph.close()
     for k in vals:
-        assert_close(grads[0][k], grads[1][k], 2e-2, f"grad {k}")
+        assert_close(grads[0][k], grads[1][k], 2e-2, f"grad {k}", step=True)  # five bf16 ops composed
 
 
 def test_head_dim_without_a_fused_kernel_bf16_mixed_step(ctx):
