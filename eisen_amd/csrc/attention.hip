@@ -44,6 +44,15 @@ struct AttnArgs {
     const float2* rope;
 };
 
+// Scratch of eisen_hip_attention_backward_noalloc: D = rowsum(dO o O), one float per (batch, query head, position).
+// A file-scope device array instead of a workspace allocation, so that entry point never calls an allocator.  Every
+// GPU the library runs on holds its own 4 MiB copy until the process ends; the name below is only a host-side handle,
+// the device address of each GPU's copy comes from hipGetSymbolAddress (eisen_attention_scratch_init).
+constexpr size_t kNoAllocMaxRows = size_t(1) << 20;
+static __device__ __align__(256) float g_attn_bwd_scratch[kNoAllocMaxRows];
+constexpr int kMaxDevices = 64;
+static float* g_attn_bwd_scratch_ptr[kMaxDevices] = {nullptr};  // per device, filled once
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -882,11 +891,25 @@ extern "C" int eisen_hip_attention_forward(eisen_ctx* ctx, const void* q, const 
     return 0;
 }
 
+int eisen_attention_scratch_init(eisen_ctx* ctx) {
+    EISEN_REQUIRE(ctx, ctx->device >= 0 && ctx->device < kMaxDevices, EISEN_E_ARG, "device index %d beyond the %d this library keeps scratch for", ctx->device, kMaxDevices);
+    if (!g_attn_bwd_scratch_ptr[ctx->device]) {
+        float* p = nullptr;
+        EISEN_HIP_TRY(ctx, hipSetDevice(ctx->device));
+        EISEN_HIP_TRY(ctx, hipGetSymbolAddress((void**)&p, HIP_SYMBOL(g_attn_bwd_scratch)));
+        EISEN_REQUIRE(ctx, p != nullptr, EISEN_E_STATE, "hipGetSymbolAddress returned a null address for the attention scratch");
+        g_attn_bwd_scratch_ptr[ctx->device] = p;
+    }
+    ctx->attn_scratch = g_attn_bwd_scratch_ptr[ctx->device];
+    return 0;
+}
+
+// scratch: where D = rowsum(dO o O) goes; nullptr = the context's grow-only workspace
 static int attention_backward_common(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
                                      const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype,
                                      size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
                                      const long long* q_strides, const long long* kv_strides, float scale,
-                                     int causal, bool rope) {
+                                     int causal, bool rope, float* scratch = nullptr) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, q && k && v && out && dout && lse && dq && dk && dv, EISEN_E_ARG, "attention_backward: null pointer");
     AttnArgs a{};
@@ -894,10 +917,14 @@ static int attention_backward_common(eisen_ctx* ctx, const void* q, const void* 
     if (rc) return rc;
     a.Q = q; a.K = k; a.V = v; a.O = out; a.dO = dout; a.LSE = const_cast<float*>(lse);
     a.dQ = dq; a.dK = dk; a.dV = dv;
-    void* ws = nullptr;
-    rc = eisen_workspace(ctx, B * Hq * S * sizeof(float), &ws);
-    if (rc) return rc;
-    a.D = static_cast<float*>(ws);
+    if (scratch) {
+        a.D = scratch;
+    } else {
+        void* ws = nullptr;
+        rc = eisen_workspace(ctx, B * Hq * S * sizeof(float), &ws);
+        if (rc) return rc;
+        a.D = static_cast<float*>(ws);
+    }
     if (rope) {
         rc = eisen_rope_table_get(ctx, S, hd, &a.rope);
         if (rc) return rc;
@@ -926,6 +953,26 @@ extern "C" int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const
                                             const long long* q_strides, const long long* kv_strides, float scale,
                                             int causal) {
     return attention_backward_common(ctx, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, q_strides, kv_strides, scale, causal, false);
+}
+
+extern "C" int eisen_hip_attention_backward_noalloc(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                                    const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype,
+                                                    size_t B, size_t S, size_t Hq, size_t Hkv, size_t hd,
+                                                    const long long* q_strides, const long long* kv_strides, float scale,
+                                                    int causal) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, ctx->attn_scratch != nullptr, EISEN_E_STATE, "attention_backward_noalloc: the context has no scratch address");
+    EISEN_REQUIRE(ctx, B > 0 && S > 0 && Hq > 0 && B <= kNoAllocMaxRows && S <= kNoAllocMaxRows && Hq <= kNoAllocMaxRows &&
+                           B * Hq <= kNoAllocMaxRows && B * Hq * S <= kNoAllocMaxRows,
+                  EISEN_E_SHAPE, "attention_backward_noalloc: batch * query heads * seq = %zu * %zu * %zu exceeds the %zu rows of the fixed scratch",
+                  B, Hq, S, kNoAllocMaxRows);
+    // per-kernel profiling creates events on first use: off for the duration of this call
+    const bool prof_was = ctx->prof.enabled;
+    ctx->prof.enabled = false;
+    const int rc = attention_backward_common(ctx, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, q_strides, kv_strides, scale, causal,
+                                             false, ctx->attn_scratch);
+    ctx->prof.enabled = prof_was;
+    return rc;
 }
 
 extern "C" int eisen_hip_attention_rope_backward(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,

@@ -60,12 +60,17 @@ struct eisen_ctx {
     void* ws = nullptr;
     size_t ws_bytes = 0;
     std::vector<eisen_rope_table> rope_tables;
+    float* attn_scratch = nullptr;  // this device's copy of the file-scope scratch array in attention.hip (never freed)
     eisen_prof prof;
     char last_error[512] = {0};
 };
 
 // cos/sin table of the rotary embedding, [seq][head_dim/2] float2 on the device, cached in the context (rope.hip)
 int eisen_rope_table_get(eisen_ctx* ctx, size_t seq, size_t head_dim, const float2** out);
+
+// Looks up, once per device, the device address of the file-scope scratch array that eisen_hip_attention_backward_noalloc
+// uses, and stores it in the context (attention.hip); called by eisen_hip_init with the context's device current.
+int eisen_attention_scratch_init(eisen_ctx* ctx);
 
 // Brackets the launches issued during its lifetime when profiling is on; free when it is off.
 int eisen_prof_begin(eisen_ctx* ctx, const char* name, double work, bool is_flops);

@@ -47,6 +47,11 @@ extern "C" int eisen_hip_init(int device, eisen_ctx** out) {
         delete ctx;
         return (int)e;
     }
+    const int rc = eisen_attention_scratch_init(ctx);
+    if (rc != 0) {
+        (void)eisen_hip_destroy(ctx);
+        return rc;
+    }
     *out = ctx;
     return 0;
 }

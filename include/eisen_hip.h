@@ -293,6 +293,19 @@ int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const void* k, c
                                  size_t S, size_t Hq, size_t Hkv, size_t hd, const long long* q_strides,
                                  const long long* kv_strides, float scale, int causal);
 
+/* eisen_hip_attention_backward for callers that cannot allocate (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and the same
+ * results; the one buffer the kernels need beyond the inputs and outputs, D = rowsum(dO o O) with one float per
+ * (batch, query head, position), lives in a fixed 4 MiB device array of the library instead of the context's growing
+ * workspace, so the call reaches no hipMalloc / hipFree / pool routine.  Limit: B * Hq * S <= 1,048,576, larger
+ * shapes return EISEN_E_SHAPE.  Every call on one GPU uses that GPU's one array: calls that overlap on a GPU (two
+ * contexts, two streams) race; calls on one context are ordered by its stream.  Nothing in the array has to be
+ * cleared between calls: the dQ kernel writes every row that the dK/dV kernel reads. */
+int eisen_hip_attention_backward_noalloc(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
+                                         const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype, size_t B,
+                                         size_t S, size_t Hq, size_t Hkv, size_t hd, const long long* q_strides,
+                                         const long long* kv_strides, float scale, int causal);
+
 /* eisen_hip_attention_backward for q and k that are rotary-embedded projections, q = rope(q0), k = rope(k0)
  * (src/nn/attention.rs:316-317 applies `g.rope` to both before the attention chain): dq and dk receive the
  * gradients of q0 and k0, i.e. the rotary backward (src/graph/ops/transform.rs:592-595) is applied to the f32
