@@ -31,49 +31,70 @@ def ctx():
     c.close()
 
 
-def assert_close(actual, expected, rtol, name="", row_scale=False, l2=None, step=False):
+# Every assert_close call leaves its observed figures here; tests/conftest.py prints the worst per tolerance class at the
+# end of the run, so the head-room (or lack of it) under the bounds above is visible in the test log.
+OBSERVED = []
+
+
+def _record(name, kind, rtol, a_size, rel_l2, frac_outside, worst_ratio):
+    OBSERVED.append(dict(name=name, kind=kind, rtol=rtol, n=int(a_size), rel_l2=float(rel_l2), frac_outside=float(frac_outside),
+                         worst_ratio=float(worst_ratio)))
+
+
+def assert_close(actual, expected, rtol, name="", row_scale=False, l2=None, step=False, step_outliers=0.0):
     """step: the composed-step criterion above (scale = max|e| instead of rms(e), no outlier allowance,
-    relative L2 <= rtol).
+    relative L2 <= rtol).  step_outliers: fraction of the elements that may exceed the step bound, by at most 4x -- only
+    for comparisons of two bf16 results with each other (both sides carry rounding noise), never against the oracle.
     row_scale: take rms(e) per last-dim row instead of over the whole tensor -- for tensors whose
     rows differ by orders of magnitude (an embedding gradient: untouched rows are exactly zero, hot
     rows are large), where one global RMS is not the scale of any element.  l2: bound on the
-    relative L2 error for the bf16 check (default 1e-2)."""
+    relative L2 error for the bf16 check (default 1e-2).
+    Every failure message carries the observed relative L2 error, the fraction of elements outside the
+    per-element bound and the worst error as a multiple of that bound."""
     a = np.asarray(actual, np.float64)
     e = np.asarray(expected, np.float64)
     assert a.shape == e.shape, f"{name}: shape {a.shape} vs {e.shape}"
     assert np.isfinite(a).all(), f"{name}: non-finite values in the result"
+    err = np.abs(a - e)
+    den = float(np.sum(e * e))
+    rel_l2 = float(np.sqrt(np.sum(err * err) / den)) if den > 0 else 0.0
     if step:
         scale_el = np.abs(e).max(axis=-1, keepdims=True) if (row_scale and e.ndim >= 2) else np.abs(e).max()
-        err = np.abs(a - e)
         tol = rtol * np.abs(e) + rtol * scale_el + 1e-30
-        if (err > tol).any():
-            i = int(np.argmax((err / tol).reshape(-1)))
-            raise AssertionError(f"{name}: {int((err > tol).sum())}/{a.size} elements outside the step bound; worst at {i}: "
-                                 f"got {a.reshape(-1)[i]:.8g}, expected {e.reshape(-1)[i]:.8g}")
-        den = float(np.sum(e * e))
-        if den > 0:
-            rel_l2 = float(np.sqrt(np.sum(err * err) / den))
-            assert rel_l2 <= rtol, f"{name}: relative L2 error {rel_l2:.3g} > {rtol:g}"
+        ratio = err / tol
+        frac = float((ratio > 1).mean()) if a.size else 0.0
+        worst = float(ratio.max()) if a.size else 0.0
+        _record(name, "bf16 step", rtol, a.size, rel_l2, frac, worst)
+        seen = f"observed: relative L2 {rel_l2:.3g}, {frac:.3g} of the elements outside the bound, worst error {worst:.3g} x bound"
+        if (ratio > 1).sum() > int(step_outliers * a.size) or worst > 4:
+            i = int(np.argmax(ratio.reshape(-1)))
+            raise AssertionError(f"{name}: {int((ratio > 1).sum())}/{a.size} elements outside the step bound; worst at {i}: "
+                                 f"got {a.reshape(-1)[i]:.8g}, expected {e.reshape(-1)[i]:.8g}; {seen}")
+        bound = rtol if l2 is None else l2
+        assert rel_l2 <= bound, f"{name}: relative L2 error {rel_l2:.3g} > {bound:g}; {seen}"
         return
     if row_scale and e.ndim >= 2:
         rms_el = np.broadcast_to(np.sqrt(np.mean(e * e, axis=-1, keepdims=True)), e.shape).reshape(-1)
     else:
         rms_el = None
-    a, e = a.reshape(-1), e.reshape(-1)
+    a, e, err = a.reshape(-1), e.reshape(-1), err.reshape(-1)
     rms = float(np.sqrt(np.mean(e * e))) if e.size else 0.0
     tol = rtol * np.abs(e) + rtol * (rms_el if rms_el is not None else rms) + 1e-30
-    err = np.abs(a - e)
-    bad = err > tol
+    ratio = err / tol
+    bad = ratio > 1
+    frac = float(bad.mean()) if a.size else 0.0
+    worst = float(ratio.max()) if a.size else 0.0
     loose = rtol >= RTOL_BF16          # bf16: allow 1e-4 of the elements up to 2x the bound
+    _record(name, "bf16 kernel" if loose else "f32 kernel", rtol, a.size, rel_l2, frac, worst)
+    seen = f"observed: relative L2 {rel_l2:.3g}, {frac:.3g} of the elements outside the bound, worst error {worst:.3g} x bound"
     allowed = int(1e-4 * a.size) + 1 if loose else 0
-    if bad.sum() > allowed or (loose and (err > 2 * tol).any()):
-        i = int(np.argmax(err / tol))
+    if bad.sum() > allowed or (loose and worst > 2):
+        i = int(np.argmax(ratio))
         raise AssertionError(f"{name}: {int(bad.sum())}/{a.size} elements outside rtol {rtol:g}; worst at {i}: "
-                             f"got {a[i]:.8g}, expected {e[i]:.8g}, rms {rms:.4g}")
+                             f"got {a[i]:.8g}, expected {e[i]:.8g}, rms {rms:.4g}; {seen}")
     if loose and rms > 0:
-        rel_l2 = float(np.sqrt(np.sum(err * err) / np.sum(e * e)))
         bound = 1e-2 if l2 is None else l2
-        assert rel_l2 <= bound, f"{name}: relative L2 error {rel_l2:.3g} > {bound:g}"
+        assert rel_l2 <= bound, f"{name}: relative L2 error {rel_l2:.3g} > {bound:g}; {seen}"
 
 
 def tol_for(dtype):

@@ -1012,31 +1012,44 @@ def test_attention_rope_backward(ctx, dtype, B, S, Hq, Hkv, hd):
         x.free()
 
 
-def test_attention_config3_full_size_properties(ctx):
-    """B8 S1024 Hq16 Hkv4 hd64 bf16 (config 3): too large for the unfused oracle in seconds, so check
-    one batch element's heads of one KV group against the oracle (S=1024 is kept), and size-independent
-    properties on the whole output: row-stochastic P implies O of a constant V is that constant; the
-    deterministic kernels give identical bits on a second run."""
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+def test_attention_config3_full_size_properties(ctx, layout):
+    """B8 S1024 Hq16 Hkv4 hd64 bf16 (config 3), in the [B,H,S,hd] layout config 3 states (the reference's q_t layout,
+    addressed through strides) and in the [B,S,H,hd] layout the projections produce: too large for the unfused oracle in
+    seconds, so check one batch element's heads of one KV group against the oracle (S=1024 is kept), and size-independent
+    properties on the whole output: row-stochastic P implies O of a constant V is that constant; the deterministic kernels
+    give identical bits on a second run."""
     B, S, Hq, Hkv, hd = 8, 1024, 16, 4, 64
     sd = 1.0 / 8
+    # generated as [B,S,H,hd] (the oracle's layout); `dev` puts a tensor into the layout under test, `host` brings it back
     q, do = prep(gen.normal(600, (B, S, Hq, hd), sd), BF16), prep(gen.normal(601, (B, S, Hq, hd), sd), BF16)
     k, v = prep(gen.normal(602, (B, S, Hkv, hd), sd), BF16), prep(gen.normal(603, (B, S, Hkv, hd), sd), BF16)
-    dq_, dk_, dv_, ddo = up(ctx, q, BF16), up(ctx, k, BF16), up(ctx, v, BF16), up(ctx, do, BF16)
+    if layout == "bhsd":
+        qs, ks = (Hq * S * hd, hd, S * hd), (Hkv * S * hd, hd, S * hd)
+        dev = lambda x: np.ascontiguousarray(x.transpose(0, 2, 1, 3))
+        host = lambda buf, ref: dn(ctx, buf, dev(ref).shape, BF16).transpose(0, 2, 1, 3)
+    else:
+        qs = ks = None
+        dev = lambda x: x
+        host = lambda buf, ref: dn(ctx, buf, ref.shape, BF16)
+    dq_, dk_, dv_, ddo = up(ctx, dev(q), BF16), up(ctx, dev(k), BF16), up(ctx, dev(v), BF16), up(ctx, dev(do), BF16)
     out, lse = ctx.malloc(q.size * 2), ctx.malloc(B * Hq * S * 4)
     gq, gk, gv = ctx.malloc(q.size * 2), ctx.malloc(k.size * 2), ctx.malloc(k.size * 2)
-    ctx.attention_forward(dq_, dk_, dv_, out, lse, BF16, B, S, Hq, Hkv, hd, 0.125, True)
-    ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, BF16, B, S, Hq, Hkv, hd, 0.125, True)
-    o1, q1, k1, v1 = dn(ctx, out, q.shape, BF16), dn(ctx, gq, q.shape, BF16), dn(ctx, gk, k.shape, BF16), dn(ctx, gv, k.shape, BF16)
+    ctx.attention_forward(dq_, dk_, dv_, out, lse, BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+    ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+    o1, q1, k1, v1 = host(out, q), host(gq, q), host(gk, k), host(gv, k)
     # slice: batch 3, KV group 2 (query heads 8..11) -> an independent sub-problem
     b, grp = 3, 2
     hs = slice(grp * 4, grp * 4 + 4)
     eo, edq, edk, edv = oracle_attention(q[b:b + 1, :, hs], k[b:b + 1, :, grp:grp + 1], v[b:b + 1, :, grp:grp + 1], do[b:b + 1, :, hs], np.float32(0.125))
-    assert_close(o1[b:b + 1, :, hs], eo, 2e-2, "O slice")
-    assert_close(q1[b:b + 1, :, hs], edq, 2e-2, "dQ slice")
-    assert_close(k1[b:b + 1, :, grp:grp + 1], edk, 2e-2, "dK slice")
-    assert_close(v1[b:b + 1, :, grp:grp + 1], edv, 2e-2, "dV slice")
-    ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, BF16, B, S, Hq, Hkv, hd, 0.125, True)
-    assert np.array_equal(dn(ctx, gq, q.shape, BF16), q1) and np.array_equal(dn(ctx, gk, k.shape, BF16), k1)
+    assert_close(o1[b:b + 1, :, hs], eo, 2e-2, f"config 3 {layout} O slice")
+    assert_close(q1[b:b + 1, :, hs], edq, 2e-2, f"config 3 {layout} dQ slice")
+    assert_close(k1[b:b + 1, :, grp:grp + 1], edk, 2e-2, f"config 3 {layout} dK slice")
+    assert_close(v1[b:b + 1, :, grp:grp + 1], edv, 2e-2, f"config 3 {layout} dV slice")
+    ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+    assert np.array_equal(host(gq, q), q1) and np.array_equal(host(gk, k), k1) and np.array_equal(host(gv, k), v1)
     ones = up(ctx, np.full(k.shape, 0.5, np.float32), BF16)
-    ctx.attention_forward(dq_, dk_, ones, out, lse, BF16, B, S, Hq, Hkv, hd, 0.125, True)
+    ctx.attention_forward(dq_, dk_, ones, out, lse, BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
     assert np.abs(dn(ctx, out, q.shape, BF16) - 0.5).max() <= 0.5 * 2e-2
+    for x in (dq_, dk_, dv_, ddo, out, lse, gq, gk, gv, ones):
+        x.free()
