@@ -1,20 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the training step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c4|c3|c2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c5|c4|c3|c2]
 
-Default workload c5 = the headline configuration (config 5): the "~1.1B" Llama-style model (vocab 32000, d 2048,
-16 layers, 32 query / 8 KV heads, head_dim 64, SiLU-gated MLP 5632, untied lm_head), seq 1024,
-micro-batch 4, gradient accumulation 8 (32,768 tokens per optimiser step), bf16 activations and
-matmuls, f32 master weights and AdamW state, synthetic Zipf(1.1) token ids, N(0, 0.02) weights.
-One "step" = zero_grad, 8 x (upload ids, forward, fused cross entropy, backward), gradient-norm
-clip, fused AdamW -- the loop of examples/train_llm.rs:386-477.
+The headline line is config 5: the "~1.1B" Llama-style model (vocab 32000, d 2048, 16 layers, 32 query / 8 KV
+heads, head_dim 64, SiLU-gated MLP 5632, untied lm_head), seq 1024, micro-batch 4, gradient accumulation 8
+(32,768 tokens per optimiser step), bf16 activations and matmuls, f32 master weights and AdamW state, synthetic
+Zipf(1.1) token ids, N(0, 0.02) weights.  One "step" = zero_grad, 8 x (upload ids, forward, fused cross entropy,
+loss read-back, backward), gradient-norm clip, fused AdamW -- the loop of examples/train_llm.rs:386-477, the
+per-micro-batch loss read-back of :450 included (the copy is queued before the backward pass and collected
+after it, so reading it does not drain the device).
 
-Prints one JSON line.  `value` is tokens/s over K timed steps (inputs resident in host memory,
-weights and optimiser state resident in HBM).  `roofline` describes the kernel that takes the
-largest share of the step, timed with HIP events on the library's stream in one extra,
-instrumented step.  `cpu_baseline` times the CPU oracle (a single-threaded restatement of the
-reference's Device::Cpu path) on a bounded sample of the same architecture.
+Prints one JSON line.  `value` is tokens/s over K timed steps (inputs resident in host memory, weights and
+optimiser state resident in HBM).  `roofline` describes the kernel symbol that takes the largest share of the
+step, timed with HIP events on the library's stream in one extra, instrumented step; `kernels` lists every
+instrumented launch family with its achieved TFLOP/s or GB/s.  `cpu_baseline` times the CPU oracle (a
+restatement of the reference's Device::Cpu path) on a bounded sample of the same architecture.  With the default
+`--workload all` the line also carries `other_configs`: the same figures for config 4 (the "14M" model), config 3
+(flash attention forward + backward: the MFMA utilisation of the backward) and config 2 (fused cross entropy).
 """
 import argparse
 import json
@@ -32,14 +35,11 @@ from eisen_amd import synth as gen  # noqa: E402  (seeded synthetic inputs, the 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic_pmc.md
-# (fetch x 1.997, write x 1.000 after calibration on the library's copy kernel), per workload and per profile
-# name the library reports.  The config-5 GEMM figures are averages over that entry's launches in the step.
+# HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs, per workload and per kernel symbol as
+# `symbol_of` names it; the summaries (command, calibration factors, per-kernel rows) are the files named here.
+TRAFFIC_SOURCE = {"c5": "profiles/c5_step_hbm_traffic_pmc.md", "c3": "profiles/c2_c3_hbm_traffic_pmc.md", "c2": "profiles/c2_c3_hbm_traffic_pmc.md"}
 MEASURED_TRAFFIC = {
-    "c5": {"gemm_nn_bf16_bf16out_256x128x64": 253.7e6, "gemm_nt_bf16_bf16out_256x128x64": 437.4e6,
-           "gemm_nt_bf16_bf16out_256x128x64_swiglu_bwd": 473.7e6, "gemm_nn_bf16_swiglu_256x128x32": 565.8e6,
-           "gemm_tn_bf16_f32out_256x128x32": 576.6e6, "gemm_tn_bf16_f32out_256x128x32_grouped": 1252.8e6,
-           "gemm_nn_bf16_bf16out_128x128x64": 84.1e6, "gemm_nn_bf16_bf16out_256x256x32": 1561.1e6, "ce_fused_bf16": 524.6e6},
+    "c5": {},
     "c4": {},
     "c3": {"attn_bwd": 78.0e6 + 51.7e6},
     "c2": {"ce_fused_bf16": 1048.9e6},
@@ -65,64 +65,101 @@ def arch(c):
     return {k: c[k] for k in ("vocab", "hidden", "heads", "kv_heads", "ffn", "layers", "tie")}
 
 
-def pick_dominant(prof, workload):
-    name = max(prof, key=lambda k: prof[k]["ms"])
-    e = prof[name]
-    per_launch_ms = e["ms"] / e["launches"]
+def symbol_of(name):
+    """Profile entries name one launch family; families that run the same kernel symbol (the plain and the grouped
+    launch of one GEMM instantiation) are one row of a rocprofv3 kernel trace and are added up here as well."""
+    return name[:-len("_grouped")] if name.endswith("_grouped") else name
+
+
+def by_symbol(prof):
+    out = {}
+    for name, e in prof.items():
+        s = out.setdefault(symbol_of(name), dict(ms=0.0, launches=0, work=0.0, unit=e["unit"], families=[]))
+        s["ms"] += e["ms"]
+        s["launches"] += e["launches"]
+        s["work"] += e["work"]
+        s["families"].append(name)
+    return out
+
+
+def roofline_of(name, e, workload):
+    """achieved = algorithmic work of the symbol's launches / their summed duration (= work per launch / average
+    launch duration, weighted over the shapes the symbol ran)."""
+    traffic = MEASURED_TRAFFIC.get(workload, {}).get(name)
+    src = TRAFFIC_SOURCE.get(workload) if traffic is not None else None
     if e["unit"] == "flop":
-        achieved = e["work"] / e["launches"] / (per_launch_ms * 1e-3) / 1e12
-        return name, dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                          frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(workload, {}).get(name))
-    achieved = e["work"] / e["launches"] / (per_launch_ms * 1e-3) / 1e9
-    return name, dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(workload, {}).get(name))
+        achieved = e["work"] / (e["ms"] * 1e-3) / 1e12
+        r = dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s", frac=round(achieved / PEAK_BF16_TFLOPS, 4))
+    else:
+        achieved = e["work"] / (e["ms"] * 1e-3) / 1e9
+        r = dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s", frac=round(achieved / PEAK_HBM_GBS, 4))
+    r.update(traffic=traffic, traffic_source=src, kernel=name, launches=e["launches"], avg_us=round(1e3 * e["ms"] / e["launches"], 2))
+    return r
+
+
+def pick_dominant(prof, workload):
+    sym = by_symbol(prof)
+    name = max(sym, key=lambda k: sym[k]["ms"])
+    r = roofline_of(name, sym[name], workload)
+    if len(sym[name]["families"]) > 1:
+        r["families"] = sorted(sym[name]["families"])
+    return r
 
 
 def kernel_table(prof):
     rows = []
     for name, e in sorted(prof.items(), key=lambda kv: -kv[1]["ms"]):
         rate = e["work"] / (e["ms"] * 1e-3) if e["ms"] > 0 else 0.0
+        flop = e["unit"] == "flop"
         rows.append(dict(kernel=name, ms=round(e["ms"], 3), launches=e["launches"], avg_us=round(1e3 * e["ms"] / e["launches"], 2),
-                         rate=round(rate / (1e12 if e["unit"] == "flop" else 1e9), 2), rate_unit="TFLOP/s" if e["unit"] == "flop" else "GB/s"))
+                         rate=round(rate / (1e12 if flop else 1e9), 2), rate_unit="TFLOP/s" if flop else "GB/s",
+                         frac=round(rate / (1e12 * PEAK_BF16_TFLOPS if flop else 1e9 * PEAK_HBM_GBS), 4)))
     return rows
 
 
 # ---------------------------------------------------------------------------------------------
-# CPU baseline: the oracle (port of the reference's single-threaded CPU arms) on a bounded sample
+# CPU baseline: the oracle (port of the reference's CPU arms) on a bounded sample
 # ---------------------------------------------------------------------------------------------
 
-def cpu_baseline_lm(c, budget_tokens):
-    """Times fwd+bwd of a 1-layer and a 2-layer model of the same width/vocab on `budget_tokens` tokens,
-    separates the per-layer from the embedding/lm_head/CE cost, and extrapolates to the full depth."""
+def cpu_threads():
+    return max(1, min(16, os.cpu_count() or 1))
+
+
+def cpu_baseline_lm(c, seq, mb=1):
+    """One micro-step (forward, cross entropy, backward) of a 0-layer and a 1-layer model of the configuration's width
+    and vocabulary on mb x seq tokens: the difference is one transformer layer (attention with its S^2 part at this
+    seq), the 0-layer run is embedding + final norm + lm_head + cross entropy.  Extrapolated to the full depth."""
     from oracle import cpu_ref as R
-    R.set_threads(1)
+    threads = cpu_threads()
+    R.set_threads(threads)
     times = {}
-    for layers in (1, 2):
+    for layers in (0, 1):
         cfg = dict(arch(c), layers=layers)
         g = R.Graph()
         lm = R.TransformerLM(g, **cfg)
         for pid, (_, w) in enumerate(gen.lm_weights(5, **cfg)):
             g.load_tensor_data(pid, w)
         g.mark_params()
-        x, y = gen.lm_batch(9, 1, budget_tokens, c["vocab"], "zipf")
-        lm.micro_step(x, y)                      # untimed: first touch of the gradient pages
+        x, y = gen.lm_batch(9, mb, seq, c["vocab"], "zipf")
         t0 = time.perf_counter()
         lm.micro_step(x, y)
         times[layers] = time.perf_counter() - t0
         del lm, g
-    per_layer = max(times[2] - times[1], 1e-9)
-    head = max(times[1] - per_layer, 0.0)
-    per_token = (c["layers"] * per_layer + head) / budget_tokens
-    return dict(value=round(1.0 / per_token, 3), unit="tokens/s", cores=1, kind="port",
-                sample=(f"oracle fwd+bwd of 1- and 2-layer models of this width/vocab on {budget_tokens} tokens (seq {budget_tokens}, so the "
-                        f"S^2 attention share is understated), {times[1]:.1f}s + {times[2]:.1f}s, extrapolated to {c['layers']} layers; AdamW excluded"))
+    per_layer = max(times[1] - times[0], 1e-9)
+    per_token = (c["layers"] * per_layer + times[0]) / (mb * seq)
+    note = "" if seq >= c["seq"] else f" (at seq {seq} the S^2 attention term has {seq / c['seq']:.2g} of its share at seq {c['seq']})"
+    return dict(value=round(1.0 / per_token, 3), unit="tokens/s", cores=threads, kind="port",
+                sample=(f"oracle forward + cross entropy + backward on {mb} x {seq} tokens of this width and vocabulary: 0 layers "
+                        f"(embedding, final norm, lm_head, CE) {times[0]:.1f} s, 1 layer {times[1]:.1f} s, extrapolated to {c['layers']} layers{note}; "
+                        f"AdamW excluded; the reference's CPU path itself is single-threaded, the port runs its row loops on {threads} threads "
+                        f"with identical results"))
 
 
 # ---------------------------------------------------------------------------------------------
 # workloads
 # ---------------------------------------------------------------------------------------------
 
-def bench_lm(name, steps, warmup, cpu_tokens):
+def bench_lm(name, steps, warmup, with_cpu=True):
     from eisen_amd import graph as G
     from eisen_amd import hip
     c = CONFIGS[name]
@@ -145,7 +182,7 @@ def bench_lm(name, steps, warmup, cpu_tokens):
 
     step_no = [0]
 
-    def one_step(want_loss=False):
+    def one_step():
         # linear warm-up of the reference's CosineScheduler (src/nn/scheduler.rs:45-55; train_llm.rs:391-392)
         opt.config(g.cosine_lr(3e-4, 3e-5, 100, 10000, step_no[0]), 0.9, 0.95, 1e-8, 0.1, 1.0)
         step_no[0] += 1
@@ -153,7 +190,7 @@ def bench_lm(name, steps, warmup, cpu_tokens):
         loss = None
         for _ in range(c["accum"]):
             x, y = next(it)
-            loss = lm.micro_step(x, y, want_loss=want_loss)
+            loss = lm.micro_step(x, y, want_loss=True)    # train_llm.rs:450 reads every micro-batch's loss
         opt.step()
         return loss
 
@@ -167,22 +204,21 @@ def bench_lm(name, steps, warmup, cpu_tokens):
     elapsed = time.perf_counter() - t0
     # one more, instrumented step for the per-kernel numbers (not part of `value`)
     ctx.profile_start()
-    last_loss = one_step(want_loss=True)
+    last_loss = one_step()
     prof = ctx.profile_stop()
     tokens_per_step = c["accum"] * c["mb"] * c["seq"]
     value = steps * tokens_per_step / elapsed
-    dom, roofline = pick_dominant(prof, name)
-    roofline["kernel"] = dom
     step_flops = flops_per_token(c) * tokens_per_step
     out = dict(metric="train tokens/sec (fwd+bwd+AdamW)", value=round(value, 1), unit="tokens/s", n_gpus=1, steps=steps, warmup=warmup,
                ms_per_step=round(1e3 * elapsed / steps, 3), higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16",
                data="synthetic",
                config=dict(workload=c["label"], tokens_per_step=tokens_per_step, parallelism="single GPU",
-                           step_model_tflops=round(step_flops / 1e12, 2),
+                           step_model_tflops=round(step_flops / 1e12, 4),
                            mfma_frac_of_step=round(step_flops / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 4), last_loss=round(float(last_loss), 4)),
-               roofline=roofline, kernels=kernel_table(prof))
+               roofline=pick_dominant(prof, name), kernels=kernel_table(prof))
     ctx.close()
-    out["cpu_baseline"] = cpu_baseline_lm(c, cpu_tokens)
+    if with_cpu:
+        out["cpu_baseline"] = cpu_baseline_lm(c, c["seq"], 1 if name == "c5" else 8)
     return out
 
 
@@ -216,7 +252,8 @@ def bench_c3(steps, warmup):
     for _ in range(steps):
         step()
     prof = ctx.profile_stop()
-    bwd_ms = (prof["attn_bwd_dq_bf16"]["ms"] + prof["attn_bwd_dkv_bf16"]["ms"]) / steps
+    bwd_keys = [k_ for k_ in prof if k_.startswith("attn_bwd")]
+    bwd_ms = sum(prof[k_]["ms"] for k_ in bwd_keys) / steps
     bwd_flops = 4 * 2 * hd * (S * (S + 1) / 2) * B * Hq          # 34.39 GFLOP: four GEMMs, causal pairs, no recompute
     achieved = bwd_flops / (bwd_ms * 1e-3) / 1e12
     tokens = B * S
@@ -232,8 +269,9 @@ def bench_c3(steps, warmup):
                 vs_baseline=None, dtype="bf16", data="synthetic",
                 config=dict(workload="config3 causal GQA flash attention fwd+bwd, B8 S1024 Hq16 Hkv4 hd64, [B,H,S,hd]"),
                 roofline=dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                              frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC["c3"]["attn_bwd"],
-                              kernel="attn_bwd (dq + dkv kernels)"),
+                              frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC["c3"]["attn_bwd"], traffic_source=TRAFFIC_SOURCE["c3"],
+                              kernel="attn_bwd (" + " + ".join(sorted(bwd_keys)) + ")", bwd_us=round(1e3 * bwd_ms, 2),
+                              algorithmic_gflop=round(bwd_flops / 1e9, 2)),
                 kernels=kernel_table(prof),
                 cpu_baseline=dict(value=round(tokens / cpu_s, 2), unit="tokens/s", cores=1, kind="port",
                                   sample="oracle unfused attention chain fwd+bwd on 1 of 32 (batch, KV group) slices, scaled x32"))
@@ -266,8 +304,7 @@ def bench_c2(steps, warmup):
     for _ in range(steps):
         step()
     prof = ctx.profile_stop()
-    dom, roofline = pick_dominant(prof, "c2")
-    roofline["kernel"] = dom
+    roofline = pick_dominant(prof, "c2")
     ctx.close()
     R.set_threads(1)
     sample = 64
@@ -282,23 +319,31 @@ def bench_c2(steps, warmup):
                 cpu_baseline=dict(value=round(cpu_rows_s, 2), unit="rows/s", cores=1, kind="port", sample=f"oracle CE fwd+bwd on {sample} of 8192 rows"))
 
 
+def brief(r):
+    """The part of a workload's line that the combined line keeps."""
+    keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "dtype", "config", "roofline", "cpu_baseline")
+    return {k: r[k] for k in keep if k in r}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="c5", choices=["c5", "c4", "c3", "c2"])
-    ap.add_argument("--cpu-tokens", type=int, default=None, help="tokens in the CPU-baseline sample")
+    ap.add_argument("--workload", default="all", choices=["all", "c5", "c4", "c3", "c2"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
-    if args.workload in ("c5", "c4"):
-        steps = args.steps if args.steps is not None else (3 if args.workload == "c5" else 20)
-        warmup = args.warmup if args.warmup is not None else (1 if args.workload == "c5" else 3)
-        cpu_tokens = args.cpu_tokens or (16 if args.workload == "c5" else 256)
-        out = bench_lm(args.workload, steps, warmup, cpu_tokens)
-    elif args.workload == "c3":
+    w = args.workload
+    if w in ("all", "c5"):
+        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu)
+        if w == "all":
+            out["other_configs"] = dict(c4=brief(bench_lm("c4", 20, 3, not args.no_cpu)), c3=brief(bench_c3(20, 3)), c2=brief(bench_c2(20, 3)))
+    elif w == "c4":
+        out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu)
+    elif w == "c3":
         out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3)
     else:
         out = bench_c2(args.steps or 20, args.warmup if args.warmup is not None else 3)

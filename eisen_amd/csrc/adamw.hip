@@ -226,6 +226,9 @@ extern "C" int eisen_hip_adamw_step(eisen_ctx* ctx, const eisen_param_slot* slot
     int rc = upload_slots(ctx, slots, n_slots, true, &dev, &blocks, "adamw_step");
     if (rc) return rc;
     AdamParams p{lr, beta1, beta2, eps, weight_decay, bc1, bc2};
+    double bytes = 0.0;  // per parameter: w, g, m, v read, w, m, v written (28 B) and the bf16 copy written where there is one
+    for (size_t i = 0; i < n_slots; i++) bytes += (double)slots[i].n * (slots[i].w_bf16 ? 30.0 : 28.0);
+    EisenProfScope prof(ctx, "adamw", bytes);
     adamw_kernel<<<(unsigned)blocks, kThreads, 0, ctx->stream>>>(dev, (int)n_slots, p, grad_scale_device);
     EISEN_LAUNCH_CHECK(ctx, "adamw_kernel");
     return eisen_hip_free(ctx, dev);
@@ -256,6 +259,9 @@ extern "C" int eisen_hip_grad_norm(eisen_ctx* ctx, const eisen_param_slot* slots
         (void)eisen_hip_free(ctx, dev);
         return rc;
     }
+    double bytes = 0.0;
+    for (size_t i = 0; i < n_slots; i++) bytes += (double)slots[i].n * 4.0;
+    EisenProfScope prof(ctx, "grad_sumsq", bytes);
     sumsq_kernel<<<(unsigned)blocks, kThreads, 0, ctx->stream>>>(dev, (int)n_slots, (double*)ws);
     EISEN_LAUNCH_CHECK(ctx, "sumsq_kernel");
     norm_finish_kernel<<<1, 1024, 0, ctx->stream>>>((const double*)ws, blocks, max_norm, out_device);

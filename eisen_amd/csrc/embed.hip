@@ -100,6 +100,7 @@ extern "C" int eisen_hip_gather(eisen_ctx* ctx, const void* weight, const int32_
     const bool vec = hidden % n == 0 && eisen_aligned(weight, 16) && eisen_aligned(out, 16);
     const int cpr = (int)(vec ? hidden / n : hidden);
     const size_t chunks = n_ids * cpr;
+    EisenProfScope prof(ctx, dtype == EISEN_BF16 ? "gather_bf16" : "gather_f32", 2.0 * (double)n_ids * (double)hidden * eisen_dtype_size(dtype) + 4.0 * (double)n_ids);
     const unsigned blocks = (unsigned)std::min<size_t>(256 * 16, eisen_ceil_div(chunks, kThreads));
     if (dtype == EISEN_F32) {
         if (vec) gather_kernel<float, 4><<<blocks, kThreads, 0, ctx->stream>>>((const float*)weight, ids, (float*)out, chunks, cpr);
@@ -154,6 +155,9 @@ extern "C" int eisen_hip_gather_backward(eisen_ctx* ctx, const int32_t* ids_host
     const int32_t* d_begin = d_row + n_seg;
     const size_t n = dtype == EISEN_F32 ? 4 : 8;
     const bool vec = hidden % n == 0 && eisen_aligned(go, 16) && eisen_aligned(gw, 16);
+    // algorithmic bytes: every row of dOut read once, every touched row of the f32 gradient read and written once
+    EisenProfScope prof(ctx, dtype == EISEN_BF16 ? "scatter_rows_bf16" : "scatter_rows_f32",
+                        (double)n_ids * (double)hidden * eisen_dtype_size(dtype) + 8.0 * (double)n_seg * (double)hidden + 4.0 * (double)total);
     if (vec) {
         const int slabs = (int)eisen_ceil_div(hidden, (size_t)kWave * n);
         const size_t waves = n_seg * slabs;

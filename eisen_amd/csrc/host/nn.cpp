@@ -398,8 +398,18 @@ void lm_micro_step(Graph& g, const TransformerLM& lm, const float* ids, const in
     g.reinterpret_shape(logits, {mb * seq, lm.vocab_size});  // train_llm.rs:440 reshapes (a copy); the view is equivalent
     const std::vector<int64_t> t(targets, targets + mb * seq);
     const size_t loss = g.cross_entropy_masked(logits, t);
-    if (loss_out) *loss_out = g.sync_to_cpu(loss)[0];
-    g.backward(loss);
+    // the loss is read back every micro-batch (train_llm.rs:450); the copy is queued here and collected after the backward
+    // pass has been queued behind it, so the device never runs dry while the host waits
+    int ticket = -1;
+    if (loss_out) g.check(eisen_hip_dtoh_begin(g.ctx(), g.at(loss).data.ptr, sizeof(float), &ticket), "loss read-back");
+    try {
+        g.backward(loss);
+    } catch (...) {
+        float dropped;
+        if (ticket >= 0) (void)eisen_hip_dtoh_finish(g.ctx(), ticket, &dropped, sizeof(float));
+        throw;
+    }
+    if (loss_out) g.check(eisen_hip_dtoh_finish(g.ctx(), ticket, loss_out, sizeof(float)), "loss read-back");
     g.clear_activations();
 }
 

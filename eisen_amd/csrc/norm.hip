@@ -263,6 +263,8 @@ template <typename T>
 int rms_norm_fwd(eisen_ctx* ctx, const void* x, const float* w, void* out, float* rrms, size_t rows, size_t dim, float eps) {
     const unsigned blocks = (unsigned)eisen_ceil_div(rows, kRowWaves);
     const bool vec = dim % Pack<T>::N == 0 && eisen_aligned(x, 16) && eisen_aligned(out, 16) && eisen_aligned(w, 16);
+    // algorithmic bytes: x read, y written, one rrms per row
+    EisenProfScope prof(ctx, sizeof(T) == 2 ? "rms_norm_fwd_bf16" : "rms_norm_fwd_f32", 2.0 * (double)rows * (double)dim * sizeof(T) + 4.0 * (double)rows);
     if (vec)
         rms_norm_fwd_kernel<T, true><<<blocks, kRowThreads, 0, ctx->stream>>>((const T*)x, w, (T*)out, rrms, rows, (int)dim, eps);
     else
@@ -290,6 +292,9 @@ int rms_norm_bwd_partial(eisen_ctx* ctx, const void* x, const float* w, const fl
     constexpr int N = Pack<T>::N;
     const bool vec = dim % N == 0 && eisen_aligned(x, 16) && eisen_aligned(go, 16) && eisen_aligned(gx, 16) && eisen_aligned(w, 16) &&
                      dim <= (size_t)kWave * N * 8 && (size_t)kBwdWaves * dim * sizeof(float) <= 64 * 1024;
+    // algorithmic bytes: x and dy read, dx written (and read first when the call accumulates), one rrms per row
+    EisenProfScope prof(ctx, sizeof(T) == 2 ? "rms_norm_bwd_bf16" : "rms_norm_bwd_f32",
+                        (accumulate_x ? 4.0 : 3.0) * (double)rows * (double)dim * sizeof(T) + 4.0 * (double)rows);
     if (vec) {
         // enough waves to cover the chip a few times over, few enough that the partial rows stay small
         const unsigned blocks = (unsigned)std::min<size_t>(eisen_ceil_div(rows, kBwdWaves), kMaxPartialRows);
@@ -312,6 +317,9 @@ int rms_norm_bwd_partial(eisen_ctx* ctx, const void* x, const float* w, const fl
 }
 
 int rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim) {
+    double bytes = 0.0;
+    for (size_t i = 0; i < n; i++) bytes += ((double)nrows[i] + 2.0) * (double)dim * 4.0;
+    EisenProfScope prof(ctx, "rms_norm_dw_finish", bytes);
     for (size_t first = 0; first < n; first += kFinishSlots) {
         FinishSlots slots{};
         const size_t m = std::min<size_t>(kFinishSlots, n - first);

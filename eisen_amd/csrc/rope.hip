@@ -220,6 +220,8 @@ extern "C" int eisen_hip_rope_pair(eisen_ctx* ctx, const void* q, void* q_out, s
     const int rc = eisen_rope_table_get(ctx, seq, head_dim, &table);
     if (rc) return rc;
     const size_t n0 = batch * seq * hidden_q / n, n1 = batch * seq * hidden_k / n;
+    // algorithmic bytes: every element read once and written once
+    EisenProfScope prof(ctx, dtype == EISEN_BF16 ? "rope_pair_bf16" : "rope_pair_f32", 2.0 * (double)(n0 + n1) * 16.0);
     const unsigned blocks = (unsigned)std::min<size_t>(256 * 16, eisen_ceil_div(n0 + n1, kThreads));
     if (dtype == EISEN_F32)
         rope_pair_kernel<float><<<blocks, kThreads, 0, ctx->stream>>>((const float*)q, (float*)q_out, n0, (int)hidden_q, (const float*)k, (float*)k_out, n1,

@@ -52,6 +52,7 @@ struct eisen_ctx {
         size_t bytes = 0;
         hipEvent_t done = nullptr;
         bool in_flight = false;
+        bool reserved = false;  // holds the result of a device-to-host copy that eisen_hip_dtoh_finish has not collected yet
     };
     static constexpr int kStageSlots = 16;
     StageSlot stage[kStageSlots];

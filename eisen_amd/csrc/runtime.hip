@@ -224,6 +224,12 @@ int eisen_workspace(eisen_ctx* ctx, size_t bytes, void** out) {
 }
 
 int eisen_staging(eisen_ctx* ctx, size_t bytes, eisen_ctx::StageSlot** out) {
+    int tries = 0;
+    while (ctx->stage[ctx->stage_next].reserved && tries < eisen_ctx::kStageSlots) {
+        ctx->stage_next = (ctx->stage_next + 1) % eisen_ctx::kStageSlots;
+        tries++;
+    }
+    EISEN_REQUIRE(ctx, tries < eisen_ctx::kStageSlots, EISEN_E_STATE, "every staging slot holds an uncollected eisen_hip_dtoh_begin result");
     eisen_ctx::StageSlot& s = ctx->stage[ctx->stage_next];
     ctx->stage_next = (ctx->stage_next + 1) % eisen_ctx::kStageSlots;
     if (!s.done) EISEN_HIP_TRY(ctx, hipEventCreateWithFlags(&s.done, hipEventDisableTiming));
@@ -271,6 +277,38 @@ extern "C" int eisen_hip_dtoh(eisen_ctx* ctx, void* dst, const void* src, size_t
     if (bytes == 0) return 0;
     EISEN_HIP_TRY(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
     EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return 0;
+}
+
+extern "C" int eisen_hip_dtoh_begin(eisen_ctx* ctx, const void* src, size_t bytes, int* ticket_out) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, src && ticket_out, EISEN_E_ARG, "eisen_hip_dtoh_begin: null pointer");
+    EISEN_REQUIRE(ctx, bytes > 0 && bytes <= kStageLimit, EISEN_E_SHAPE, "eisen_hip_dtoh_begin: %zu bytes (1 .. %zu supported)", bytes, kStageLimit);
+    int reserved = 0;
+    for (const auto& sl : ctx->stage) reserved += sl.reserved ? 1 : 0;
+    EISEN_REQUIRE(ctx, reserved < eisen_ctx::kStageSlots / 2, EISEN_E_STATE, "eisen_hip_dtoh_begin: %d copies not collected yet", reserved);
+    eisen_ctx::StageSlot* st = nullptr;
+    int rc = eisen_staging(ctx, bytes, &st);
+    if (rc) return rc;
+    EISEN_HIP_TRY(ctx, hipMemcpyAsync(st->ptr, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    EISEN_HIP_TRY(ctx, hipEventRecord(st->done, ctx->stream));
+    st->in_flight = true;
+    st->reserved = true;
+    *ticket_out = (int)(st - ctx->stage);
+    return 0;
+}
+
+extern "C" int eisen_hip_dtoh_finish(eisen_ctx* ctx, int ticket, void* dst, size_t bytes) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, dst != nullptr, EISEN_E_ARG, "eisen_hip_dtoh_finish: null pointer");
+    EISEN_REQUIRE(ctx, ticket >= 0 && ticket < eisen_ctx::kStageSlots && ctx->stage[ticket].reserved, EISEN_E_STATE,
+                  "eisen_hip_dtoh_finish: ticket %d names no pending copy", ticket);
+    eisen_ctx::StageSlot& s = ctx->stage[ticket];
+    EISEN_REQUIRE(ctx, bytes <= s.bytes, EISEN_E_ARG, "eisen_hip_dtoh_finish: %zu bytes asked of a %zu-byte slot", bytes, s.bytes);
+    s.reserved = false;
+    EISEN_HIP_TRY(ctx, hipEventSynchronize(s.done));  // waits for this copy only: later work stays queued
+    s.in_flight = false;
+    memcpy(dst, s.ptr, bytes);
     return 0;
 }
 

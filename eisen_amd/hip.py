@@ -125,6 +125,17 @@ class Context:
             self._call("eisen_hip_dtoh", out.ctypes.data_as(_vp), _ptr(buf), _sz(out.nbytes))
         return bf16_bits_to_f32(out).reshape(shape) if dtype == BF16 else out
 
+    def dtoh_begin(self, buf, nbytes):
+        """Queue a device-to-host copy; returns a ticket for dtoh_finish."""
+        t = C.c_int(-1)
+        self._call("eisen_hip_dtoh_begin", _ptr(buf), _sz(nbytes), C.byref(t))
+        return t.value
+
+    def dtoh_finish(self, ticket, shape, dtype=np.float32):
+        out = np.empty(shape, dtype)
+        self._call("eisen_hip_dtoh_finish", _i(ticket), out.ctypes.data_as(_vp), _sz(out.nbytes))
+        return out
+
     def sync(self):
         self._call("eisen_hip_stream_sync")
 

@@ -85,6 +85,12 @@ int eisen_hip_pool_stats(eisen_ctx* ctx, size_t* in_use_bytes, size_t* cached_by
 int eisen_hip_htod(eisen_ctx* ctx, void* dst_device, const void* src_host, size_t bytes);
 /* stream.clone_dtoh (src/tensor.rs:177-223): synchronises the stream before returning. */
 int eisen_hip_dtoh(eisen_ctx* ctx, void* dst_host, const void* src_device, size_t bytes);
+/* clone_dtoh in two halves, for a value the host wants without draining the stream (the loss of a micro-batch,
+ * examples/train_llm.rs:450, read while the backward pass is already queued): `begin` enqueues the copy into pinned
+ * memory of the library and returns a ticket, `finish` waits for that copy alone and fills dst_host.  At most 8 tickets
+ * may be outstanding; bytes <= 8 MiB. */
+int eisen_hip_dtoh_begin(eisen_ctx* ctx, const void* src_device, size_t bytes, int* ticket_out);
+int eisen_hip_dtoh_finish(eisen_ctx* ctx, int ticket, void* dst_host, size_t bytes);
 int eisen_hip_dtod(eisen_ctx* ctx, void* dst_device, const void* src_device, size_t bytes);
 int eisen_hip_memset_zero(eisen_ctx* ctx, void* dst_device, size_t bytes);
 

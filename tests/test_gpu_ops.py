@@ -55,6 +55,19 @@ def test_runtime_roundtrip_pool_and_errors(ctx):
     ctx.timer_start()
     ms = ctx.timer_stop()
     assert ms >= 0.0
+    # the two-phase read-back: copies queued, uploads and kernels issued behind them, results collected out of order
+    vals = [gen.normal(10 + i, (256,)) for i in range(3)]
+    bufs = [ctx.upload(v) for v in vals]
+    tickets = [ctx.dtoh_begin(bf, 1024) for bf in bufs]
+    for bf in bufs:
+        ctx.fill(bf, F32, 7.0, 256)                            # later work on the stream must not reach the copies
+    other = [ctx.upload(gen.normal(20 + i, (64,))) for i in range(20)]   # more uploads than staging slots
+    for i in (2, 0, 1):
+        assert np.array_equal(ctx.dtoh_finish(tickets[i], (256,)), vals[i])
+    with pytest.raises(hip.EisenHipError):
+        ctx.dtoh_finish(tickets[0], (256,))                    # already collected
+    for bf in bufs + other:
+        bf.free()
 
 
 def test_module_load_and_launch_by_name(ctx):
