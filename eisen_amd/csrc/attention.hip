@@ -22,179 +22,18 @@
 //     every query head of the group and every visible query tile; Q/dO tiles go through LDS.
 //     No atomics anywhere: dQ has its own query-stationary pass, so results are reproducible.
 // f32 path (any head_dim): one wave per query row / key row, plain FMA, for small shapes.
-#include <type_traits>
-
-#include "device_utils.cuh"
-#include "runtime.h"
+#include "attention_common.cuh"
 
 namespace {
 
-struct AttnArgs {
-    const void *Q, *K, *V, *O, *dO;
-    void *Out, *dQ, *dK, *dV;
-    float *LSE, *D;
-    int B, S, Hq, Hkv, G, hd;
-    long long q_sb, q_ss, q_sh;
-    long long k_sb, k_ss, k_sh;
-    float scale, scale_log2e;
-    int causal;
-    int paired;  // query-stationary kernels: a block runs a long query block and its short mirror image
-    // backward only: when set ([S][hd/2] cos/sin), Q and K are rotary-embedded projections and dQ, dK are the
-    // gradients of the projections before the rotation (the inverse rotation is applied as the gradients are stored)
-    const float2* rope;
-};
-
-// Scratch of eisen_hip_attention_backward_noalloc: D = rowsum(dO o O), one float per (batch, query head, position).
-// A file-scope device array instead of a workspace allocation, so that entry point never calls an allocator.  Every
-// GPU the library runs on holds its own 4 MiB copy until the process ends; the name below is only a host-side handle,
-// the device address of each GPU's copy comes from hipGetSymbolAddress (eisen_attention_scratch_init).
+// Scratch of eisen_hip_attention_backward_noalloc: D = rowsum(dO o O) and LSE * log2(e), two floats per (batch, query
+// head, position).  A file-scope device array instead of a workspace allocation, so that entry point never calls an
+// allocator.  Every GPU the library runs on holds its own 8 MiB copy until the process ends; the name below is only a
+// host-side handle, the device address of each GPU's copy comes from hipGetSymbolAddress (eisen_attention_scratch_init).
 constexpr size_t kNoAllocMaxRows = size_t(1) << 20;
-static __device__ __align__(256) float g_attn_bwd_scratch[kNoAllocMaxRows];
+static __device__ __align__(256) float g_attn_bwd_scratch[2 * kNoAllocMaxRows];
 constexpr int kMaxDevices = 64;
 static float* g_attn_bwd_scratch_ptr[kMaxDevices] = {nullptr};  // per device, filled once
-
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
-
-typedef bf16x4 __attribute__((address_space(3))) * lds_bf16x4_ptr;
-
-// 4 consecutive rows of a column out of a row-major LDS tile: within each group of 16 lanes,
-// lane i receives rows r0..r0+3 of column c0+i when lane L passes &tile[r0 + L/4][c0 + 4*(L%4)].
-__device__ __forceinline__ bf16x4 lds_read_tr(const bf16_t* p) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p));
-}
-__device__ __forceinline__ bf16x8 concat4(bf16x4 lo, bf16x4 hi) {
-    bf16x8 r;
-    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
-    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
-    return r;
-}
-// Row index inside a 32x32 MFMA accumulator tile held by register v of a lane in half g.
-__device__ __forceinline__ int acc_row(int v, int g) { return 8 * (v >> 2) + 4 * g + (v & 3); }
-
-// Backward of the rotary embedding on NP interleaved pairs: dx0 = g0 c + g1 s, dx1 = -g0 s + g1 c
-// (src/graph/ops/transform.rs:592-595); cs points at the (cos, sin) of the first pair.
-template <int NP>
-__device__ __forceinline__ void unrotate_pairs(float* x, const float2* cs) {
-#pragma unroll
-    for (int j = 0; j < NP; j++) {
-        const float2 t = cs[j];
-        const float g0 = x[2 * j], g1 = x[2 * j + 1];
-        x[2 * j] = g0 * t.x + g1 * t.y;
-        x[2 * j + 1] = -g0 * t.y + g1 * t.x;
-    }
-}
-
-// K-operand (8 values along the contraction) for contraction step t of a [32-row k-dim] x
-// [32-col] block of a row-major LDS tile, in the order the accumulator registers 8t..8t+7 use.
-__device__ __forceinline__ bf16x8 lds_tr_operand(const bf16_t* tile, int pitch, int row0, int col0, int t, int lane) {
-    const int g = lane >> 5, L = lane & 15, half = (lane >> 4) & 1;
-    const bf16_t* p = tile + (row0 + 16 * t + 4 * g + (L >> 2)) * pitch + col0 + 16 * half + 4 * (L & 3);
-    return concat4(lds_read_tr(p), lds_read_tr(p + 8 * pitch));
-}
-
-// Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  This
-// renumbering gives XCD j the contiguous id range [j*total/8, (j+1)*total/8), in dispatch order, so
-// workgroups that are neighbours in the renumbered order (and share operands) also share an L2.
-__device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
-    const int per = total / 8;
-    return linear < per * 8 ? (linear % 8) * per + linear / 8 : linear;
-}
-
-// 2^x as the bare hardware instruction: results below 2^-126 flush to zero, which is what a softmax
-// weight that small should be; the library exp2f spends four more instructions per value on them.
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// A ROWS x HD bf16 tile on its way from a strided global tensor into LDS, held in registers in
-// between so the global loads of tile i+1 are in flight while tile i is being used.
-template <int HD, int ROWS, int THREADS>
-struct TilePrefetch {
-    static constexpr int PITCH = HD + 8, CPR = HD / 8, TOTAL = ROWS * CPR;
-    static constexpr int CH = (TOTAL + THREADS - 1) / THREADS;
-    bf16x8 r[CH];
-    __device__ __forceinline__ void fetch(const bf16_t* src, long long row_stride, int first_row, int limit_rows) {
-        const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (first_row + ROWS <= limit_rows) {  // whole tile in range (uniform): plain loads, no selects
-#pragma unroll
-            for (int i = 0; i < CH; i++) {
-                const int c = i * THREADS + threadIdx.x;
-                if (TOTAL % THREADS == 0 || c < TOTAL)
-                    r[i] = *reinterpret_cast<const bf16x8*>(src + (long long)(first_row + c / CPR) * row_stride + (c % CPR) * 8);
-            }
-            return;
-        }
-#pragma unroll
-        for (int i = 0; i < CH; i++) {
-            const int c = i * THREADS + threadIdx.x;
-            const int row = c / CPR, cc = c % CPR, gr = first_row + row;
-            r[i] = (c < TOTAL && gr < limit_rows) ? *reinterpret_cast<const bf16x8*>(src + (long long)gr * row_stride + cc * 8) : zero8;
-        }
-    }
-    __device__ __forceinline__ void commit(bf16_t* dst) const {
-#pragma unroll
-        for (int i = 0; i < CH; i++) {
-            const int c = i * THREADS + threadIdx.x;
-            if (c < TOTAL) *reinterpret_cast<bf16x8*>(dst + (c / CPR) * PITCH + (c % CPR) * 8) = r[i];
-        }
-    }
-};
-
-// ---- tiles loaded straight into LDS ----------------------------------------------------------
-// Unpadded rows of HD bf16 with permuted chunks (lds_swz in device_utils.cuh).
-template <int HD>
-__device__ __forceinline__ int tile_swz(int row) { return lds_swz<HD * 2>(row); }
-template <int HD>
-__device__ __forceinline__ int tile_at(int row, int col) {
-    return row * HD + ((((col >> 3) ^ tile_swz<HD>(row)) << 3) | (col & 7));
-}
-// lds_tr_operand for a swizzled tile
-template <int HD>
-__device__ __forceinline__ bf16x8 lds_tr_operand_swz(const bf16_t* tile, int row0, int col0, int t, int lane) {
-    const int g = lane >> 5, L = lane & 15, half = (lane >> 4) & 1;
-    const int row = row0 + 16 * t + 4 * g + (L >> 2), col = col0 + 16 * half + 4 * (L & 3);
-    return concat4(lds_read_tr(tile + tile_at<HD>(row, col)), lds_read_tr(tile + tile_at<HD>(row + 8, col)));
-}
-
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-typedef __attribute__((address_space(1))) const void* global_void_ptr;
-
-// A ROWS x HD bf16 tile of a strided global tensor, loaded into a swizzled LDS tile by WAVES waves with
-// no registers in between.  Each wave instruction moves 1 KB (512 / HD rows).  Rows past `limit_rows`
-// re-read the last valid row: the kernels mask or zero-weight them, they only have to be finite.
-// The loads are asynchronous: wait_direct_loads() before the barrier that publishes the tile.
-template <int HD, int ROWS, int WAVES>
-struct DirectTile {
-    static constexpr int CPR = HD / 8, RPB = 64 / CPR, BLOCKS = ROWS / RPB, PER_WAVE = BLOCKS / WAVES;
-    static_assert(ROWS % RPB == 0 && BLOCKS % WAVES == 0, "tile does not split into whole wave loads");
-    unsigned off[PER_WAVE];  // byte offset of this lane's chunk from the tile's first row (loop-invariant)
-    __device__ __forceinline__ static int lane_row(int wave, int i, int lane) { return (wave * PER_WAVE + i) * RPB + lane / CPR; }
-    __device__ __forceinline__ static int lane_chunk(int row, int lane) { return (lane % CPR) ^ tile_swz<HD>(row); }
-    __device__ __forceinline__ void init(long long row_stride, int wave, int lane) {
-#pragma unroll
-        for (int i = 0; i < PER_WAVE; i++) {
-            const int row = lane_row(wave, i, lane);
-            off[i] = (unsigned)((row * row_stride + lane_chunk(row, lane) * 8) * 2);
-        }
-    }
-    __device__ __forceinline__ void load(const bf16_t* src, long long row_stride, int first_row, int limit_rows, bf16_t* lds_tile,
-                                         int wave, int lane) const {
-        if (first_row + ROWS <= limit_rows) {  // whole tile in range (uniform)
-            const char* base = reinterpret_cast<const char*>(src + (long long)first_row * row_stride);
-#pragma unroll
-            for (int i = 0; i < PER_WAVE; i++)
-                __builtin_amdgcn_global_load_lds((global_void_ptr)(base + off[i]), (lds_void_ptr)(lds_tile + (wave * PER_WAVE + i) * 512), 16, 0, 0);
-            return;
-        }
-#pragma unroll
-        for (int i = 0; i < PER_WAVE; i++) {
-            const int row = lane_row(wave, i, lane);
-            const int gr = min(first_row + row, limit_rows - 1);
-            __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (long long)gr * row_stride + lane_chunk(row, lane) * 8),
-                                             (lds_void_ptr)(lds_tile + (wave * PER_WAVE + i) * 512), 16, 0, 0);
-        }
-    }
-};
-__device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // ---- forward -------------------------------------------------------------------------------
 // Grid of the two query-stationary kernels: one block per (pair of query blocks, GW query heads of a
@@ -400,8 +239,11 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
         }
         const float Dq = dpart + __shfl_xor(dpart, 32, 64);
         const long long stat = ((long long)b * a.Hq + hq) * a.S + q;
-        if (valid_q && g == 0) a.D[stat] = Dq;
         const float lse2 = valid_q ? a.LSE[stat] * kLog2e : INFINITY;
+        if (valid_q && g == 0) {
+            a.D[stat] = Dq;
+            a.L2[stat] = -a.LSE[stat] / a.scale;  // start value of the dK / dV kernel's score accumulators
+        }
 
         f32x16 dq[DT];
 #pragma unroll
@@ -860,7 +702,8 @@ void launch_bwd(eisen_ctx* ctx, AttnArgs a) {
     dim3 grid2((unsigned)((n_kb + 1) / 2 * a.Hkv * a.B));
     {   // dP, dV, dK: three of the four backward GEMMs
         EisenProfScope prof(ctx, "attn_bwd_dkv_bf16", 3.0 * attn_pair_flops(a), true);
-        fa_bwd_dkv_kernel<HD><<<grid2, 256, 0, ctx->stream>>>(a);
+        if (HD <= 64 && eisen_attention_dkv32_supports(a)) eisen_attention_launch_dkv32(ctx, a);
+        else fa_bwd_dkv_kernel<HD><<<grid2, 256, 0, ctx->stream>>>(a);
     }
 }
 
@@ -921,10 +764,11 @@ static int attention_backward_common(eisen_ctx* ctx, const void* q, const void* 
         a.D = scratch;
     } else {
         void* ws = nullptr;
-        rc = eisen_workspace(ctx, B * Hq * S * sizeof(float), &ws);
+        rc = eisen_workspace(ctx, 2 * B * Hq * S * sizeof(float), &ws);
         if (rc) return rc;
         a.D = static_cast<float*>(ws);
     }
+    a.L2 = a.D + B * Hq * S;
     if (rope) {
         rc = eisen_rope_table_get(ctx, S, hd, &a.rope);
         if (rc) return rc;

@@ -1,0 +1,255 @@
+// Flash-attention backward, the key-stationary pass: dK and dV (head_dim 32 and 64, bf16 MFMA).
+//
+//   dV = P^T dO,  dK = scale dS^T Q,  dS = P o (dO V^T - D),  P = exp2(log2e (scale Q K^T - LSE))
+// summed over the query heads of a KV group (the repeat_kv backward, src/graph/ops/gqa.rs:168-184) and over every
+// query that sees the key (the bmm backward of the reference's chain, src/graph/ops/linear.rs:1482-1498, and the
+// softmax backward, src/graph/ops/reduction.rs:504-512).  The reference has no such kernel; what it must equal is
+// that chain.
+//
+// Shape of the kernel
+//   * A workgroup owns the keys of two 32-key blocks of one KV head, a heavy one and its light mirror image under the
+//     causal mask (equal work everywhere).  Its four waves each take every fourth (query head of the group, 32-query
+//     tile) item; their partial dK / dV meet in LDS once per key block, in wave order (no atomics).
+//   * A wave issues in order and its MFMAs and vector ALU work do not overlap each other; they overlap with those of
+//     the other wave on the SIMD.  So a wave must fit 256 registers (two per SIMD) and should spend as few cycles as
+//     possible on anything but MFMAs and the softmax:
+//       - every MFMA takes its accumulator in ordinary VGPRs (the file is compiled that way): with the AGPR form the
+//         compiler copies the score accumulators between the register files around the softmax of every tile;
+//       - Q / dO tiles and the two per-query statistics go from global memory straight into a private two-stage LDS
+//         ring of the wave (global_load_lds with a scalar base: no staging registers, no LDS stores, no address
+//         arithmetic in vector registers, no barrier in the loop);
+//       - the score accumulator starts at -LSE / scale and the dP accumulator at D (read from the ring straight into
+//         the accumulator registers), and the sign of V is flipped once per key block, so the MFMA chains deliver
+//         S - LSE / scale and D - dP: a probability is one multiply and one exp2, -dS one more multiply; -scale is
+//         applied when dK is stored.
+#include "attention_common.cuh"
+
+namespace {
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// One wave instruction of a direct-to-LDS load with a wave-uniform 64-bit base and a 32-bit byte offset per lane: lane l's
+// SIZE bytes land at lds_dst + SIZE * l.  Two scalar instructions and the load; no address arithmetic in vector registers.
+__device__ __forceinline__ void load_lds_16(const void* base, unsigned lane_offset, const void* lds_dst) {
+    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void load_lds_4(const void* base, unsigned lane_offset, const void* lds_dst) {
+    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
+}
+
+__device__ __forceinline__ void mfma(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+}
+
+template <int HD>
+__global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
+    constexpr int KSTEPS = HD / 16, DT = HD / 32, NST = 2;
+    constexpr int TILE = 32 * HD;                        // elements of a Q or dO tile
+    constexpr int STAGE_BYTES = 2 * TILE * 2 + 256;      // Q tile, dO tile, 32 x (-LSE / scale | D)
+    using Loader = DirectTile<HD, 32, 1>;
+    constexpr int LOADS = 2 * Loader::PER_WAVE + 1;      // load instructions per tile
+    static_assert(LOADS <= 63, "the tile in flight must fit the vmcnt counter");
+    static_assert(4 * 32 * HD * sizeof(float) <= 4 * NST * STAGE_BYTES, "the reduction reuses the rings");
+    __shared__ __attribute__((aligned(1024))) char lds[4 * NST * STAGE_BYTES];
+
+    const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_qt = (a.S + 31) / 32, n_pairs = (n_qt + 1) / 2;
+    // grid: x = key-block pair, fastest; then KV head, then batch.  Blocks of one (batch, KV head) read the same
+    // Q / dO tiles, so they are kept on one XCD.
+    const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int pair = bid % n_pairs, kvh = (bid / n_pairs) % a.Hkv, b = bid / (n_pairs * a.Hkv);
+    char* ring = lds + wave * (NST * STAGE_BYTES);
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    // lanes 0-31 fetch the tile's -LSE / scale, lanes 32-63 its D: byte offset of the lane's value from D's entry for the
+    // tile's first query (the launcher has checked that the statistics are less than 2 GiB apart)
+    const unsigned stat_off = (unsigned)(g == 0 ? (a.L2 - a.D) * 4 : 0) + 4 * (unsigned)c;
+    Loader loader;
+    loader.init(a.q_ss, 0, lane);
+
+    for (int pass = 0; pass < 2; pass++) {
+        const int kb = pass == 0 ? pair : n_qt - 1 - pair;
+        if (pass == 1 && kb <= pair) break;  // odd block count: the middle block has no mirror
+        const int k0 = kb * 32, key = k0 + c;
+        bf16x8 kf[KSTEPS], vn[KSTEPS];  // K and -V of the 32 keys, MFMA B operands
+        {
+            const long long koff = b * a.k_sb + kvh * a.k_sh + (long long)key * a.k_ss;
+#pragma unroll
+            for (int st = 0; st < KSTEPS; st++) {
+                const int d = st * 16 + 8 * g;
+                kf[st] = key < a.S ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.K) + koff + d) : zero8;
+                vn[st] = key < a.S ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.V) + koff + d) : zero8;
+                typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+                u32x4 bits = __builtin_bit_cast(u32x4, vn[st]) ^ 0x80008000u;  // sign flip of the eight bf16 values
+                vn[st] = __builtin_bit_cast(bf16x8, bits);
+                // the flip is done here, once, not again at every use; and both operands have arrived before the loop (a
+                // pending load of theirs would make the compiler wait for every outstanding load at their first use in it,
+                // the prefetched tile's included)
+                asm volatile("" : "+v"(vn[st]), "+v"(kf[st]));
+            }
+        }
+        f32x16 dk[DT], dv[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) { dk[dt][v] = 0.f; dv[dt][v] = 0.f; }
+
+        const int qt_start = a.causal ? kb : 0;  // the diagonal tile is the first one that sees these keys
+        const int per_head = n_qt - qt_start;
+        const int n_items = a.G * per_head;       // (query head of the group, query tile), head-major
+        const int n_mine = n_items > wave ? (n_items - wave + 3) / 4 : 0;
+
+        auto stage_of = [&](int i) { return ring + (i % NST) * STAGE_BYTES; };
+        auto issue = [&](int i) {  // the loads of this wave's i-th tile into ring stage i % NST
+            const int item = wave + 4 * i;
+            const int hq = kvh * a.G + item / per_head, q0 = (qt_start + item % per_head) * 32;
+            char* stage = stage_of(i);
+            const long long tile0 = b * a.q_sb + hq * a.q_sh + (long long)q0 * a.q_ss;  // wave-uniform
+            const char* qbase = reinterpret_cast<const char*>(static_cast<const bf16_t*>(a.Q) + tile0);
+            const char* dobase = reinterpret_cast<const char*>(static_cast<const bf16_t*>(a.dO) + tile0);
+            const char* sbase = reinterpret_cast<const char*>(a.D + ((long long)b * a.Hq + hq) * a.S + q0);
+            if (q0 + 32 <= a.S) {
+#pragma unroll
+                for (int r = 0; r < Loader::PER_WAVE; r++) {
+                    load_lds_16(qbase, loader.off[r], stage + r * 1024);
+                    load_lds_16(dobase, loader.off[r], stage + TILE * 2 + r * 1024);
+                }
+                load_lds_4(sbase, stat_off, stage + 2 * TILE * 2);
+            } else {  // ragged last tile: rows past the end re-read the last row (they are given zero weight)
+#pragma unroll
+                for (int r = 0; r < Loader::PER_WAVE; r++) {
+                    const int row = Loader::lane_row(0, r, lane), gr = min(row, a.S - 1 - q0);
+                    const unsigned off = (unsigned)((gr * a.q_ss + Loader::lane_chunk(row, lane) * 8) * 2);
+                    load_lds_16(qbase, off, stage + r * 1024);
+                    load_lds_16(dobase, off, stage + TILE * 2 + r * 1024);
+                }
+                load_lds_4(sbase, stat_off - 4 * (unsigned)(c - min(c, a.S - 1 - q0)), stage + 2 * TILE * 2);
+            }
+        };
+
+        if (n_mine > 0) issue(0);
+        for (int i = 0; i < n_mine; i++) {
+            // the other stage was read by tile i - 1, whose operand reads have all returned (its MFMAs were issued)
+            if (i + 1 < n_mine) {
+                issue(i + 1);
+                wait_vmcnt<LOADS>();
+            } else {
+                wait_vmcnt<0>();
+            }
+            const int item = wave + 4 * i;
+            const int q0 = (qt_start + item % per_head) * 32;
+            const bf16_t* Qs = reinterpret_cast<const bf16_t*>(stage_of(i));
+            const bf16_t* dOs = Qs + TILE;
+            float* st = reinterpret_cast<float*>(stage_of(i) + 2 * TILE * 2);
+            if (q0 + 32 > a.S) {  // a query past the end gets LSE = +inf (stored negated): its probabilities are exactly zero
+                if (g == 0 && q0 + c >= a.S) st[c] = -INFINITY;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            }
+            // scores: S - LSE / scale and D - dP, the start values read straight into the accumulator registers
+            f32x16 s, dp;
+#pragma unroll
+            for (int vg = 0; vg < 4; vg++) {
+                const float4 l4 = *reinterpret_cast<const float4*>(st + 8 * vg + 4 * g);
+                const float4 d4 = *reinterpret_cast<const float4*>(st + 32 + 8 * vg + 4 * g);
+                s[4 * vg] = l4.x; s[4 * vg + 1] = l4.y; s[4 * vg + 2] = l4.z; s[4 * vg + 3] = l4.w;
+                dp[4 * vg] = d4.x; dp[4 * vg + 1] = d4.y; dp[4 * vg + 2] = d4.z; dp[4 * vg + 3] = d4.w;
+            }
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ks++) {
+                const bf16x8 qa = *reinterpret_cast<const bf16x8*>(Qs + tile_at<HD>(c, ks * 16 + 8 * g));
+                const bf16x8 da = *reinterpret_cast<const bf16x8*>(dOs + tile_at<HD>(c, ks * 16 + 8 * g));
+                mfma(s, qa, kf[ks]);
+                mfma(dp, da, vn[ks]);
+            }
+            // the transposed operands of the accumulation, requested before the softmax so that they arrive under it
+            bf16x8 dotr[DT][2], qtr[DT][2];
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    dotr[dt][t] = lds_tr_operand_swz<HD>(dOs, 0, dt * 32, t, lane);
+                    qtr[dt][t] = lds_tr_operand_swz<HD>(Qs, 0, dt * 32, t, lane);
+                }
+            float p[16];
+#pragma unroll
+            for (int v = 0; v < 16; v++) p[v] = fast_exp2(s[v] * a.scale_log2e);
+            // only the diagonal tile is cut by the causal mask
+            if (a.causal && q0 == k0) {
+                asm volatile("" ::: "memory");  // keeps this a branch taken once per head, not 16 selects per tile
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    if (c > acc_row(v, g)) p[v] = 0.f;  // key k0 + c is after query q0 + row
+            }
+            bf16x8 pf[2], dsf[2];
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                pf[v >> 3][v & 7] = (bf16_t)p[v];
+                dsf[v >> 3][v & 7] = (bf16_t)(p[v] * dp[v]);  // = -dS: dp holds D - dP
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    mfma(dv[dt], pf[t], dotr[dt][t]);
+                    mfma(dk[dt], dsf[t], qtr[dt][t]);
+                }
+        }
+
+        // Sum the four waves' partial results through the (now idle) rings, dK then dV, and store.
+        float* red = reinterpret_cast<float*>(lds);  // [wave][32 keys][HD]
+        bf16_t* outs[2] = {static_cast<bf16_t*>(a.dK) + b * a.k_sb + kvh * a.k_sh, static_cast<bf16_t*>(a.dV) + b * a.k_sb + kvh * a.k_sh};
+#pragma unroll
+        for (int which = 0; which < 2; which++) {
+            __syncthreads();  // every wave is done with its ring / with the previous reduction
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    red[(wave * 32 + acc_row(v, g)) * HD + dt * 32 + c] = which == 0 ? dk[dt][v] * -a.scale : dv[dt][v];
+            __syncthreads();
+            for (int e0 = threadIdx.x * 8; e0 < 32 * HD; e0 += 256 * 8) {
+                float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const float* src = red + w * 32 * HD + e0;
+                    const float4 x0 = *reinterpret_cast<const float4*>(src);
+                    const float4 x1 = *reinterpret_cast<const float4*>(src + 4);
+                    acc8[0] += x0.x; acc8[1] += x0.y; acc8[2] += x0.z; acc8[3] += x0.w;
+                    acc8[4] += x1.x; acc8[5] += x1.y; acc8[6] += x1.z; acc8[7] += x1.w;
+                }
+                const int kr = k0 + e0 / HD;
+                if (kr < a.S) {
+                    if (which == 0 && a.rope) unrotate_pairs<4>(acc8, a.rope + (size_t)kr * (HD / 2) + (e0 % HD) / 2);
+                    bf16x8 o8;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) o8[e] = (bf16_t)acc8[e];
+                    *reinterpret_cast<bf16x8*>(outs[which] + (long long)kr * a.k_ss + e0 % HD) = o8;
+                }
+            }
+        }
+        __syncthreads();  // the reduction's reads are over before the next pass refills the rings
+    }
+}
+
+}  // namespace
+
+// What the kernel above covers: head_dim 32 and 64, and shapes whose byte offsets inside a tile (31 rows of the query
+// stride) and between the two statistics arrays fit 32 bits.
+bool eisen_attention_dkv32_supports(const AttnArgs& a) {
+    return (a.hd == 32 || a.hd == 64) && a.q_ss > 0 && a.q_ss * 32 * 2 < (1ll << 31) && a.L2 > a.D && (a.L2 - a.D) * 4 < (1ll << 31);
+}
+
+// a.L2 (-LSE / scale) and a.D must have been written (by the dQ kernel).
+void eisen_attention_launch_dkv32(eisen_ctx* ctx, const AttnArgs& a) {
+    const int n_kb = (a.S + 31) / 32;  // 32-key blocks, handled in heavy / light pairs
+    dim3 grid((unsigned)((n_kb + 1) / 2 * a.Hkv * a.B));
+    if (a.hd == 64) fa_bwd_dkv32_kernel<64><<<grid, 256, 0, ctx->stream>>>(a);
+    else fa_bwd_dkv32_kernel<32><<<grid, 256, 0, ctx->stream>>>(a);
+}

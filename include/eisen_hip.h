@@ -301,8 +301,8 @@ int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const void* k, c
 
 /* eisen_hip_attention_backward for callers that cannot allocate (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and the same
- * results; the one buffer the kernels need beyond the inputs and outputs, D = rowsum(dO o O) with one float per
- * (batch, query head, position), lives in a fixed 4 MiB device array of the library instead of the context's growing
+ * results; the scratch the kernels need beyond the inputs and outputs, D = rowsum(dO o O) and -LSE/scale with one float
+ * each per (batch, query head, position), lives in a fixed 8 MiB device array of the library instead of the context's growing
  * workspace, so the call reaches no hipMalloc / hipFree / pool routine.  Limit: B * Hq * S <= 1,048,576, larger
  * shapes return EISEN_E_SHAPE.  Every call on one GPU uses that GPU's one array: calls that overlap on a GPU (two
  * contexts, two streams) race; calls on one context are ordered by its stream.  Nothing in the array has to be
