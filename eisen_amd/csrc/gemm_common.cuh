@@ -1,0 +1,246 @@
+// Pieces shared by the GEMM kernels of gemm.hip and gemm_wide.hip: the launch argument block, the operand tiles
+// filled by direct-to-LDS loads, and the epilogue that stores a wave's accumulators.
+#pragma once
+#include <utility>
+
+#include "device_utils.cuh"
+#include "runtime.h"
+
+constexpr int kMaxGroup = 8;  // products of one grouped launch
+struct GemmArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int M, N, K;
+    int lda, ldb, ldc;                 // leading dimensions in elements
+    long long sA, sB, sC;              // batch strides in elements
+    int accumulate;
+    const void* R;                     // optional residual with C's layout: C = R + A*B (accumulate must be 0)
+    int split;                         // > 1: K is cut into this many parts; part p > 0 assigns into partial[p-1]
+    int k_part;                        // contraction length of one part (a multiple of the slab)
+    float* partial;                    // [batch][split-1][M][N] f32, summed into C by a second kernel
+    // SwiGLU-backward epilogue (gate != nullptr): the product is dH, the gradient of h = silu(gate) * up; C receives
+    // dgate = dH * up * silu'(gate) and C2 receives dup = dH * silu(gate) (all with C's layout, no accumulation, no split-K)
+    const void* gate;
+    const void* up;
+    void* C2;
+    // Grouped launch (direct kernel, ngroup > 0): blockIdx.x enumerates the tiles of up to kMaxGroup products that share M, K
+    // and the operand orders but have their own A, B, C and N; grp_tile_end[p] = number of tiles of products 0..p
+    int ngroup;
+    const void* grp_A[kMaxGroup];
+    const void* grp_B[kMaxGroup];
+    void* grp_C[kMaxGroup];
+    int grp_N[kMaxGroup];
+    int grp_tile_end[kMaxGroup];
+    int tile_group;                    // direct kernel: > 0 = N tiles per group of the tile order (see the kernel), 0 = row-major order
+    int vec_c;                         // C rows are 16-byte aligned at every 8th column: the epilogue may use 16-byte accesses
+    // K made of up to three segments with their own operands, C (+)= sum_s op(A_s) op(B_s): segment 0 is A/B/lda/ldb,
+    // seg_end[s] is the contraction offset at which segment s ends (multiples of 64); nseg <= 1 means plain
+    int nseg;
+    const void* A_seg[2];
+    const void* B_seg[2];
+    int lda_seg[2], ldb_seg[2];
+    int seg_end[2];
+};
+
+// gemm_wide.hip: 256 x 256 tiles, four waves of 128 x 128 (plain products, whole tiles only)
+bool eisen_gemm_wide_supports(const GemmArgs& g, bool a_kc, bool b_kc, int batch, int dtype_c);
+void eisen_gemm_launch_wide(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int dtype_c);
+
+namespace {
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a constant expression
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+
+typedef bf16x4 __attribute__((address_space(3))) * lds_bf16x4_ptr;
+
+// d(silu(gate) * up) for one element, given dh (src/graph/ops/elementwise.rs:442-455 for silu, :294-331 for mul)
+__device__ __forceinline__ void swiglu_backward_elem(float gate, float up, float dh, float& dgate, float& dup) {
+    const float sig = 1.0f / (1.0f + __expf(-gate));
+    const float silu = gate * sig;
+    dgate = (dh * up) * (silu + sig * (1.0f - silu));
+    dup = dh * silu;
+}
+
+// Epilogue shared by the MFMA kernels.  Accumulator register v of lane l holds
+// C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.  `lds_f32` is the operand LDS (LDS_BYTES bytes), idle by now
+// and used as a staging area.
+template <int BM, int BN, int WGM, int WGN, bool EDGE, size_t LDS_BYTES, typename TC>
+__device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], float* lds_f32, TC* C,
+                                                const TC* Rsrc, bool add_old, int bz, int split, int part, int m0, int n0, int wave,
+                                                int wm, int wn, int lane) {
+    constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+    float* P = part > 0 ? g.partial + ((long long)bz * (split - 1) + (part - 1)) * g.M * g.N : nullptr;
+    constexpr int SP = WN + 4;  // staging pitch in floats
+    constexpr bool kCanStage = LDS_BYTES >= (size_t)WGM * WGN * 32 * SP * sizeof(float);
+    if (kCanStage && !EDGE && g.vec_c) {
+        // Each wave turns its accumulators, one 32-row band at a time, through a private piece of the
+        // (now idle) operand LDS so that a lane ends up with 8 consecutive columns of one row: C leaves in
+        // 16-byte stores covering whole 128/256-byte row segments instead of 2- or 4-byte ones.
+        float* stage = lds_f32 + wave * (32 * SP);
+        constexpr int LPR = WN / 8, PASSES = 32 * LPR / 64;  // lanes per row, passes per band
+        static_assert(32 * LPR % 64 == 0, "band must split evenly over the wave");
+        const int c = lane & 31, gh = lane >> 5;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) stage[(8 * (v / 4) + 4 * gh + (v % 4)) * SP + j * 32 + c] = acc[i][j][v];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ps++) {
+                const int idx = ps * 64 + lane, r = idx / LPR, cg = idx % LPR;
+                const float4 lo = *reinterpret_cast<const float4*>(stage + r * SP + cg * 8);
+                const float4 hi = *reinterpret_cast<const float4*>(stage + r * SP + cg * 8 + 4);
+                float val[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                const int m = m0 + wm * WM + i * 32 + r, n = n0 + wn * WN + cg * 8;
+                if (P) {
+                    float* dst = P + (long long)m * g.N + n;
+                    *reinterpret_cast<float4*>(dst) = lo;
+                    *reinterpret_cast<float4*>(dst + 4) = hi;
+                } else if (g.gate) {
+                    const long long at = (long long)bz * g.sC + (long long)m * g.ldc + n;
+                    const TC* gsrc = static_cast<const TC*>(g.gate) + at;
+                    const TC* usrc = static_cast<const TC*>(g.up) + at;
+                    Pack<TC> og[8 / Pack<TC>::N], ou[8 / Pack<TC>::N];
+#pragma unroll
+                    for (int k = 0; k < 8 / Pack<TC>::N; k++) {
+                        og[k] = load_pack(gsrc + k * Pack<TC>::N);
+                        ou[k] = load_pack(usrc + k * Pack<TC>::N);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        float dgate, dup;
+                        swiglu_backward_elem(og[e / Pack<TC>::N].get(e % Pack<TC>::N), ou[e / Pack<TC>::N].get(e % Pack<TC>::N), val[e], dgate, dup);
+                        og[e / Pack<TC>::N].set(e % Pack<TC>::N, dgate);
+                        ou[e / Pack<TC>::N].set(e % Pack<TC>::N, dup);
+                    }
+                    TC* d1 = C + (long long)m * g.ldc + n;
+                    TC* d2 = static_cast<TC*>(g.C2) + at;
+#pragma unroll
+                    for (int k = 0; k < 8 / Pack<TC>::N; k++) {
+                        store_pack(d1 + k * Pack<TC>::N, og[k]);
+                        store_pack(d2 + k * Pack<TC>::N, ou[k]);
+                    }
+                } else {
+                    TC* dst = C + (long long)m * g.ldc + n;
+                    Pack<TC> o[8 / Pack<TC>::N];
+                    if (add_old) {
+                        const TC* src = Rsrc + (long long)m * g.ldc + n;
+#pragma unroll
+                        for (int k = 0; k < 8 / Pack<TC>::N; k++) o[k] = load_pack(src + k * Pack<TC>::N);
+#pragma unroll
+                        for (int e = 0; e < 8; e++) val[e] += o[e / Pack<TC>::N].get(e % Pack<TC>::N);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; e++) o[e / Pack<TC>::N].set(e % Pack<TC>::N, val[e]);
+#pragma unroll
+                    for (int k = 0; k < 8 / Pack<TC>::N; k++) store_pack(dst + k * Pack<TC>::N, o[k]);
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wn * WN + j * 32 + (lane & 31);
+            if (EDGE && n >= g.N) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (!EDGE || m < g.M) {
+                    const float val = acc[i][j][v];
+                    if (P) {
+                        P[(long long)m * g.N + n] = val;
+                    } else if (g.gate) {
+                        const long long at = (long long)bz * g.sC + (long long)m * g.ldc + n;
+                        float dgate, dup;
+                        swiglu_backward_elem(to_f32(static_cast<const TC*>(g.gate)[at]), to_f32(static_cast<const TC*>(g.up)[at]), val, dgate, dup);
+                        C[(long long)m * g.ldc + n] = from_f32<TC>(dgate);
+                        static_cast<TC*>(g.C2)[at] = from_f32<TC>(dup);
+                    } else {
+                        TC* dst = C + (long long)m * g.ldc + n;
+                        *dst = from_f32<TC>(add_old ? to_f32(Rsrc[(long long)m * g.ldc + n]) + val : val);
+                    }
+                }
+            }
+        }
+}
+
+// ---- MFMA kernel with operands loaded straight into LDS ------------------------------------------
+// global_load_lds_dwordx4 moves 16 bytes per lane from global memory into LDS without passing through
+// registers: no staging registers, no LDS store instructions, no address arithmetic per chunk.  One wave
+// instruction fills 1 KB of consecutive LDS, so the tiles are unpadded and their rows are chunk-permuted
+// (lds_swz in device_utils.cuh) to keep the operand reads free of bank conflicts.
+// Three LDS stages: slab kt is multiplied while slabs kt+1 and kt+2 are in flight, one barrier per slab.
+// The loads are issued from inline assembly so that waiting for them stays in this file's hands
+// (vmcnt counts them in issue order); the kernel has no other vector memory loads in its main loop.
+template <int ROWS, bool KC, int BK, int WAVES>
+struct DirectOperandTile {
+    static constexpr int LDS_ROW = KC ? BK : ROWS;  // elements of one LDS row = one contiguous run of the operand in memory
+    static constexpr int ELEMS = ROWS * BK;
+    static constexpr int CPR = LDS_ROW / 8;         // 16-byte chunks per LDS row
+    static constexpr int RPB = 64 / CPR;            // LDS rows filled by one wave instruction
+    static constexpr int LOADS = ELEMS / 512 / WAVES;  // wave instructions per wave and slab
+    static_assert(CPR >= 4 && 64 % CPR == 0 && ELEMS % (512 * WAVES) == 0, "slab must split into whole 1 KB wave loads");
+
+    // LDS row and (permuted) chunk this lane fetches in load i of its wave
+    static __device__ __forceinline__ void lane_chunk(int i, int wave, int lane, int& row, int& chunk) {
+        row = (wave * LOADS + i) * RPB + lane / CPR;
+        chunk = (lane % CPR) ^ lds_swz<LDS_ROW * 2>(row);
+    }
+    static __device__ __forceinline__ int lds_block(int i, int wave) { return (wave * LOADS + i) * 512; }  // element offset in the tile
+
+    // MFMA operand of the 32 operand rows starting at `row0` for contraction offsets ks..ks+15 (same register
+    // contents as OperandTile::fragment)
+    static __device__ __forceinline__ bf16x8 fragment(const bf16_t* tile, int row0, int ks, int lane) {
+        if (KC) {
+            const int r = row0 + (lane & 31);
+            return *reinterpret_cast<const bf16x8*>(tile + r * BK + ((((ks >> 3) + (lane >> 5)) ^ lds_swz<BK * 2>(r)) << 3));
+        }
+        const int L = lane & 15, half = (lane >> 4) & 1;
+        const int k = ks + 8 * (lane >> 5) + (L >> 2), col = row0 + 16 * half + 4 * (L & 3);
+        const bf16_t* p_lo = tile + k * ROWS + ((((col >> 3) ^ lds_swz<ROWS * 2>(k)) << 3) | (col & 7));
+        const bf16_t* p_hi = tile + (k + 4) * ROWS + ((((col >> 3) ^ lds_swz<ROWS * 2>(k + 4)) << 3) | (col & 7));
+        const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p_lo));
+        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p_hi));
+        bf16x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    }
+};
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+// one wave instruction: lane l's 16 bytes at `src` land at lds_dst + 16*l (lds_dst is wave-uniform)
+__device__ __forceinline__ void load_to_lds_16(const void* src, bf16_t* lds_dst) {
+    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {  // until at most N of this wave's vector memory loads are outstanding
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// barrier without the memory fence of __syncthreads (which would wait for every outstanding load)
+__device__ __forceinline__ void barrier_no_fence() {
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_s_barrier();
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+
+}  // namespace

@@ -678,6 +678,15 @@ def test_gemm_bf16_wide_tile_grouped_order(ctx, ta, tb):
     _gemm_case(ctx, 3840, 8704, 192, ta, tb, BF16, F32, True, seed=483)
 
 
+@pytest.mark.parametrize("M,N,K", [(2816, 4096, 128), (2816, 4096, 384), (1536, 8448, 256)])
+def test_gemm_weight_gradient_256x256_tiles(ctx, M, N, K):
+    # dW = X^T dY from 176 tiles of 256 x 256 up: four waves of 128 x 128, a ring of four 32-deep slabs (K = 128 is one
+    # turn of the ring, 384 three); 8448 columns = 33 tiles walked in groups of 16, the last group one tile wide
+    _gemm_case(ctx, M, N, K, 1, 0, BF16, F32, True, seed=485)
+    _gemm_case(ctx, M, N, K, 1, 0, BF16, F32, False, seed=487)
+    _gemm_case(ctx, M, N, K, 1, 0, BF16, BF16, False, seed=489)
+
+
 def test_gemm_wide_tile_batched_and_segmented(ctx):
     # the launch-saving entry points at a shape that takes the 256x128 tile (256 tiles)
     M, N, K = 4096, 1024, 128
@@ -768,11 +777,12 @@ def test_side_stream_orders_after_fork_and_before_join(ctx):
         t.free()
 
 
-@pytest.mark.parametrize("M,K,Ns", [(2048, 128, (2048, 512, 512, 2048)), (2048, 192, (1024, 3072)), (256, 64, (128, 256, 128))])
+@pytest.mark.parametrize("M,K,Ns", [(2048, 128, (2048, 512, 512, 2048)), (2048, 192, (1024, 3072)), (256, 64, (128, 256, 128)),
+                                    (2048, 256, (2048, 512, 3072))])
 @pytest.mark.parametrize("accumulate", [0, 1])
 def test_gemm_grouped_weight_gradients(ctx, M, K, Ns, accumulate):
     # dW_p (+)= X_p^T dY_p with X_p [K, M] and dY_p [K, N_p] (here K is the token count): the first two shapes run as one
-    # grid of 128x128 tiles, the last one falls back to one launch per product
+    # grid of 128x128 tiles, the third falls back to one launch per product, the last is one grid of 176 tiles of 256x256
     xs = [prep(gen.normal(550 + i, (K, M)), BF16) for i in range(len(Ns))]
     dys = [prep(gen.normal(560 + i, (K, n)), BF16) for i, n in enumerate(Ns)]
     c0 = [gen.normal(570 + i, (M, n)).astype(np.float32) for i, n in enumerate(Ns)]
