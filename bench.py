@@ -159,7 +159,7 @@ def cpu_baseline_lm(c, seq, mb=1):
 # workloads
 # ---------------------------------------------------------------------------------------------
 
-def bench_lm(name, steps, warmup, with_cpu=True):
+def bench_lm(name, steps, warmup, with_cpu=True, recompute=False):
     from eisen_amd import graph as G
     from eisen_amd import hip
     c = CONFIGS[name]
@@ -172,6 +172,7 @@ def bench_lm(name, steps, warmup, with_cpu=True):
         if len(shape) == 2:   # matrices N(0, 0.02); norm gains stay 1.0
             g.load_tensor_data(pid, rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02))
     g.mark_params()
+    lm.set_checkpointing(recompute)   # per-block recompute: off in the headline run (the reference's train_llm.rs does not use it)
     opt = G.AdamW(g, lm.params(), 1e-3)
     opt.config(1e-3, 0.9, 0.95, 1e-8, 0.1, 1.0)      # train_llm.rs:266-270 + grad clip 1.0
     opt.init_moments()
@@ -212,7 +213,7 @@ def bench_lm(name, steps, warmup, with_cpu=True):
     out = dict(metric="train tokens/sec (fwd+bwd+AdamW)", value=round(value, 1), unit="tokens/s", n_gpus=1, steps=steps, warmup=warmup,
                ms_per_step=round(1e3 * elapsed / steps, 3), higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16",
                data="synthetic",
-               config=dict(workload=c["label"], tokens_per_step=tokens_per_step, parallelism="single GPU",
+               config=dict(workload=c["label"] + (", per-block recompute" if recompute else ""), tokens_per_step=tokens_per_step, parallelism="single GPU",
                            step_model_tflops=round(step_flops / 1e12, 4),
                            mfma_frac_of_step=round(step_flops / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 4), last_loss=round(float(last_loss), 4)),
                roofline=pick_dominant(prof, name), kernels=kernel_table(prof))
@@ -332,17 +333,18 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="all", choices=["all", "c5", "c4", "c3", "c2"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
+    ap.add_argument("--recompute", action="store_true", help="c5 / c4: per-block recompute (lower activation memory, one more forward pass per block)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
     w = args.workload
     if w in ("all", "c5"):
-        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu)
+        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute)
         if w == "all":
             out["other_configs"] = dict(c4=brief(bench_lm("c4", 20, 3, not args.no_cpu)), c3=brief(bench_c3(20, 3)), c2=brief(bench_c2(20, 3)))
     elif w == "c4":
-        out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu)
+        out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute)
     elif w == "c3":
         out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3)
     else:

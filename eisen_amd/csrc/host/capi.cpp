@@ -84,6 +84,9 @@ int eisen_graph_load_tensor_data(eisen_graph* g, size_t id, const float* host, s
 int eisen_graph_mark_params(eisen_graph* g) { return guarded(g, [&](Graph& G) { G.mark_params(); }); }
 int eisen_graph_mark_save_point(eisen_graph* g, size_t* out) { return guarded(g, [&](Graph& G) { need(out, "out"); *out = G.mark_save_point(); }); }
 int eisen_graph_restore_save_point(eisen_graph* g, size_t sp) { return guarded(g, [&](Graph& G) { G.restore_save_point(sp); }); }
+int eisen_graph_restore_save_point_keep(eisen_graph* g, size_t sp, size_t keep, size_t* out) {
+    return guarded(g, [&](Graph& G) { need(out, "out"); *out = G.restore_save_point_keep(sp, keep); });
+}
 int eisen_graph_clear_activations(eisen_graph* g) { return guarded(g, [&](Graph& G) { G.clear_activations(); }); }
 int eisen_graph_reinterpret_shape(eisen_graph* g, size_t id, const size_t* shape, int rank) {
     return guarded(g, [&](Graph& G) { G.reinterpret_shape(id, shape_of(shape, rank)); });
@@ -181,6 +184,11 @@ int eisen_lm_forward(eisen_graph* g, eisen_lm* lm, size_t x_id, size_t* out) {
 int eisen_lm_set_fused(eisen_lm* lm, int fused) {
     if (!lm) return -1;
     lm->lm->set_fused(fused != 0);
+    return 0;
+}
+int eisen_lm_set_checkpointing(eisen_lm* lm, int on) {
+    if (!lm) return -1;
+    lm->lm->set_checkpointing(on != 0);
     return 0;
 }
 int eisen_lm_micro_step(eisen_graph* g, eisen_lm* lm, const float* ids, const int64_t* targets, size_t mb, size_t seq, float* loss_out) {

@@ -196,13 +196,22 @@ void Graph::restore_save_point(size_t save_point) {
         tensors.pop_back();
     }
 }
+size_t Graph::restore_save_point_keep(size_t save_point, size_t keep) {
+    if (keep < save_point || keep >= tensors.size()) throw Error("restore_save_point_keep: the tensor to keep is not above the save point");
+    Tensor kept = std::move(tensors[keep]);
+    tensors[keep] = Tensor();  // nothing left to release there
+    restore_save_point(save_point);
+    kept.id = tensors.size();
+    tensors.push_back(std::move(kept));
+    return tensors.size() - 1;
+}
 void Graph::clear_activations() {
     tape.nodes.clear();
     restore_save_point(num_params);
 }
 
 void Graph::record(std::vector<size_t> inputs, size_t output, std::function<void(Graph&)> fn) {
-    if (no_grad) return;  // e.g. src/graph/ops/linear.rs:288
+    if (no_grad || tape_paused) return;  // e.g. src/graph/ops/linear.rs:288
     tape.nodes.push_back(TapeNode{std::move(inputs), output, std::move(fn)});
 }
 
@@ -281,19 +290,24 @@ void Graph::backward(size_t loss_id) {
     int acc = 0;
     Storage& lg = grad_for_write(loss_id, &acc);
     check(eisen_hip_fill(ctx_, lg.ptr, lg.dtype, 1.0f, lg.numel), "backward seed");
-    for (size_t i = tape.nodes.size(); i-- > 0;) {
-        TapeNode& node = tape.nodes[i];
-        Tensor& out = at(node.output);
-        // an output nobody differentiated through has a zero gradient: nothing to propagate
-        if (!out.is_param && !(out.grad.valid() && out.grad_written)) continue;
-        node.backward_fn(*this);
-    }
+    backward_nodes_from(0);
     backward_root_ = (size_t)-1;
     flush_norm_dw(true);
     side_join();
     if (!pending_dw.empty()) {
         pending_dw.clear();
         throw Error("backward: a deferred weight gradient was not collected by a matmul_group");
+    }
+}
+
+void Graph::backward_nodes_from(size_t first_node) {
+    for (size_t i = tape.nodes.size(); i-- > first_node;) {
+        const Tensor& out = at(tape.nodes[i].output);
+        // an output nobody differentiated through has a zero gradient: nothing to propagate
+        if (!out.is_param && !(out.grad.valid() && out.grad_written)) continue;
+        // a copy: the closure may record further nodes (a recomputed block), which can move the tape's storage
+        const std::function<void(Graph&)> fn = tape.nodes[i].backward_fn;
+        fn(*this);
     }
 }
 

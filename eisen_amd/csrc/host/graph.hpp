@@ -72,6 +72,9 @@ class Graph {
     Tape tape;
     size_t num_params = 0;
     bool no_grad = false;
+    // Like no_grad for the tape only: ops record nothing but still choose the kernels of a training forward pass (no_grad
+    // also switches attention to the inference path, src/nn/attention.rs:335-336, whose bits differ from the chain's).
+    bool tape_paused = false;
     PrecisionMode precision_mode;
 
     Graph(eisen_ctx* ctx, PrecisionMode mode);
@@ -88,6 +91,11 @@ class Graph {
     void mark_params() { num_params = tensors.size(); }
     size_t mark_save_point() const { return tensors.size(); }
     void restore_save_point(size_t save_point);
+    // restore_save_point that lets one of the dropped tensors live on: `keep` (>= save_point) becomes tensor
+    // `save_point`, everything else above the save point is released.  Returns the new id.  (The reference's test of the
+    // primitives, tests/gpu_kernels.rs:560-610, copies the value out instead; a block-by-block recompute needs it on the
+    // device.)
+    size_t restore_save_point_keep(size_t save_point, size_t keep);
     void clear_activations();
     size_t alloc(const std::vector<size_t>& shape, const std::vector<float>& data);
     size_t alloc(const std::vector<size_t>& shape, const float* data, size_t n);
@@ -141,6 +149,9 @@ class Graph {
 
     // src/graph/mod.rs:670-796
     void backward(size_t loss_id);
+    // Replays tape nodes [first_node, end) in reverse, as backward() does for the whole tape: for a backward closure that
+    // recorded more nodes (a recomputed block) and now differentiates through them.
+    void backward_nodes_from(size_t first_node);
 
     // ---- helpers for optimisers and backward closures -----------------------------------------
     Tensor& at(size_t id);

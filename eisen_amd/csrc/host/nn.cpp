@@ -266,10 +266,48 @@ void TransformerLM::set_fused(bool fused) {
     for (auto& b : blocks) b.attn.fused = fused;
 }
 
+// One block under per-block recompute.  Forward: the block runs with the tape paused (the kernels of a training forward
+// pass, no tape nodes), then everything it allocated
+// except its output goes back to the pool.  The one tape node recorded for it re-runs the block from its input when the
+// backward pass reaches it, seeds the recomputed output's gradient with the gradient that arrived at the kept output,
+// replays the new nodes and drops them again.  The kernels are deterministic, so the recomputed activations and the
+// gradients equal those of the plain step bit for bit.
+static size_t checkpointed_block(Graph& g, const TransformerBlock& block, size_t x_id) {
+    const size_t sp = g.mark_save_point();
+    g.tape_paused = true;
+    size_t y;
+    try {
+        y = block.forward_with_mask(g, x_id, true);
+    } catch (...) {
+        g.tape_paused = false;
+        throw;
+    }
+    g.tape_paused = false;
+    y = g.restore_save_point_keep(sp, y);
+    const TransformerBlock* b = &block;  // blocks live as long as the model, which outlives the tape
+    g.tape.nodes.push_back(TapeNode{{x_id}, y, [b, x_id, y](Graph& G) {
+        const size_t sp2 = G.mark_save_point(), first = G.tape.nodes.size();
+        const size_t y2 = b->forward_with_mask(G, x_id, true);
+        {   // the gradient buffer moves over: the recomputed output owns it from here on (it travels on to the residual)
+            Tensor& ty = G.at(y);
+            Tensor& t2 = G.at(y2);
+            t2.grad = ty.grad;
+            t2.grad_written = true;
+            ty.grad = Storage();
+            ty.grad_written = false;
+        }
+        G.backward_nodes_from(first);
+        G.tape.nodes.erase(G.tape.nodes.begin() + first, G.tape.nodes.end());
+        G.flush_norm_dw(true);  // the gain gradients' partial rows belong to this block
+        G.restore_save_point(sp2);
+    }});
+    return y;
+}
+
 // TransformerLM::forward (src/nn/transformer.rs:184-196).
 size_t TransformerLM::forward(Graph& g, size_t x_id) const {
     size_t h = token_emb.forward(g, x_id);
-    for (const TransformerBlock& b : blocks) h = b.forward_with_mask(g, h, true);
+    for (const TransformerBlock& b : blocks) h = checkpointing && !g.no_grad ? checkpointed_block(g, b, h) : b.forward_with_mask(g, h, true);
     h = norm_f.forward(g, h);
     if (tie_weights) return g.matmul_trans_b(h, lm_head.weight_id);
     return lm_head.forward(g, h);

@@ -91,6 +91,11 @@ struct TransformerLM : Module {
     std::vector<std::pair<std::string, size_t>> named_params() const;
     void tag_parameters(Graph& g) const;
     void set_fused(bool fused);
+    // Per-block recompute on the save-point primitives (src/graph/mod.rs:332-365, exercised block-wise by
+    // tests/gpu_kernels.rs:560-610): forward() runs each block without a tape and keeps only its output; backward re-runs
+    // the block from its input, differentiates it and drops its activations again.  Same gradients, bit for bit.
+    bool checkpointing = false;
+    void set_checkpointing(bool on) { checkpointing = on; }
     size_t forward(Graph& g, size_t x_id) const override;
     std::vector<size_t> params() const override;
 };

@@ -46,6 +46,7 @@ struct eisen_ctx {
     std::unordered_map<size_t, std::vector<void*>> free_lists;
     std::unordered_map<void*, size_t> live;
     size_t in_use_bytes = 0, cached_bytes = 0;
+    size_t peak_in_use_bytes = 0;  // high-water mark of in_use_bytes since the last reset
     // pinned staging ring for asynchronous uploads: a slot is reused only after its copy's event fired
     struct StageSlot {
         void* ptr = nullptr;

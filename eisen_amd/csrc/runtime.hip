@@ -168,6 +168,7 @@ extern "C" int eisen_hip_malloc(eisen_ctx* ctx, size_t bytes, void** out) {
     }
     ctx->live[p] = bytes;
     ctx->in_use_bytes += bytes;
+    if (ctx->in_use_bytes > ctx->peak_in_use_bytes) ctx->peak_in_use_bytes = ctx->in_use_bytes;
     *out = p;
     return 0;
 }
@@ -188,6 +189,13 @@ extern "C" int eisen_hip_free(eisen_ctx* ctx, void* ptr) {
     ctx->in_use_bytes -= bytes;
     ctx->free_lists[bytes].push_back(ptr);
     ctx->cached_bytes += bytes;
+    return 0;
+}
+
+extern "C" int eisen_hip_pool_peak(eisen_ctx* ctx, size_t* peak_in_use_bytes, int reset) {
+    EISEN_CHECK_CTX(ctx);
+    if (peak_in_use_bytes) *peak_in_use_bytes = ctx->peak_in_use_bytes;
+    if (reset) ctx->peak_in_use_bytes = ctx->in_use_bytes;
     return 0;
 }
 

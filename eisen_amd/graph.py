@@ -88,6 +88,11 @@ class Graph:
     def set_no_grad(self, v): self._call("eisen_graph_set_no_grad", _i(int(v)))
     def restore_save_point(self, sp): self._call("eisen_graph_restore_save_point", _sz(sp))
 
+    def restore_save_point_keep(self, sp, keep):
+        out = _sz()
+        self._call("eisen_graph_restore_save_point_keep", _sz(sp), _sz(keep), C.byref(out))
+        return out.value
+
     def mark_save_point(self):
         out = _sz()
         self._call("eisen_graph_mark_save_point", C.byref(out))
@@ -200,6 +205,9 @@ class TransformerLM:
 
     def set_fused(self, fused):
         self._check("eisen_lm_set_fused", self.g.lib.eisen_lm_set_fused(self.h, _i(int(fused))))
+
+    def set_checkpointing(self, on):
+        self._check("eisen_lm_set_checkpointing", self.g.lib.eisen_lm_set_checkpointing(self.h, _i(int(on))))
 
     def forward(self, x_id):
         return self.g._op("eisen_lm_forward", self.h, _sz(x_id))

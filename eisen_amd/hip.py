@@ -149,6 +149,11 @@ class Context:
         self._call("eisen_hip_pool_stats", C.byref(a), C.byref(b))
         return a.value, b.value
 
+    def pool_peak(self, reset=False):
+        a = _sz()
+        self._call("eisen_hip_pool_peak", C.byref(a), _i(int(reset)))
+        return a.value
+
     def pool_trim(self):
         self._call("eisen_hip_pool_trim")
 

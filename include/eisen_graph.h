@@ -44,6 +44,11 @@ int eisen_graph_load_tensor_data(eisen_graph* g, size_t id, const float* host, s
 int eisen_graph_mark_params(eisen_graph* g);
 int eisen_graph_mark_save_point(eisen_graph* g, size_t* save_point_out);
 int eisen_graph_restore_save_point(eisen_graph* g, size_t save_point);
+/* restore_save_point that keeps one of the dropped tensors: `keep` (>= save_point) becomes tensor `save_point`
+ * (its new id is returned), everything else above the save point goes back to the pool.  The reference's test of the
+ * primitives (tests/gpu_kernels.rs:560-610) copies the block output to the host instead; recompute block by block
+ * needs it to stay on the device. */
+int eisen_graph_restore_save_point_keep(eisen_graph* g, size_t save_point, size_t keep, size_t* new_id_out);
 int eisen_graph_clear_activations(eisen_graph* g);
 int eisen_graph_reinterpret_shape(eisen_graph* g, size_t id, const size_t* shape, int rank);
 int eisen_graph_set_no_grad(eisen_graph* g, int no_grad);
@@ -92,6 +97,10 @@ int eisen_lm_params(eisen_lm* lm, size_t* ids_out, size_t capacity, size_t* coun
 int eisen_lm_forward(eisen_graph* g, eisen_lm* lm, size_t x_id, size_t* logits_out);
 /* 1: fused attention + SwiGLU ops (default); 0: the reference's materialised op chain. */
 int eisen_lm_set_fused(eisen_lm* lm, int fused);
+/* 1: per-block recompute on mark_save_point / restore_save_point (src/graph/mod.rs:332-365): forward keeps each block's
+ * output only, backward re-runs the block before differentiating it.  Gradients are those of the plain step bit for
+ * bit; the activation high-water mark drops from all blocks' activations to one block's.  Default 0. */
+int eisen_lm_set_checkpointing(eisen_lm* lm, int on);
 /* One micro-step of examples/train_llm.rs:433-458 (upload ids, forward, cross entropy, backward,
  * clear_activations).  ids: f32 token ids [mb*seq]; targets int64 [mb*seq].  loss_out may be
  * NULL, in which case nothing synchronises. */

@@ -78,6 +78,8 @@ int eisen_hip_pool_trim(eisen_ctx* ctx);
 int eisen_hip_mem_info(eisen_ctx* ctx, size_t* free_bytes, size_t* total_bytes);
 /* Bytes currently handed out / cached by the pool (diagnostics, tests). */
 int eisen_hip_pool_stats(eisen_ctx* ctx, size_t* in_use_bytes, size_t* cached_bytes);
+/* Largest value in_use_bytes has had since the last call with reset != 0 (the activation high-water mark of a step). */
+int eisen_hip_pool_peak(eisen_ctx* ctx, size_t* peak_in_use_bytes, int reset);
 
 /* stream.memcpy_htod / clone_htod (src/graph/mod.rs:368-430, src/tensor.rs:156-160):
  * asynchronous on the stream; the host buffer is copied to a staging area first, so it may

@@ -91,10 +91,28 @@ def test_config5_full_model_micro_step(ctx):
 
     # ---- the same micro-step through lm.micro_step: identical bits (no atomics, ordered streams)
     opt.zero_grad()
+    ctx.sync()
+    ctx.pool_peak(reset=True)
+    in_use = ctx.pool_stats()[0]
     loss2 = lm.micro_step(x, y)
+    peak_plain = ctx.pool_peak() - in_use
     assert loss2 == loss
     for p, d in zip(params, digests):
         assert _digest(gg.sync_grad_to_cpu(p)) == d, f"gradient of tensor {p} differs between two runs"
+
+    # ---- per-block recompute (set_checkpointing): the same bits again, with one block's activations alive at a time
+    lm.set_checkpointing(True)
+    opt.zero_grad()
+    ctx.sync()
+    ctx.pool_peak(reset=True)
+    loss_ck = lm.micro_step(x, y)
+    peak_ck = ctx.pool_peak() - in_use
+    lm.set_checkpointing(False)
+    assert loss_ck == loss
+    for p, d in zip(params, digests):
+        assert _digest(gg.sync_grad_to_cpu(p)) == d, f"gradient of tensor {p} differs under per-block recompute"
+    print(f"\nconfig 5, 4 x 1024 tokens: activation high-water mark {peak_plain / 2**30:.2f} GiB plain, {peak_ck / 2**30:.2f} GiB with per-block recompute")
+    assert peak_ck < 0.5 * peak_plain, (peak_plain, peak_ck)
 
     # ---- the fused path against the reference's op-by-op chain, all 16 layers (separately oracle-checked kernels)
     lm.set_fused(False)

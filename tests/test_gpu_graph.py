@@ -141,6 +141,58 @@ def test_gradient_checkpoint_primitives_are_deterministic(g):
     assert g.num_tensors() == g.num_params() and g.tape_len() == 0
 
 
+def test_restore_save_point_keep_moves_one_tensor_down(g):
+    a = g.alloc((2, 2), [1, 2, 3, 4])
+    g.mark_params()
+    sp = g.mark_save_point()
+    g.set_no_grad(True)
+    b = g.add(a, a)
+    c = g.mul(b, b)
+    d = g.add(c, a)
+    kept = g.restore_save_point_keep(sp, c)
+    g.set_no_grad(False)
+    assert kept == sp and g.num_tensors() == sp + 1 and d >= g.num_tensors()
+    assert g.sync_to_cpu(kept).reshape(-1).tolist() == [4.0, 16.0, 36.0, 64.0]
+    with pytest.raises(EisenHipError):
+        g.restore_save_point_keep(sp + 1, sp)   # the tensor to keep lies below the save point
+
+
+@pytest.mark.parametrize("precision,fused", [(G.FP32, True), (G.FP32, False), (G.BF16_MIXED, True), (G.BF16_MIXED, False)],
+                         ids=["f32-fused", "f32-chain", "bf16-fused", "bf16-chain"])
+def test_per_block_recompute_gives_the_same_bits_and_a_lower_high_water_mark(ctx, precision, fused):
+    # TransformerLM::set_checkpointing on mark_save_point / restore_save_point (src/graph/mod.rs:332-365): each block's
+    # forward re-runs inside backward.  Deterministic kernels => losses and every gradient bit-identical to the plain
+    # step, over two accumulated micro-batches; the peak of pool bytes in use drops.
+    cfg = dict(vocab=512, hidden=256, heads=4, kv_heads=2, ffn=512, layers=6, tie=False)
+    mb, seq = 4, 128
+    batches = [gen.lm_batch(900 + i, mb, seq, cfg["vocab"]) for i in range(2)]
+    results = []
+    for checkpointing in (False, True):
+        gg = G.Graph(ctx, precision)
+        lm = G.TransformerLM(gg, **cfg)
+        for pid, (_, w) in enumerate(gen.lm_weights(33, perturb_norm=0.1, **cfg)):
+            gg.load_tensor_data(pid, w)
+        gg.mark_params()
+        lm.set_fused(fused)
+        lm.set_checkpointing(checkpointing)
+        params = lm.params()
+        opt = G.AdamW(gg, params, 1e-3)
+        opt.zero_grad()
+        ctx.sync()
+        ctx.pool_peak(reset=True)
+        base = ctx.pool_stats()[0]
+        losses = [lm.micro_step(x, y) for x, y in batches]
+        peak = ctx.pool_peak() - base
+        assert gg.num_tensors() == gg.num_params() and gg.tape_len() == 0
+        results.append((losses, [gg.sync_grad_to_cpu(p) for p in params], peak))
+        gg.close()
+    (l0, g0, peak0), (l1, g1, peak1) = results
+    assert l0 == l1
+    for i, (a, b) in enumerate(zip(g0, g1)):
+        assert a.any() and np.array_equal(a, b), f"gradient of parameter {i} differs under per-block recompute"
+    assert peak1 < 0.6 * peak0, (peak0, peak1)
+
+
 # ---- composed training step against the oracle ---------------------------------------------------
 
 def _build_pair(ctx, cfg, weights, precision):
