@@ -87,6 +87,188 @@ __global__ __launch_bounds__(kThreads) void scatter_rows_scalar_kernel(const T* 
     gw[(size_t)seg_row[seg] * hidden + col] = acc;
 }
 
+// ---- position index built on the device ---------------------------------------------------------
+// Keys id * n_pow2 + position are unique, so sorting them is the stable sort of the positions by id.  One workgroup of
+// 1024 threads sorts 1024 * R of them (R = 1..16) with a bitonic network whose keys stay in registers: thread t holds
+// elements t, t + 1024, ...; a compare-exchange at distance j >= 1024 pairs two registers of one thread, j < 64 two
+// lanes of one wave (a shuffle), and only the distances 64..512 go through LDS (18 to 26 of the 55 to 105 steps).  The
+// kernel writes the ids and positions in key order; ids outside [0, vocab) get the padding key and drop out.
+constexpr int kSortThreads = 1024, kSortMax = 16384;
+template <int R>
+__global__ __launch_bounds__(kSortThreads) void scatter_sort_kernel(const int32_t* __restrict__ ids, int n, int shift, int vocab,
+                                                                   int32_t* __restrict__ sorted_ids, int32_t* __restrict__ order,
+                                                                   int32_t* __restrict__ run_end) {
+    constexpr int NP = kSortThreads * R;
+    __shared__ unsigned keys[NP];
+    const int tid = threadIdx.x;
+    unsigned key[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kSortThreads + tid;
+        unsigned v = 0xffffffffu;
+        if (i < n) {
+            const int id = ids[i];
+            if (id >= 0 && id < vocab) v = ((unsigned)id << shift) | (unsigned)i;
+        }
+        key[r] = v;
+    }
+#pragma unroll
+    for (int k = 2; k <= NP; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            if (j >= kSortThreads) {
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const int rp = r ^ (j / kSortThreads);
+                    if (rp > r) {  // registers r and rp of this thread: element r * 1024 + tid is the lower one
+                        const bool asc = (((r * kSortThreads) & k) == 0);  // bit k of the element index lies in the register part (k > j >= 1024)
+                        const unsigned lo = min(key[r], key[rp]), hi = max(key[r], key[rp]);
+                        key[r] = asc ? lo : hi;
+                        key[rp] = asc ? hi : lo;
+                    }
+                }
+            } else {
+                if (j >= 64) {
+                    __syncthreads();  // the previous exchange's reads are done
+#pragma unroll
+                    for (int r = 0; r < R; r++) keys[r * kSortThreads + tid] = key[r];
+                    __syncthreads();
+                }
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const int i = r * kSortThreads + tid;
+                    const unsigned other = j >= 64 ? keys[r * kSortThreads + (tid ^ j)] : (unsigned)__shfl_xor((int)key[r], j, 64);
+                    const bool keep_min = ((i & j) == 0) == ((i & k) == 0);
+                    key[r] = keep_min ? min(key[r], other) : max(key[r], other);
+                }
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < R; r++) keys[r * kSortThreads + tid] = key[r];
+    __syncthreads();
+    // ids and positions in key order; where a run of equal ids starts, the index one past its end (binary search in the
+    // sorted keys), elsewhere -1
+    for (int i = threadIdx.x; i < n; i += kSortThreads) {
+        const unsigned key = keys[i];
+        const bool real = key != 0xffffffffu;
+        const unsigned id = key >> shift;
+        sorted_ids[i] = real ? (int32_t)id : -1;
+        order[i] = (int32_t)(key & ((1u << shift) - 1));
+        int end = -1;
+        if (real && (i == 0 || (keys[i - 1] >> shift) != id)) {
+            int lo = i + 1, hi = n;  // first index in [lo, hi] whose id differs (padding keys count as different)
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                const unsigned km = keys[mid];
+                if (km != 0xffffffffu && (km >> shift) == id) lo = mid + 1;
+                else hi = mid;
+            }
+            end = lo;
+        }
+        run_end[i] = end;
+    }
+}
+
+// scatter_rows_kernel without the host-built segment table: a wave looks at sorted position k, leaves unless k starts
+// a run of equal ids, and adds the run's rows in order.  The hot rows of a Zipf batch are chains of hundreds of
+// dependent adds whose speed is set by how many row loads are in flight, so a lane takes only two columns (a wave 128)
+// and a long run is walked 64 rows at a time, all 64 loads issued before the first add.
+template <typename T> struct Pair;
+template <> struct Pair<float> { typedef float2 type; };
+template <> struct Pair<bf16_t> { typedef __attribute__((ext_vector_type(2))) __bf16 type; };
+template <typename T>
+__global__ __launch_bounds__(kThreads) void scatter_runs_kernel(const T* __restrict__ go, float* __restrict__ gw,
+                                                                const int32_t* __restrict__ sorted_ids,
+                                                                const int32_t* __restrict__ order,
+                                                                const int32_t* __restrict__ run_end, int n, int hidden, int slabs) {
+    typedef typename Pair<T>::type P2;
+    const int lane = threadIdx.x & 63;
+    const size_t wave = __builtin_amdgcn_readfirstlane((int)(((size_t)blockIdx.x * kThreads + threadIdx.x) >> 6));
+    const int begin = (int)(wave / slabs);
+    if (begin >= n) return;
+    const int end = run_end[begin];
+    if (end < 0) return;  // not the start of a run
+    const int row = sorted_ids[begin];
+    const int col = ((int)(wave % slabs) * kWave + lane) * 2;
+    if (col >= hidden) return;
+    float* dst = gw + (size_t)row * hidden + col;
+    float2 acc = *reinterpret_cast<const float2*>(dst);
+    const T* src = go + col;
+    int k = begin;
+    for (; k + 64 <= end; k += 64) {
+        P2 p[64];
+#pragma unroll
+        for (int u = 0; u < 64; u++) p[u] = *reinterpret_cast<const P2*>(src + (size_t)order[k + u] * hidden);
+#pragma unroll
+        for (int u = 0; u < 64; u++) {
+            acc.x += (float)p[u][0];
+            acc.y += (float)p[u][1];
+        }
+    }
+    for (; k + 8 <= end; k += 8) {
+        P2 p[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) p[u] = *reinterpret_cast<const P2*>(src + (size_t)order[k + u] * hidden);
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            acc.x += (float)p[u][0];
+            acc.y += (float)p[u][1];
+        }
+    }
+    for (; k < end; k++) {
+        const P2 p = *reinterpret_cast<const P2*>(src + (size_t)order[k] * hidden);
+        acc.x += (float)p[0];
+        acc.y += (float)p[1];
+    }
+    *reinterpret_cast<float2*>(dst) = acc;
+}
+
+// The device route takes batches whose keys fit 32 bits and whose rows are whole column pairs.
+bool scatter_on_device(const void* go, const float* gw, int dtype, size_t n_ids, size_t vocab, size_t hidden, int* n_pow2, int* shift) {
+    if (n_ids == 0 || n_ids > (size_t)kSortMax) return false;
+    int p = kSortThreads, sh = 10;  // the sort works on whole multiples of its 1024 threads
+    while ((size_t)p < n_ids) { p <<= 1; sh++; }
+    if ((unsigned long long)vocab << sh >= 0xffffffffull) return false;
+    (void)dtype;
+    if (hidden % 2 != 0 || !eisen_aligned(go, 8) || !eisen_aligned(gw, 8)) return false;
+    *n_pow2 = p;
+    *shift = sh;
+    return true;
+}
+
+int scatter_device_route(eisen_ctx* ctx, const int32_t* ids_dev, const void* go, float* gw, int dtype, size_t n_ids, size_t vocab, size_t hidden,
+                         int n_pow2, int shift) {
+    void* dev = nullptr;
+    int rc = eisen_hip_malloc(ctx, 3 * n_ids * sizeof(int32_t), &dev);
+    if (rc) return rc;
+    int32_t* sorted_ids = (int32_t*)dev;
+    int32_t* order = sorted_ids + n_ids;
+    int32_t* run_end = order + n_ids;
+    {
+        // algorithmic bytes: every row of dOut read once, every touched row of the f32 gradient read and written once; the
+        // touched rows are not known on the host here, so the entry counts dOut and the index only (a lower bound)
+        EisenProfScope prof(ctx, dtype == EISEN_BF16 ? "scatter_rows_bf16" : "scatter_rows_f32",
+                            (double)n_ids * (double)hidden * eisen_dtype_size(dtype) + 16.0 * (double)n_ids);
+        switch (n_pow2 / kSortThreads) {
+            case 1: scatter_sort_kernel<1><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+            case 2: scatter_sort_kernel<2><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+            case 4: scatter_sort_kernel<4><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+            case 8: scatter_sort_kernel<8><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+            default: scatter_sort_kernel<16><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+        }
+        const int slabs = (int)eisen_ceil_div(hidden, (size_t)kWave * 2);
+        const unsigned blocks = (unsigned)eisen_ceil_div(n_ids * slabs, (size_t)(kThreads / kWave));
+        if (dtype == EISEN_F32) scatter_runs_kernel<float><<<blocks, kThreads, 0, ctx->stream>>>((const float*)go, gw, sorted_ids, order, run_end, (int)n_ids, (int)hidden, slabs);
+        else scatter_runs_kernel<bf16_t><<<blocks, kThreads, 0, ctx->stream>>>((const bf16_t*)go, gw, sorted_ids, order, run_end, (int)n_ids, (int)hidden, slabs);
+    }
+    hipError_t e = hipGetLastError();
+    const int rc_free = eisen_hip_free(ctx, dev);  // stream-ordered: the block is reused only by later work
+    if (e != hipSuccess) return eisen_set_error(ctx, (int)e, "scatter kernels: %s", hipGetErrorString(e));
+    return rc_free;
+}
+
 }  // namespace
 
 extern "C" int eisen_hip_gather(eisen_ctx* ctx, const void* weight, const int32_t* ids, void* out, int dtype,
@@ -124,7 +306,18 @@ extern "C" int eisen_hip_gather_backward(eisen_ctx* ctx, const int32_t* ids_host
     for (size_t i = 0; i < n_ids; i++)
         EISEN_REQUIRE(ctx, ids_host[i] >= 0 && (size_t)ids_host[i] < vocab, EISEN_E_ARG,
                       "gather_backward: id %d at position %zu outside [0, %zu)", ids_host[i], i, vocab);
-    // stable order of positions by token id: ties keep ascending position
+    int n_pow2 = 0, shift = 0;
+    if (scatter_on_device(go, gw, dtype, n_ids, vocab, hidden, &n_pow2, &shift)) {
+        // the index is built on the device: the host only hands the ids over
+        void* dids = nullptr;
+        int rc = eisen_hip_malloc(ctx, n_ids * sizeof(int32_t), &dids);
+        if (rc) return rc;
+        rc = eisen_hip_htod(ctx, dids, ids_host, n_ids * sizeof(int32_t));
+        if (!rc) rc = scatter_device_route(ctx, (const int32_t*)dids, go, gw, dtype, n_ids, vocab, hidden, n_pow2, shift);
+        const int rc_free = eisen_hip_free(ctx, dids);
+        return rc ? rc : rc_free;
+    }
+    // larger batches: stable order of positions by token id on the host, ties keep ascending position
     std::vector<int32_t> order(n_ids);
     std::iota(order.begin(), order.end(), 0);
     std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return ids_host[a] < ids_host[b]; });
@@ -176,4 +369,22 @@ extern "C" int eisen_hip_gather_backward(eisen_ctx* ctx, const int32_t* ids_host
         EISEN_LAUNCH_CHECK(ctx, "scatter_rows_scalar_kernel");
     }
     return eisen_hip_free(ctx, dev);  // stream-ordered: the block is reused only by later work
+}
+
+extern "C" int eisen_hip_gather_backward_dev(eisen_ctx* ctx, const int32_t* ids_dev, const void* go, float* gw, int dtype, size_t n_ids,
+                                             size_t vocab, size_t hidden) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, ids_dev && go && gw, EISEN_E_ARG, "gather_backward_dev: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "gather_backward_dev: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, vocab > 0 && vocab < (size_t(1) << 31) && hidden > 0 && hidden < (size_t(1) << 30) && n_ids < (size_t(1) << 31),
+                  EISEN_E_SHAPE, "gather_backward_dev: sizes out of range");
+    if (n_ids == 0) return 0;
+    int n_pow2 = 0, shift = 0;
+    if (scatter_on_device(go, gw, dtype, n_ids, vocab, hidden, &n_pow2, &shift))
+        return scatter_device_route(ctx, ids_dev, go, gw, dtype, n_ids, vocab, hidden, n_pow2, shift);
+    // shapes the device route does not take: the ids come back to the host (this synchronises) for the host-built index
+    std::vector<int32_t> host(n_ids);
+    int rc = eisen_hip_dtoh(ctx, host.data(), ids_dev, n_ids * sizeof(int32_t));
+    if (rc) return rc;
+    return eisen_hip_gather_backward(ctx, host.data(), go, gw, dtype, n_ids, vocab, hidden);
 }

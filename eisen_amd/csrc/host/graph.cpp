@@ -892,7 +892,8 @@ size_t Graph::transpose_0213(size_t a) {
 }
 
 // Graph::gather (src/graph/ops/transform.rs:132-324).  Indices are a tensor of f32 ids loaded from
-// the host (`as usize` truncation, :294); their host copy drives the deterministic backward.
+// the host (`as usize` truncation, :294); the host copy is checked against the vocabulary here, the int32 copy on the
+// device feeds the gather and the deterministic backward scatter.
 size_t Graph::gather(size_t weights, size_t indices) {
     const std::vector<size_t> sw = at(weights).shape;
     if (sw.size() != 2) throw Error("gather: weights must be [vocab, hidden]");
@@ -913,11 +914,12 @@ size_t Graph::gather(size_t weights, size_t indices) {
     const Storage dw = compute_data(weights);
     std::vector<size_t> os = at(indices).shape;
     os.push_back(hidden);
+    // the ids as int32 on the device: a pooled tensor, so that the backward pass finds them there and they leave with
+    // the activations
+    const size_t dids = push_tensor({n}, EISEN_F32, true);  // int32 payload
     const size_t out = push_tensor(os, dw.dtype, true);
-    Storage dids = device_alloc(n, EISEN_F32, false);  // int32 payload
-    check(eisen_hip_htod(ctx_, dids.ptr, ids.data(), n * sizeof(int32_t)), "gather ids");
-    check(eisen_hip_gather(ctx_, dw.ptr, (const int32_t*)dids.ptr, at(out).data.ptr, dw.dtype, n, vocab, hidden), "gather");
-    device_free(dids);
+    check(eisen_hip_htod(ctx_, at(dids).data.ptr, ids.data(), n * sizeof(int32_t)), "gather ids");
+    check(eisen_hip_gather(ctx_, dw.ptr, (const int32_t*)at(dids).data.ptr, at(out).data.ptr, dw.dtype, n, vocab, hidden), "gather");
     record({weights, indices}, out, [=](Graph& g) {
         const Storage& go = g.grad_for_read(out);
         g.materialize_grad(weights);  // the scatter touches only the rows that occur
@@ -928,7 +930,8 @@ size_t Graph::gather(size_t weights, size_t indices) {
             if (!acc) g.check(eisen_hip_memset_zero(g.ctx(), gw0.ptr, gw0.numel * (gw0.dtype == EISEN_BF16 ? 2 : 4)), "gather backward");
         }
         if (w.grad.dtype != EISEN_F32) throw Error("gather backward: the embedding gradient must be f32");
-        g.check(eisen_hip_gather_backward(g.ctx(), ids.data(), go.ptr, (float*)w.grad.ptr, go.dtype, n, vocab, hidden), "gather backward");
+        g.check(eisen_hip_gather_backward_dev(g.ctx(), (const int32_t*)g.at(dids).data.ptr, go.ptr, (float*)w.grad.ptr, go.dtype, n, vocab, hidden),
+                "gather backward");
     });
     return out;
 }

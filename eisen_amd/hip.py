@@ -369,6 +369,10 @@ class Context:
         ids_host = np.ascontiguousarray(ids_host, dtype=np.int32).reshape(-1)
         self._call("eisen_hip_gather_backward", ids_host.ctypes.data_as(_vp), _ptr(go), _ptr(gw), _i(dtype), _sz(ids_host.size), _sz(vocab), _sz(hidden))
 
+    def gather_backward_dev(self, ids_dev, go, gw, dtype, n_ids, vocab, hidden):
+        """The scatter with int32 ids already on the device."""
+        self._call("eisen_hip_gather_backward_dev", _ptr(ids_dev), _ptr(go), _ptr(gw), _i(dtype), _sz(n_ids), _sz(vocab), _sz(hidden))
+
     # ---- loss -------------------------------------------------------------------------
     def cross_entropy(self, logits, targets, dlogits, row_loss, loss_out, dtype, rows, classes, normalizer, grad_scale=1.0,
                       argmax_out=None, target_logit_out=None):

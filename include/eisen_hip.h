@@ -333,9 +333,17 @@ int eisen_hip_gather(eisen_ctx* ctx, const void* weight, const int32_t* ids, voi
  * kernels/ops_f32.cu:526-537).  gw[ids[i], :] += go[i, :], every row receiving its addends
  * in ascending i exactly like the CPU arm (src/graph/ops/transform.rs:306-315).
  * `ids_host` is the host copy of the ids (they originate on the host in every caller,
- * examples/train_llm.rs:433-435); the call builds a stable position index from it. */
+ * examples/train_llm.rs:433-435); the call checks them, uploads them and indexes them on the device where
+ * eisen_hip_gather_backward_dev can, otherwise it builds the stable position index on the host. */
 int eisen_hip_gather_backward(eisen_ctx* ctx, const int32_t* ids_host, const void* go, float* gw, int dtype,
                               size_t n_ids, size_t vocab, size_t hidden);
+/* The same scatter with the ids already on the device (the int32 buffer eisen_hip_gather read): nothing is sorted or
+ * uploaded by the host.  Up to 16384 ids with vocab * next_pow2(n_ids) < 2^32 are indexed by one workgroup (a stable
+ * sort of the positions by id in LDS) and scattered run by run; other shapes read the ids back (which synchronises)
+ * and take eisen_hip_gather_backward.  The ids must lie in [0, vocab), as they did for the gather; an id outside is
+ * skipped on the device route. */
+int eisen_hip_gather_backward_dev(eisen_ctx* ctx, const int32_t* ids_dev, const void* go, float* gw, int dtype,
+                                  size_t n_ids, size_t vocab, size_t hidden);
 
 /* ---- loss ------------------------------------------------------------------------------ */
 

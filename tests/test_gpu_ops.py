@@ -407,6 +407,34 @@ def test_gather_and_deterministic_scatter(ctx, dtype):
     assert np.array_equal(dn(ctx, gw, (vocab, hidden), F32), exp)
     with pytest.raises(hip.EisenHipError):
         ctx.gather_backward(np.array([0, 999], np.int32), dgo, gw, dtype, vocab, hidden)
+    # the same scatter from ids that are already on the device: same bits
+    gw2 = ctx.upload(gw0)
+    ctx.gather_backward_dev(dids, dgo, gw2, dtype, n, vocab, hidden)
+    assert np.array_equal(dn(ctx, gw2, (vocab, hidden), F32), exp)
+
+
+@pytest.mark.parametrize("n,vocab,hidden", [(1, 16, 8), (2, 16, 64), (4096, 32000, 128), (16384, 600, 64), (16385, 600, 64), (3000, 3_000_000, 8), (777, 512, 20), (777, 512, 21)])
+def test_scatter_index_on_device_and_on_host(ctx, n, vocab, hidden):
+    # up to 16384 ids are indexed on the device (one workgroup's stable sort by id); 16385 ids, a vocabulary whose keys
+    # do not fit 32 bits and rows of odd length take the host-built index; both entry points, the same bits
+    ids = gen.zipf_ids(40 + n % 7, (n,), min(vocab, 5000)).astype(np.int32)
+    ids[0] = vocab - 1
+    go = prep(gen.normal(41, (n, hidden)), BF16)
+    gw0 = np.zeros((vocab, hidden), np.float32)
+    gw0[: min(vocab, 5000)] = gen.normal(42, (min(vocab, 5000), hidden))
+    exp = R.gather_bwd(ids.astype(np.float32), go, vocab, gw0.copy())
+    dids, dgo = ctx.upload(ids), up(ctx, go, BF16)
+    for entry in ("host ids", "device ids"):
+        gw = ctx.upload(gw0)
+        if entry == "host ids":
+            ctx.gather_backward(ids, dgo, gw, BF16, vocab, hidden)
+        else:
+            ctx.gather_backward_dev(dids, dgo, gw, BF16, n, vocab, hidden)
+        got = dn(ctx, gw, (vocab, hidden), F32)
+        assert np.array_equal(got, exp), entry
+        gw.free()
+    for b in (dids, dgo):
+        b.free()
 
 
 # ---------------------------------------------------------------------------
