@@ -223,13 +223,16 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
     if (g.ngroup > 0) {  // which product this tile belongs to (uniform); static indices keep the tables in scalar registers
         const int t = blockIdx.x;
         int first = 0;
+        long long partial_off = g.grp_partial_off[0];
         g.A = g.grp_A[0]; g.B = g.grp_B[0]; g.C = g.grp_C[0]; g.N = g.grp_N[0];
 #pragma unroll
         for (int q = 1; q < kMaxGroup; q++)
             if (q < g.ngroup && t >= g.grp_tile_end[q - 1]) {
                 first = g.grp_tile_end[q - 1];
+                partial_off = g.grp_partial_off[q];
                 g.A = g.grp_A[q]; g.B = g.grp_B[q]; g.C = g.grp_C[q]; g.N = g.grp_N[q];
             }
+        if (g.split > 1) g.partial += partial_off;
         const int n_tiles = g.N / BN;
         mt = (t - first) / n_tiles;
         nt = (t - first) % n_tiles;
@@ -574,6 +577,31 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmArgs g, int
     }
 #pragma unroll
     for (int i = 0; i < 4; i++) dst[i] = from_f32<TC>(sum[i]);
+}
+
+// The same for a grouped launch: blockIdx.y is the product (f32 results, no batch).
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_grouped_kernel(GemmArgs g) {
+    const int p = blockIdx.y;
+    const int N = g.grp_N[p];
+    const long long per = (long long)g.M * N, quads = per / 4;
+    const long long q = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (q >= quads) return;
+    float* dst = static_cast<float*>(g.grp_C[p]) + q * 4;
+    float4 sum = *reinterpret_cast<const float4*>(dst);  // part 0 already went into C (assigned or accumulated)
+    const float* part0 = g.partial + g.grp_partial_off[p] + q * 4;
+    for (int p0 = 0; p0 < g.split - 1; p0 += 8) {
+        float4 x[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            x[i] = p0 + i < g.split - 1 ? *reinterpret_cast<const float4*>(part0 + (long long)(p0 + i) * per) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (p0 + i < g.split - 1) {
+                sum.x += x[i].x; sum.y += x[i].y; sum.z += x[i].z; sum.w += x[i].w;
+            }
+        }
+    }
+    *reinterpret_cast<float4*>(dst) = sum;
 }
 
 // ---- generic kernel (f32, or bf16 with shapes the MFMA kernel does not take) ---------------
@@ -1009,6 +1037,56 @@ extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* cons
         else gemm_mfma_direct_kernel<128, 128, 32, 2, 2, false, false, float, false><<<dim3((unsigned)end, 1, 1), 256, 0, ctx->stream>>>(g);
         EISEN_LAUNCH_CHECK(ctx, "eisen_hip_gemm_grouped");
         return 0;
+    }
+    // Few tiles and a long contraction (the weight gradients of a narrow model: 256 x 64 ... 256 x 1024 over thousands of
+    // tokens): one launch of 64 x 64 tiles over every product and every part of a split contraction, then one launch
+    // that adds each product's partial results in part order.  Instead of a GEMM and a reduction per product.
+    bool small = n >= 2 && dtype_ab == EISEN_BF16 && dtype_c == EISEN_F32 && trans_a && !trans_b && M % 64 == 0 && K % 32 == 0 && K >= 1024 &&
+                 M < (size_t(1) << 30) && K < (size_t(1) << 30);
+    long long tiles64 = 0, out_elems = 0;
+    size_t max_n = 0;
+    for (size_t p = 0; p < n && small; p++) {
+        small = A[p] && B[p] && C[p] && N[p] > 0 && N[p] % 64 == 0 && N[p] < (size_t(1) << 30) && eisen_aligned(A[p], 16) && eisen_aligned(B[p], 16) &&
+                eisen_aligned(C[p], 16);
+        tiles64 += (long long)(M / 64) * (long long)(N[p] / 64);
+        out_elems += (long long)M * (long long)N[p];
+        max_n = std::max(max_n, N[p]);
+    }
+    if (small && tiles64 <= 512) {
+        int split = 1;
+        while (split < 32 && tiles64 * split < 1024 && K % ((size_t)split * 2 * 32) == 0 && K / ((size_t)split * 2) >= 256) split *= 2;
+        if (split > 1) {
+            void* ws = nullptr;
+            int rc = eisen_workspace(ctx, (size_t)(split - 1) * (size_t)out_elems * sizeof(float), &ws);
+            if (rc) return rc;
+            GemmArgs g{};
+            g.M = (int)M; g.K = (int)K;
+            g.lda = (int)M;
+            g.accumulate = accumulate;
+            g.vec_c = 1;
+            g.ngroup = (int)n;
+            g.split = split;
+            g.k_part = (int)(K / split);
+            g.partial = static_cast<float*>(ws);
+            int end = 0;
+            long long off = 0;
+            double flops = 0.0;
+            for (size_t p = 0; p < n; p++) {
+                g.grp_A[p] = A[p]; g.grp_B[p] = B[p]; g.grp_C[p] = C[p];
+                g.grp_N[p] = (int)N[p];
+                end += (int)((M / 64) * (N[p] / 64));
+                g.grp_tile_end[p] = end;
+                g.grp_partial_off[p] = off;
+                off += (long long)(split - 1) * (long long)M * (long long)N[p];
+                flops += 2.0 * (double)M * (double)N[p] * (double)K;
+            }
+            EisenProfScope prof(ctx, "gemm_tn_bf16_f32out_64x64x32_grouped_splitk", flops, true);
+            gemm_mfma_direct_kernel<64, 64, 32, 1, 1, false, false, float, false><<<dim3((unsigned)end, 1, (unsigned)split), 64, 0, ctx->stream>>>(g);
+            const unsigned blocks = (unsigned)eisen_ceil_div((size_t)M * max_n / 4, (size_t)256);
+            gemm_splitk_reduce_grouped_kernel<<<dim3(blocks, (unsigned)n, 1), 256, 0, ctx->stream>>>(g);
+            EISEN_LAUNCH_CHECK(ctx, "eisen_hip_gemm_grouped");
+            return 0;
+        }
     }
     for (size_t p = 0; p < n; p++) {
         const int rc = gemm_common(ctx, A[p], B[p], C[p], dtype_ab, dtype_c, trans_a, trans_b, M, N[p], K, 1, 0, 0, 0, accumulate, "eisen_hip_gemm_grouped");

@@ -32,6 +32,7 @@ struct GemmArgs {
     void* grp_C[kMaxGroup];
     int grp_N[kMaxGroup];
     int grp_tile_end[kMaxGroup];
+    long long grp_partial_off[kMaxGroup];  // grouped launch with split > 1: where product p's partial results start inside `partial`
     int tile_group;                    // direct kernel: > 0 = N tiles per group of the tile order (see the kernel), 0 = row-major order
     int vec_c;                         // C rows are 16-byte aligned at every 8th column: the epilogue may use 16-byte accesses
     // K made of up to three segments with their own operands, C (+)= sum_s op(A_s) op(B_s): segment 0 is A/B/lda/ldb,

@@ -242,13 +242,21 @@ void Graph::flush_norm_dw(bool compute) {
         std::vector<const float*> parts;
         std::vector<float*> gws;
         std::vector<size_t> nrows;
+        std::vector<int> assign;
         for (const PendingNormDW& e : list) {
-            if (e.nrows == 0) continue;
+            if (e.nrows == 0) {
+                if (e.assign) at(e.weight).grad_zero_pending = true;  // nothing was added: the clearing is still owed
+                continue;
+            }
             parts.push_back((const float*)e.partial.ptr);
             gws.push_back((float*)at(e.weight).grad.ptr);
             nrows.push_back(e.nrows);
+            assign.push_back(e.assign ? 1 : 0);
         }
-        if (!parts.empty()) rc = eisen_hip_rms_norm_dw_finish(ctx_, parts.size(), parts.data(), gws.data(), nrows.data(), list[0].dim);
+        if (!parts.empty()) rc = eisen_hip_rms_norm_dw_finish(ctx_, parts.size(), parts.data(), gws.data(), nrows.data(), list[0].dim, assign.data());
+    } else {
+        for (const PendingNormDW& e : list)
+            if (e.assign) at(e.weight).grad_zero_pending = true;
     }
     for (PendingNormDW& e : list) device_free(e.partial);
     check(rc, "rms_norm gain gradients");
@@ -642,6 +650,8 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
                 params = params && g.at(ws[i]).is_param && N[i] % 128 == 0 && g.at(ws[i]).grad.dtype == EISEN_F32;
                 wide_tiles += (K / 256) * (N[i] / 128);
             }
+            // (a narrow model's gate and up gradients stay here as well: joining the Q/K/V group's split-contraction launch
+            // measured 8 % slower on the config-4 step than the batched pair)
             if (params && wide_tiles >= 300) {
                 for (size_t i = 0; i < n; i++) g.pending_dw.push_back(PendingDW{ws[i], xa.ptr, g.grad_for_read(outs[i]).ptr, M, K, N[i]});
                 return;
@@ -982,15 +992,17 @@ size_t Graph::rms_norm(size_t x, size_t w, float eps) {
         const Storage& go = g.grad_for_read(out);
         int acc = 0;
         Storage& gx = g.grad_for_write(x, &acc);
-        g.materialize_grad(w);
         Tensor& tw = g.at(w);
+        if (!tw.is_param) g.materialize_grad(w);
         if (!tw.grad.valid() || tw.grad.dtype != EISEN_F32) throw Error("rms_norm backward: the gain needs an f32 gradient buffer");
         if (tw.is_param) {
             // the gain gradient stays in partial rows until the end of the backward pass (flush_norm_dw)
             bool clash = g.pending_norm_dw.size() >= 64;
             for (const PendingNormDW& e : g.pending_norm_dw) clash = clash || e.weight == w || e.dim != dim;
             if (clash) g.flush_norm_dw(true);
-            PendingNormDW e{g.device_alloc((size_t)EISEN_RMS_NORM_PARTIAL_ROWS * dim, EISEN_F32, false), w, 0, dim};
+            // a gradient still waiting to be cleared (zero_grad is lazy) is overwritten by the finishing launch
+            PendingNormDW e{g.device_alloc((size_t)EISEN_RMS_NORM_PARTIAL_ROWS * dim, EISEN_F32, false), w, 0, dim, tw.grad_zero_pending};
+            tw.grad_zero_pending = false;
             const int rc = eisen_hip_rms_norm_backward_partial(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr, (const float*)g.at(rr).data.ptr,
                                                                go.ptr, gx.ptr, (float*)e.partial.ptr, &e.nrows, go.dtype, rows, dim, acc);
             g.pending_norm_dw.push_back(e);  // before the check: the buffer is released with the list

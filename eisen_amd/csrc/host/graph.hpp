@@ -182,6 +182,7 @@ class Graph {
     struct PendingNormDW {
         Storage partial;
         size_t weight, nrows, dim;
+        bool assign;   // the gain's gradient was waiting to be cleared: the finishing launch overwrites it instead
     };
     std::vector<PendingNormDW> pending_norm_dw;
     void flush_norm_dw(bool compute);

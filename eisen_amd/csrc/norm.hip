@@ -167,6 +167,7 @@ struct FinishSlots {
     const float* partial[kFinishSlots];
     float* gw[kFinishSlots];
     int nrows[kFinishSlots];
+    int assign[kFinishSlots];  // 1: gw = sum (a gradient whose clearing is still pending), 0: gw += sum
 };
 __global__ __launch_bounds__(256) void rms_norm_dw_reduce_kernel(FinishSlots slots, int dim) {
     __shared__ float sh[8][32];
@@ -185,7 +186,7 @@ __global__ __launch_bounds__(256) void rms_norm_dw_reduce_kernel(FinishSlots slo
         float t = 0.f;
 #pragma unroll
         for (int k = 0; k < 8; k++) t += sh[k][cl];
-        gw[c] += t;
+        gw[c] = (slots.assign[blockIdx.y] ? 0.f : gw[c]) + t;
     }
 }
 
@@ -316,7 +317,7 @@ int rms_norm_bwd_partial(eisen_ctx* ctx, const void* x, const float* w, const fl
     return 0;
 }
 
-int rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim) {
+int rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim, const int* assign) {
     double bytes = 0.0;
     for (size_t i = 0; i < n; i++) bytes += ((double)nrows[i] + 2.0) * (double)dim * 4.0;
     EisenProfScope prof(ctx, "rms_norm_dw_finish", bytes);
@@ -327,6 +328,7 @@ int rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, fl
             slots.partial[i] = partial[first + i];
             slots.gw[i] = gw[first + i];
             slots.nrows[i] = (int)nrows[first + i];
+            slots.assign[i] = assign ? assign[first + i] : 0;
         }
         rms_norm_dw_reduce_kernel<<<dim3((unsigned)eisen_ceil_div(dim, 32), (unsigned)m, 1), 256, 0, ctx->stream>>>(slots, (int)dim);
         EISEN_LAUNCH_CHECK(ctx, "rms_norm_dw_reduce_kernel");
@@ -364,7 +366,7 @@ extern "C" int eisen_hip_rms_norm_backward(eisen_ctx* ctx, const void* x, const 
                             : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx, (float*)ws, &nrows, rows, dim, accumulate_x);
     if (rc) return rc;
     const float* p = (const float*)ws;
-    return rms_norm_dw_finish(ctx, 1, &p, &gw, &nrows, dim);
+    return rms_norm_dw_finish(ctx, 1, &p, &gw, &nrows, dim, nullptr);
 }
 
 extern "C" int eisen_hip_rms_norm_backward_partial(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx,
@@ -379,7 +381,8 @@ extern "C" int eisen_hip_rms_norm_backward_partial(eisen_ctx* ctx, const void* x
                               : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx, partial, nrows_out, rows, dim, accumulate_x);
 }
 
-extern "C" int eisen_hip_rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim) {
+extern "C" int eisen_hip_rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim,
+                                            const int* assign) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, n == 0 || (partial && gw && nrows), EISEN_E_ARG, "eisen_hip_rms_norm_dw_finish: null pointer");
     EISEN_REQUIRE(ctx, dim > 0 && dim < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_rms_norm_dw_finish: dim %zu out of range", dim);
@@ -387,7 +390,7 @@ extern "C" int eisen_hip_rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const floa
         EISEN_REQUIRE(ctx, partial[i] && gw[i] && nrows[i] <= kMaxPartialRows, EISEN_E_ARG, "eisen_hip_rms_norm_dw_finish: entry %zu is null or has too many rows", i);
         for (size_t j = 0; j < i; j++) EISEN_REQUIRE(ctx, gw[i] != gw[j], EISEN_E_ARG, "eisen_hip_rms_norm_dw_finish: entries %zu and %zu add to the same gradient", j, i);
     }
-    return rms_norm_dw_finish(ctx, n, partial, gw, nrows, dim);
+    return rms_norm_dw_finish(ctx, n, partial, gw, nrows, dim, assign);
 }
 
 extern "C" int eisen_hip_softmax(eisen_ctx* ctx, const void* x, void* out, int dtype, size_t rows, size_t n) {

@@ -257,13 +257,14 @@ class Context:
                    _sz(rows), _sz(dim), _i(accumulate_x))
         return n.value
 
-    def rms_norm_dw_finish(self, partials, gws, nrows, dim):
-        """gw_i += column sums of the first nrows_i rows of partial_i, all in one launch."""
+    def rms_norm_dw_finish(self, partials, gws, nrows, dim, assign=None):
+        """gw_i (+)= column sums of the first nrows_i rows of partial_i, all in one launch; assign[i]: overwrite gw_i."""
         n = len(partials)
         pp = (_vp * n)(*[_ptr(p) for p in partials])
         pg = (_vp * n)(*[_ptr(g) for g in gws])
         pn = (C.c_size_t * n)(*nrows)
-        self._call("eisen_hip_rms_norm_dw_finish", _sz(n), pp, pg, pn, _sz(dim))
+        pa = None if assign is None else (C.c_int * n)(*[int(a) for a in assign])
+        self._call("eisen_hip_rms_norm_dw_finish", _sz(n), pp, pg, pn, _sz(dim), pa)
 
     def rope(self, x, out, dtype, batch, seq, hidden, head_dim):
         self._call("eisen_hip_rope", _ptr(x), _ptr(out), _i(dtype), _sz(batch), _sz(seq), _sz(hidden), _sz(head_dim))

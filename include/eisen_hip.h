@@ -187,12 +187,14 @@ int eisen_hip_rms_norm_backward(eisen_ctx* ctx, const void* x, const float* w, c
 /* eisen_hip_rms_norm_backward in two parts, for a caller with many norms (a transformer block has two): `_partial`
  * writes dx and leaves the gain gradient as *nrows_out rows of per-workgroup column sums in `partial`
  * ([EISEN_RMS_NORM_PARTIAL_ROWS][dim] f32, caller's buffer); `_finish` adds the rows of n such buffers to their
- * gain gradients (gw_i += column sums of partial_i, fixed order, distinct gw_i) in one launch.  The reference runs
+ * gain gradients (gw_i += column sums of partial_i, fixed order, distinct gw_i) in one launch; where assign[i] != 0
+ * (assign may be NULL) gw_i is overwritten instead, for a gradient whose clearing is still pending.  The reference runs
  * one rmsnorm_backward_f32 per norm (src/graph/ops/normalization.rs:157-171). */
 #define EISEN_RMS_NORM_PARTIAL_ROWS 256
 int eisen_hip_rms_norm_backward_partial(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx,
                                         float* partial, size_t* nrows_out, int dtype, size_t rows, size_t dim, int accumulate_x);
-int eisen_hip_rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim);
+int eisen_hip_rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim,
+                                 const int* assign);
 /* rope_f32 / rope_backward_f32 (kernels/ops_f32.cu:724-760; Graph::rope,
  * src/graph/ops/transform.rs:467-610): x [batch, seq, hidden], interleaved pairs within each
  * head of `head_dim`, base 10000, position = index along dim 1. */

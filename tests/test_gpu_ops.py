@@ -806,11 +806,12 @@ def test_side_stream_orders_after_fork_and_before_join(ctx):
 
 
 @pytest.mark.parametrize("M,K,Ns", [(2048, 128, (2048, 512, 512, 2048)), (2048, 192, (1024, 3072)), (256, 64, (128, 256, 128)),
-                                    (2048, 256, (2048, 512, 3072))])
+                                    (2048, 256, (2048, 512, 3072)), (256, 2048, (256, 64, 64, 256, 1024, 1024)), (128, 1024, (64, 192))])
 @pytest.mark.parametrize("accumulate", [0, 1])
 def test_gemm_grouped_weight_gradients(ctx, M, K, Ns, accumulate):
     # dW_p (+)= X_p^T dY_p with X_p [K, M] and dY_p [K, N_p] (here K is the token count): the first two shapes run as one
-    # grid of 128x128 tiles, the third falls back to one launch per product, the last is one grid of 176 tiles of 256x256
+    # grid of 128x128 tiles, the third falls back to one launch per product, the fourth is one grid of 176 tiles of 256x256, the last
+    # two (few 64x64 tiles, long contraction) one grid over products and parts of the contraction plus one reduction
     xs = [prep(gen.normal(550 + i, (K, M)), BF16) for i in range(len(Ns))]
     dys = [prep(gen.normal(560 + i, (K, n)), BF16) for i, n in enumerate(Ns)]
     c0 = [gen.normal(570 + i, (M, n)).astype(np.float32) for i, n in enumerate(Ns)]
