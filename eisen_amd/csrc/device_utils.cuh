@@ -37,6 +37,14 @@ template <typename T> __device__ __forceinline__ Pack<T> load_pack(const T* p) {
 template <typename T> __device__ __forceinline__ void store_pack(T* p, const Pack<T>& v) {
     *reinterpret_cast<Pack<T>*>(p) = v;
 }
+// The same for data that is touched once (non-temporal: not kept in the caches).
+template <typename T> __device__ __forceinline__ Pack<T> load_pack_streaming(const T* p) {
+    const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+    return *reinterpret_cast<const Pack<T>*>(&t);
+}
+template <typename T> __device__ __forceinline__ void store_pack_streaming(T* p, const Pack<T>& v) {
+    __builtin_nontemporal_store(*reinterpret_cast<const f32x4*>(&v), reinterpret_cast<f32x4*>(p));
+}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
