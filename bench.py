@@ -159,7 +159,7 @@ def cpu_baseline_lm(c, seq, mb=1):
 # workloads
 # ---------------------------------------------------------------------------------------------
 
-def bench_lm(name, steps, warmup, with_cpu=True, recompute=False):
+def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True):
     from eisen_amd import graph as G
     from eisen_amd import hip
     c = CONFIGS[name]
@@ -173,6 +173,9 @@ def bench_lm(name, steps, warmup, with_cpu=True, recompute=False):
             g.load_tensor_data(pid, rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02))
     g.mark_params()
     lm.set_checkpointing(recompute)   # per-block recompute: off in the headline run (the reference's train_llm.rs does not use it)
+    # weight gradients over the whole accumulation window in one contraction (Graph::set_weight_gradient_window): the sums
+    # of train_llm.rs:386-477's micro-batch loop, each gradient read and written once per optimizer step
+    g.set_weight_gradient_window(c["accum"] if window and 2 <= c["accum"] <= 8 else 0)
     opt = G.AdamW(g, lm.params(), 1e-3)
     opt.config(1e-3, 0.9, 0.95, 1e-8, 0.1, 1.0)      # train_llm.rs:266-270 + grad clip 1.0
     opt.init_moments()
@@ -333,6 +336,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="all", choices=["all", "c5", "c4", "c3", "c2"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
+    ap.add_argument("--no-window", action="store_true", help="c5: form every micro-batch's weight gradients in its own backward pass, as the reference does, "
+                    "instead of once per optimizer step over the whole accumulation window")
     ap.add_argument("--recompute", action="store_true", help="c5 / c4: per-block recompute (lower activation memory, one more forward pass per block)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -340,11 +345,11 @@ def main():
         sys.exit(2)
     w = args.workload
     if w in ("all", "c5"):
-        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute)
+        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute, not args.no_window)
         if w == "all":
             out["other_configs"] = dict(c4=brief(bench_lm("c4", 20, 3, not args.no_cpu)), c3=brief(bench_c3(20, 3)), c2=brief(bench_c2(20, 3)))
     elif w == "c4":
-        out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute)
+        out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute, not args.no_window)
     elif w == "c3":
         out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3)
     else:

@@ -1095,6 +1095,78 @@ extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* cons
     return 0;
 }
 
+// C_p (+)= sum_s A_ps^T B_ps: the dB += A^T dC of Graph::matmul (src/graph/ops/linear.rs:281-295) for several weights and
+// several micro-batches at once.  One launch of 256 x 256 tiles whose contraction walks through the pieces when every
+// shape is a whole number of tiles; otherwise one accumulating GEMM per product and piece, in piece order.
+static_assert(kMaxWindowSegments == EISEN_GEMM_MAX_KSEGMENTS, "the kernel's table and the header disagree");
+extern "C" int eisen_hip_gemm_grouped_ksegments(eisen_ctx* ctx, size_t n_products, size_t n_segments, const void* const* A, const void* const* B,
+                                                void* const* C, const size_t* M, const size_t* N, size_t seg_k, int accumulate) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, n_products >= 1 && n_segments >= 1 && A && B && C && M && N, EISEN_E_ARG,
+                  "eisen_hip_gemm_grouped_ksegments: at least one product and one piece, no null pointers");
+    EISEN_REQUIRE(ctx, seg_k > 0 && seg_k < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_gemm_grouped_ksegments: piece length %zu out of range", seg_k);
+    for (size_t p = 0; p < n_products; p++) {
+        EISEN_REQUIRE(ctx, C[p] && M[p] > 0 && N[p] > 0 && M[p] < (size_t(1) << 30) && N[p] < (size_t(1) << 30), EISEN_E_ARG,
+                      "eisen_hip_gemm_grouped_ksegments: product %zu has a null result or an empty shape", p);
+        for (size_t s = 0; s < n_segments; s++)
+            EISEN_REQUIRE(ctx, A[p * n_segments + s] && B[p * n_segments + s], EISEN_E_ARG, "eisen_hip_gemm_grouped_ksegments: product %zu piece %zu is null", p, s);
+    }
+    bool one = n_products < (size_t(1) << 16) && n_segments <= (size_t)kMaxWindowSegments && seg_k % 32 == 0;
+    if (one) {
+        std::vector<WideWindowRow> rows(n_products);
+        WideWindow w{};
+        w.nprod = (int)n_products;
+        w.nseg = (int)n_segments;
+        w.seg_slabs = (int)(seg_k / 32);
+        w.accumulate = accumulate;
+        long long tiles = 0;
+        double flops = 0.0;
+        for (size_t p = 0; p < n_products && one; p++) {
+            WideWindowRow& r = rows[p];
+            r.M = (int)M[p];
+            r.N = (int)N[p];
+            r.pad = 0;
+            r.C = C[p];
+            one = eisen_aligned(C[p], 16);
+            for (size_t s = 0; s < (size_t)kMaxWindowSegments; s++) {
+                const size_t from = p * n_segments + std::min(s, n_segments - 1);
+                r.A[s] = A[from];
+                r.B[s] = B[from];
+                one = one && eisen_aligned(A[from], 16) && eisen_aligned(B[from], 16);
+            }
+            tiles += (long long)(M[p] / 256) * (long long)(N[p] / 256);
+            one = one && tiles < (1ll << 30);
+            r.tile_end = (int)tiles;
+            flops += 2.0 * (double)M[p] * (double)N[p] * (double)seg_k * (double)n_segments;
+        }
+        // fewer tiles than CUs would leave most of the chip idle for the whole contraction
+        one = one && tiles >= 176 && eisen_gemm_wide_window_supports(w, rows.data());
+        if (one) {
+            void* table = nullptr;
+            int rc = eisen_hip_malloc(ctx, rows.size() * sizeof(WideWindowRow), &table);
+            if (rc) return rc;
+            rc = eisen_hip_htod(ctx, table, rows.data(), rows.size() * sizeof(WideWindowRow));
+            if (!rc) {
+                w.rows = static_cast<const WideWindowRow*>(table);
+                EisenProfScope prof(ctx, "gemm_tn_bf16_f32out_256x256x32_window", flops, true);
+                eisen_gemm_launch_wide_window(ctx, w, (unsigned)tiles);
+            }
+            const int rc_free = eisen_hip_free(ctx, table);  // stream-ordered: reused only by later work
+            if (rc) return rc;
+            if (rc_free) return rc_free;
+            EISEN_LAUNCH_CHECK(ctx, "eisen_hip_gemm_grouped_ksegments");
+            return 0;
+        }
+    }
+    for (size_t p = 0; p < n_products; p++)
+        for (size_t s = 0; s < n_segments; s++) {
+            const int rc = gemm_common(ctx, A[p * n_segments + s], B[p * n_segments + s], C[p], EISEN_BF16, EISEN_F32, 1, 0, M[p], N[p], seg_k, 1, 0, 0, 0,
+                                       s == 0 ? accumulate : 1, "eisen_hip_gemm_grouped_ksegments");
+            if (rc) return rc;
+        }
+    return 0;
+}
+
 extern "C" int eisen_hip_gemm_swiglu_backward(eisen_ctx* ctx, const void* A, const void* B, const void* gate, const void* up, void* dgate,
                                               void* dup, int dtype, int trans_a, int trans_b, size_t M, size_t N, size_t K) {
     EISEN_CHECK_CTX(ctx);

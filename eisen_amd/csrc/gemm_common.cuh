@@ -1,6 +1,7 @@
 // Pieces shared by the GEMM kernels of gemm.hip and gemm_wide.hip: the launch argument block, the operand tiles
 // filled by direct-to-LDS loads, and the epilogue that stores a wave's accumulators.
 #pragma once
+#include <type_traits>
 #include <utility>
 
 #include "device_utils.cuh"
@@ -47,6 +48,29 @@ struct GemmArgs {
 // gemm_wide.hip: 256 x 256 tiles, four waves of 128 x 128 (plain products, whole tiles only)
 bool eisen_gemm_wide_supports(const GemmArgs& g, bool a_kc, bool b_kc, int batch, int dtype_c);
 void eisen_gemm_launch_wide(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b_kc, int dtype_c);
+
+// One launch of gemm_wide.hip's kernel over any number of products whose contraction is stored in several pieces:
+// C_p (+)= sum_s A_ps^T B_ps with A_ps bf16 [seg_k][M_p], B_ps bf16 [seg_k][N_p], C_p f32 [M_p][N_p] (the weight gradients
+// of the Linear layers of a model over several micro-batches, each micro-batch's activations and output gradients where
+// its forward and backward pass left them).  The products are described by a table in device memory.
+constexpr int kMaxWindowSegments = 8;
+struct WideWindowRow {
+    int M, N;
+    int tile_end;  // number of 256 x 256 tiles of products 0..p
+    int pad;
+    void* C;
+    const void* A[kMaxWindowSegments];  // entries from nseg on repeat the last piece
+    const void* B[kMaxWindowSegments];
+};
+struct WideWindow {
+    int nprod, nseg;
+    int seg_slabs;  // 32-deep slabs per piece, a multiple of 4
+    int accumulate;
+    const WideWindowRow* rows;  // device memory, nprod entries
+};
+// the host's copy of the table: shapes the kernel takes?
+bool eisen_gemm_wide_window_supports(const WideWindow& w, const WideWindowRow* host_rows);
+void eisen_gemm_launch_wide_window(eisen_ctx* ctx, const WideWindow& w, unsigned tiles);
 
 namespace {
 

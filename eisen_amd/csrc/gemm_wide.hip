@@ -23,8 +23,20 @@ __device__ __forceinline__ void wide_load_lds_16(const void* sbase, unsigned vof
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "m0");
 }
 
-template <bool A_KC, bool B_KC, typename TC>
-__global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g) {
+struct NoWindow {};
+
+// a pointer every lane holds the same value of, moved to scalar registers
+template <typename T>
+__device__ __forceinline__ T* uniform_pointer(T* p) {
+    const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return reinterpret_cast<T*>(((unsigned long long)hi << 32) | lo);
+}
+
+// WIN: the products, their shapes and the pieces of their contraction come from `w` (see WideWindow); g carries the
+// flags of the epilogue only.
+template <bool A_KC, bool B_KC, typename TC, bool WIN>
+__global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, std::conditional_t<WIN, WideWindow, NoWindow> w) {
     constexpr int TM = 4, TN = 4, WM = 128, WN = 128;
     using TA = DirectOperandTile<WBM, A_KC, WBK, WWAVES>;
     using TB = DirectOperandTile<WBN, B_KC, WBK, WWAVES>;
@@ -38,7 +50,25 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g) {
 
     // which tile (and, in a grouped launch, of which product)
     int t = blockIdx.x, mt, nt;
-    if (g.ngroup > 0) {
+    int prod = 0;
+    if constexpr (WIN) {
+        // the first product whose tiles end after t (the table is the same for every lane: scalar loads)
+        int lo = 0, hi = w.nprod - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (t >= __builtin_amdgcn_readfirstlane(w.rows[mid].tile_end)) lo = mid + 1;
+            else hi = mid;
+        }
+        prod = lo;
+        if (prod > 0) t -= __builtin_amdgcn_readfirstlane(w.rows[prod - 1].tile_end);
+        const WideWindowRow& row = w.rows[prod];
+        g.M = __builtin_amdgcn_readfirstlane(row.M); g.N = __builtin_amdgcn_readfirstlane(row.N);
+        g.C = uniform_pointer(row.C);
+        g.A = uniform_pointer(row.A[0]); g.B = uniform_pointer(row.B[0]);
+        g.lda = g.M; g.ldb = g.N; g.ldc = g.N;
+        g.K = w.nseg * w.seg_slabs * WBK;
+        g.tile_group = g.N / WBN >= 32 ? 16 : 0;
+    } else if (g.ngroup > 0) {
         int first = 0;
         g.A = g.grp_A[0]; g.B = g.grp_B[0]; g.C = g.grp_C[0]; g.N = g.grp_N[0];
 #pragma unroll
@@ -72,8 +102,22 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g) {
 
     // slab origin and per-slab advance of each operand (uniform), this lane's byte offsets inside a slab (the same
     // for every slab)
-    const char* a_base = reinterpret_cast<const char*>(A_KC ? A + (long long)m0 * g.lda : A + m0);
-    const char* b_base = reinterpret_cast<const char*>(B_KC ? B + (long long)n0 * g.ldb : B + n0);
+    const long long a_tile = (A_KC ? (long long)m0 * g.lda : (long long)m0) * 2;  // bytes from the operand's first element
+    const long long b_tile = (B_KC ? (long long)n0 * g.ldb : (long long)n0) * 2;
+    const char* a_base = reinterpret_cast<const char*>(A) + a_tile;
+    const char* b_base = reinterpret_cast<const char*>(B) + b_tile;
+    // WIN: where the tile's slabs start in the pieces after the first, in the order they will be needed
+    const char* a_seg[kMaxWindowSegments - 1];
+    const char* b_seg[kMaxWindowSegments - 1];
+    int seg_left = 0;  // slabs of the current piece not yet requested
+    if constexpr (WIN) {
+#pragma unroll
+        for (int s = 1; s < kMaxWindowSegments; s++) {
+            a_seg[s - 1] = static_cast<const char*>(uniform_pointer(w.rows[prod].A[s])) + a_tile;
+            b_seg[s - 1] = static_cast<const char*>(uniform_pointer(w.rows[prod].B[s])) + b_tile;
+        }
+        seg_left = w.seg_slabs - (WSTAGES - 1);
+    }
     const long long a_step = A_KC ? (long long)WBK * 2 : (long long)WBK * g.lda * 2;
     const long long b_step = B_KC ? (long long)WBK * 2 : (long long)WBK * g.ldb * 2;
     unsigned a_off[LA], b_off[LB];
@@ -175,8 +219,27 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g) {
             __builtin_amdgcn_sched_barrier(0);
         });
         to_issue--;
-        a_next += to_issue > 0 ? a_step : 0;
-        b_next += to_issue > 0 ? b_step : 0;
+        if constexpr (WIN) {
+            seg_left--;
+            if (to_issue > 0) {
+                if (seg_left == 0) {  // the next slab is the first of the next piece
+                    seg_left = w.seg_slabs;
+                    a_next = a_seg[0];
+                    b_next = b_seg[0];
+#pragma unroll
+                    for (int s = 0; s + 1 < kMaxWindowSegments - 1; s++) {
+                        a_seg[s] = a_seg[s + 1];
+                        b_seg[s] = b_seg[s + 1];
+                    }
+                } else {
+                    a_next += a_step;
+                    b_next += b_step;
+                }
+            }
+        } else {
+            a_next += to_issue > 0 ? a_step : 0;
+            b_next += to_issue > 0 ? b_step : 0;
+        }
     };
     static_assert(WSTAGES == 4, "the ring below is written out for four stages");
     for (int ring = 0; ring < nk / WSTAGES; ring++) {  // K is a whole number of rings (checked by the launcher)
@@ -215,7 +278,7 @@ void eisen_gemm_launch_wide(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b
     unsigned tiles;
     if (g.ngroup > 0) tiles = (unsigned)g.grp_tile_end[g.ngroup - 1];
     else tiles = (unsigned)((g.M / WBM) * (g.N / WBN));
-#define EISEN_WIDE(AK, BKC, TC) gemm_wide_kernel<AK, BKC, TC><<<dim3(tiles, 1, 1), 256, 0, ctx->stream>>>(g)
+#define EISEN_WIDE(AK, BKC, TC) gemm_wide_kernel<AK, BKC, TC, false><<<dim3(tiles, 1, 1), 256, 0, ctx->stream>>>(g, NoWindow{})
     if (dtype_c == EISEN_BF16) {
         if (a_kc && b_kc) EISEN_WIDE(true, true, bf16_t);
         else if (a_kc) EISEN_WIDE(true, false, bf16_t);
@@ -228,4 +291,24 @@ void eisen_gemm_launch_wide(eisen_ctx* ctx, const GemmArgs& g, bool a_kc, bool b
         else EISEN_WIDE(false, false, float);
     }
 #undef EISEN_WIDE
+}
+
+bool eisen_gemm_wide_window_supports(const WideWindow& w, const WideWindowRow* host_rows) {
+    if (w.nprod < 1 || w.nseg < 1 || w.nseg > kMaxWindowSegments) return false;
+    if (w.seg_slabs < WSTAGES || w.seg_slabs % WSTAGES) return false;
+    if ((long long)w.nseg * w.seg_slabs * WBK >= (1ll << 31)) return false;
+    for (int p = 0; p < w.nprod; p++) {
+        const WideWindowRow& r = host_rows[p];
+        if (r.M <= 0 || r.N <= 0 || r.M % WBM || r.N % WBN) return false;
+        // a lane's offset inside a slab is a 32-bit number of bytes
+        if ((long long)WBK * r.M * 2 >= (1ll << 31) || (long long)WBK * r.N * 2 >= (1ll << 31)) return false;
+    }
+    return true;
+}
+
+void eisen_gemm_launch_wide_window(eisen_ctx* ctx, const WideWindow& w, unsigned tiles) {
+    GemmArgs g{};
+    g.accumulate = w.accumulate;
+    g.vec_c = 1;
+    gemm_wide_kernel<false, false, float, true><<<dim3(tiles, 1, 1), 256, 0, ctx->stream>>>(g, w);
 }

@@ -91,6 +91,12 @@ int eisen_graph_clear_activations(eisen_graph* g) { return guarded(g, [&](Graph&
 int eisen_graph_reinterpret_shape(eisen_graph* g, size_t id, const size_t* shape, int rank) {
     return guarded(g, [&](Graph& G) { G.reinterpret_shape(id, shape_of(shape, rank)); });
 }
+int eisen_graph_set_weight_gradient_window(eisen_graph* g, size_t backward_passes) {
+    return guarded(g, [&](Graph& G) { G.set_weight_gradient_window(backward_passes); });
+}
+int eisen_graph_flush_weight_gradients(eisen_graph* g) {
+    return guarded(g, [&](Graph& G) { G.flush_weight_gradients(); });
+}
 int eisen_graph_set_no_grad(eisen_graph* g, int v) { return guarded(g, [&](Graph& G) { G.no_grad = v != 0; }); }
 int eisen_graph_num_tensors(eisen_graph* g, size_t* out) { return guarded(g, [&](Graph& G) { need(out, "out"); *out = G.tensors.size(); }); }
 int eisen_graph_num_params(eisen_graph* g, size_t* out) { return guarded(g, [&](Graph& G) { need(out, "out"); *out = G.num_params; }); }

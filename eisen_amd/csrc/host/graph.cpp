@@ -58,6 +58,8 @@ Graph::Graph(eisen_ctx* ctx, PrecisionMode mode) : precision_mode(mode), ctx_(ct
 Graph::~Graph() {
     (void)eisen_hip_side_wait(ctx_);
     for (auto& t : tensors) release(t);
+    for (auto& kv : retained_)
+        if (kv.second) eisen_hip_free(ctx_, const_cast<void*>(kv.first));
 }
 
 void Graph::check(int rc, const char* what) const {
@@ -77,15 +79,25 @@ Storage Graph::device_alloc(size_t numel, int dtype, bool zero) {
     check(zero ? eisen_hip_malloc_zeroed(ctx_, bytes, &s.ptr) : eisen_hip_malloc(ctx_, bytes, &s.ptr), "device allocation");
     return s;
 }
+void Graph::free_buffer(void* ptr) {
+    if (!ptr) return;
+    if (!retained_.empty()) {
+        auto it = retained_.find(ptr);
+        if (it != retained_.end()) {  // a windowed weight-gradient GEMM still has to read it: flush_weight_gradients frees it
+            it->second = true;
+            return;
+        }
+    }
+    check(eisen_hip_free(ctx_, ptr), "device free");
+}
 void Graph::device_free(Storage& s) {
-    if (s.ptr) check(eisen_hip_free(ctx_, s.ptr), "device free");
+    free_buffer(s.ptr);
     s = Storage();
 }
 void Graph::release(Tensor& t) {
-    if (t.data.ptr) eisen_hip_free(ctx_, t.data.ptr);
-    if (t.grad.ptr && !t.grad_borrowed) eisen_hip_free(ctx_, t.grad.ptr);
-    if (t.shadow.ptr) eisen_hip_free(ctx_, t.shadow.ptr);
+    void* const bufs[3] = {t.data.ptr, t.grad_borrowed ? nullptr : t.grad.ptr, t.shadow.ptr};
     t.data = t.grad = t.shadow = Storage();
+    for (void* p : bufs) free_buffer(p);
 }
 
 size_t Graph::push_tensor(const std::vector<size_t>& shape, int dtype, bool pooled) {
@@ -215,11 +227,12 @@ void Graph::record(std::vector<size_t> inputs, size_t output, std::function<void
     tape.nodes.push_back(TapeNode{std::move(inputs), output, std::move(fn)});
 }
 
-Storage& Graph::grad_for_write(size_t id, int* accumulate) {
+Storage& Graph::grad_for_write(size_t id, int* accumulate, const void** add_from) {
     Tensor& t = at(id);
     if (t.is_param) {
         *accumulate = t.grad_zero_pending ? 0 : 1;
         t.grad_zero_pending = false;
+        if (add_from) *add_from = t.grad.ptr;
         return t.grad;
     }
     if (!t.grad.valid()) {
@@ -230,6 +243,17 @@ Storage& Graph::grad_for_write(size_t id, int* accumulate) {
     }
     t.grad_written = true;
     if (!side_guards.empty() && std::find(side_guards.begin(), side_guards.end(), t.grad.ptr) != side_guards.end()) side_join();
+    if (add_from) *add_from = t.grad.ptr;
+    if (!retained_.empty() && retained_.count(t.grad.ptr)) {
+        // The buffer's present content is an operand of a weight-gradient GEMM of the window: the store goes elsewhere.
+        // Whoever else points at the old buffer (the tensor it was handed over from) only keeps it from being freed twice.
+        Storage old = t.grad;
+        t.grad = device_alloc(old.numel, old.dtype, false);
+        if (*accumulate && !add_from)
+            check(eisen_hip_dtod(ctx_, t.grad.ptr, old.ptr, old.numel * (old.dtype == EISEN_BF16 ? 2 : 4)), "gradient copy");
+        if (t.grad_borrowed) t.grad_borrowed = false;  // the fresh buffer is this tensor's own
+        else retained_[old.ptr] = true;                // the tensor owned the old one: the flush frees it
+    }
     return t.grad;
 }
 
@@ -262,6 +286,103 @@ void Graph::flush_norm_dw(bool compute) {
     check(rc, "rms_norm gain gradients");
 }
 
+// ---- weight gradients over a window of micro-batches (see graph.hpp) -----------------------------------------
+
+void Graph::set_weight_gradient_window(size_t backward_passes) {
+    if (backward_passes > (size_t)EISEN_GEMM_MAX_KSEGMENTS) throw Error("set_weight_gradient_window: at most " + std::to_string(EISEN_GEMM_MAX_KSEGMENTS) + " backward passes");
+    flush_weight_gradients();
+    window_ = backward_passes;
+}
+
+// Products the one-launch form of eisen_hip_gemm_grouped_ksegments takes and that are big enough to be worth keeping their
+// operands for: bf16 operands, an f32 parameter gradient of at least 16 whole 256 x 256 tiles, pieces of whole 128 rows.
+bool Graph::window_fits(size_t weight, int dtype, size_t rows, size_t in, size_t out) {
+    if (window_ < 2 || dtype != EISEN_BF16 || rows == 0 || rows % 128 || in % 256 || out % 256 || (in / 256) * (out / 256) < 16) return false;
+    const Tensor& tw = at(weight);
+    return tw.is_param && tw.grad.dtype == EISEN_F32 && tw.size() == in * out;
+}
+
+bool Graph::window_take(size_t weight, const void* x, const void* dy, int dtype, size_t rows, size_t in, size_t out) {
+    if (!window_fits(weight, dtype, rows, in, out)) return false;
+    WindowDW* e = nullptr;
+    for (WindowDW& c : window_dw)
+        if (c.weight == weight) e = &c;
+    if (e && (e->rows != rows || e->x.size() >= (size_t)EISEN_GEMM_MAX_KSEGMENTS)) {  // a piece of another length, or one too many
+        flush_weight_gradients();
+        e = nullptr;
+    }
+    if (!e) {
+        window_dw.push_back(WindowDW{weight, rows, in, out, {}, {}});
+        e = &window_dw.back();
+    }
+    e->x.push_back(x);
+    e->dy.push_back(dy);
+    retained_.emplace(x, false);
+    retained_.emplace(dy, false);
+    return true;
+}
+
+void Graph::flush_weight_gradients() {
+    window_passes_ = 0;
+    if (window_dw.empty() && retained_.empty()) return;
+    std::vector<WindowDW> list;
+    list.swap(window_dw);
+    // One launch per set of products with the same shape, number of pieces and accumulate state (equal tiles, and for a
+    // model of equal blocks a whole number of rounds of the chip); sets of fewer tiles than the chip has CUs share one.
+    struct Launch {
+        size_t in, out, rows, pieces;
+        int acc;
+        std::vector<const WindowDW*> members;
+    };
+    std::vector<Launch> launches;
+    for (const WindowDW& e : list) {
+        int acc = 0;
+        grad_for_write(e.weight, &acc);
+        Launch* l = nullptr;
+        for (Launch& c : launches)
+            if (c.in == e.in && c.out == e.out && c.rows == e.rows && c.pieces == e.x.size() && c.acc == acc) l = &c;
+        if (!l) {
+            launches.push_back(Launch{e.in, e.out, e.rows, e.x.size(), acc, {}});
+            l = &launches.back();
+        }
+        l->members.push_back(&e);
+    }
+    for (size_t i = 0; i < launches.size(); i++) {  // small sets join the first small set they can run with
+        Launch& a = launches[i];
+        if ((a.in / 256) * (a.out / 256) * a.members.size() >= 256) continue;
+        for (size_t j = i + 1; j < launches.size();) {
+            Launch& b = launches[j];
+            if ((b.in / 256) * (b.out / 256) * b.members.size() < 256 && b.rows == a.rows && b.pieces == a.pieces && b.acc == a.acc) {
+                a.members.insert(a.members.end(), b.members.begin(), b.members.end());
+                launches.erase(launches.begin() + (ptrdiff_t)j);
+            } else {
+                j++;
+            }
+        }
+    }
+    int rc = 0;
+    for (const Launch& l : launches) {
+        std::vector<const void*> As, Bs;
+        std::vector<void*> Cs;
+        std::vector<size_t> Ms, Ns;
+        for (const WindowDW* e : l.members) {
+            As.insert(As.end(), e->x.begin(), e->x.end());
+            Bs.insert(Bs.end(), e->dy.begin(), e->dy.end());
+            Cs.push_back(at(e->weight).grad.ptr);
+            Ms.push_back(e->in);
+            Ns.push_back(e->out);
+        }
+        rc = eisen_hip_gemm_grouped_ksegments(ctx_, Cs.size(), l.pieces, As.data(), Bs.data(), Cs.data(), Ms.data(), Ns.data(), l.rows, l.acc);
+        if (rc) break;
+    }
+    // the operands go back to the pool (stream order keeps them intact until the launches above have read them)
+    std::unordered_map<const void*, bool> held;
+    held.swap(retained_);
+    for (auto& kv : held)
+        if (kv.second) (void)eisen_hip_free(ctx_, const_cast<void*>(kv.first));
+    check(rc, "weight gradients of the window");
+}
+
 void Graph::side_join() {
     check(eisen_hip_side_wait(ctx_), "side stream join");
     side_guards.clear();
@@ -275,12 +396,18 @@ const Storage& Graph::grad_for_read(size_t id) {
 }
 
 void Graph::request_zero_grad(size_t id) {
+    if (!window_dw.empty() && at(id).is_param) flush_weight_gradients();  // what the window holds is added first, then cleared with the rest
     Tensor& t = at(id);
     if (t.is_param) t.grad_zero_pending = true;
     else if (t.grad.valid()) check(eisen_hip_memset_zero(ctx_, t.grad.ptr, t.grad.numel * (t.grad.dtype == EISEN_BF16 ? 2 : 4)), "zero_grad");
 }
 
 void Graph::materialize_grad(size_t id) {
+    if (!window_dw.empty() && at(id).is_param) flush_weight_gradients();  // a parameter's gradient is about to be read
+    apply_pending_zero(id);
+}
+
+void Graph::apply_pending_zero(size_t id) {
     Tensor& t = at(id);
     if (t.grad_zero_pending) {
         check(eisen_hip_memset_zero(ctx_, t.grad.ptr, t.grad.numel * sizeof(float)), "zero_grad");
@@ -306,6 +433,7 @@ void Graph::backward(size_t loss_id) {
         pending_dw.clear();
         throw Error("backward: a deferred weight gradient was not collected by a matmul_group");
     }
+    if (!window_dw.empty() && ++window_passes_ >= window_) flush_weight_gradients();
 }
 
 void Graph::backward_nodes_from(size_t first_node) {
@@ -439,6 +567,7 @@ size_t Graph::matmul(size_t a, size_t b) {
         int acc = 0;
         Storage& ga = g.grad_for_write(a, &acc);
         g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc), "matmul backward dA");
+        if (g.window_take(b, g.compute_data(a).ptr, go.ptr, go.dtype, M, K, N)) return;
         Storage& gb = g.grad_for_write(b, &acc);
         g.check(eisen_hip_gemm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul backward dB");
     });
@@ -477,7 +606,9 @@ size_t Graph::matmul_residual(size_t a, size_t b, size_t r, bool defer_dw) {
         }
         Storage& ga = g.grad_for_write(a, &acc);
         g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc), "matmul_residual backward dA");
-        if (defer_dw && go.dtype == EISEN_BF16 && g.at(b).is_param) {
+        if (g.window_take(b, g.compute_data(a).ptr, go.ptr, go.dtype, M, K, N)) {
+            // left for the window's launch; whoever adds to dOut's buffer (now dR's) next gets a fresh one
+        } else if (defer_dw && go.dtype == EISEN_BF16 && g.at(b).is_param) {
             // dOut's buffer (now also dR's) is only added to by nodes that run after the collecting group
             g.pending_dw.push_back(PendingDW{b, g.compute_data(a).ptr, go.ptr, M, K, N});
         } else {
@@ -524,7 +655,8 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r,
             g.check(eisen_hip_accumulate(g.ctx(), gr.ptr, go.ptr, go.dtype, M * N, acc), "swiglu_matmul_residual backward dR");
         }
         // large products only: a small one gains nothing from running beside the chain
-        const bool side = go.dtype == EISEN_BF16 && g.at(b).is_param && K % 256 == 0 && N % 128 == 0 && M % 64 == 0 && (K / 256) * (N / 128) >= 128;
+        const bool windowed = g.window_take(b, g.at(h).data.ptr, go.ptr, go.dtype, M, K, N);
+        const bool side = !windowed && go.dtype == EISEN_BF16 && g.at(b).is_param && K % 256 == 0 && N % 128 == 0 && M % 64 == 0 && (K / 256) * (N / 128) >= 128;
         if (side) {
             // dB beside the input-gradient chain: it reads h and dOut; dOut's buffer (now dR's) is next written by whoever
             // accumulates into dR, and that write waits (grad_for_write)
@@ -551,7 +683,7 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r,
                     "swiglu_matmul_residual backward");
             g.device_free(dh);
         }
-        if (!side) {
+        if (!side && !windowed) {
             Storage& gb = g.grad_for_write(b, &acc);
             g.check(eisen_hip_gemm(g.ctx(), g.at(h).data.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "swiglu_matmul_residual backward dB");
         }
@@ -641,6 +773,26 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
         // dW_i (+)= A^T dY_i.  First choice: every member, and the deferred gradients this group collects, as one grouped
         // launch (same rows, same input width, same accumulate state, f32 gradients).
         const Storage xa = g.compute_data(a);
+        if (all) {
+            // every member joins the window or none: a group split between the window and this pass gains nothing
+            bool fits = true;
+            for (size_t i = 0; i < n; i++) fits = fits && g.window_fits(ws[i], EISEN_BF16, M, K, N[i]);
+            if (fits) {
+                for (size_t i = 0; i < n; i++) g.window_take(ws[i], xa.ptr, g.grad_for_read(outs[i]).ptr, EISEN_BF16, M, K, N[i]);
+                for (size_t e = 0; e < g.pending_dw.size();) {  // gradients this group was to collect (none in a model whose layers all join the window)
+                    const PendingDW p = g.pending_dw[e];
+                    if (std::find(collect_dw.begin(), collect_dw.end(), p.weight) == collect_dw.end()) {
+                        e++;
+                        continue;
+                    }
+                    g.pending_dw.erase(g.pending_dw.begin() + (ptrdiff_t)e);
+                    int acc = 0;
+                    Storage& gw = g.grad_for_write(p.weight, &acc);
+                    g.check(eisen_hip_gemm(g.ctx(), p.x, p.dy, gw.ptr, EISEN_BF16, gw.dtype, 1, 0, p.in, p.out, p.rows, acc), "deferred dW");
+                }
+                return;
+            }
+        }
         if (defer_dw && all && collect_dw.empty()) {
             // only products that the grouped launch takes as wide tiles are worth the wait: small ones are served better by
             // the batched pair below
@@ -932,7 +1084,7 @@ size_t Graph::gather(size_t weights, size_t indices) {
     check(eisen_hip_gather(ctx_, dw.ptr, (const int32_t*)at(dids).data.ptr, at(out).data.ptr, dw.dtype, n, vocab, hidden), "gather");
     record({weights, indices}, out, [=](Graph& g) {
         const Storage& go = g.grad_for_read(out);
-        g.materialize_grad(weights);  // the scatter touches only the rows that occur
+        g.apply_pending_zero(weights);  // the scatter touches only the rows that occur
         Tensor& w = g.at(weights);
         if (!w.is_param) {
             int acc = 0;
@@ -991,9 +1143,10 @@ size_t Graph::rms_norm(size_t x, size_t w, float eps) {
     record({x, w}, out, [=](Graph& g) {
         const Storage& go = g.grad_for_read(out);
         int acc = 0;
-        Storage& gx = g.grad_for_write(x, &acc);
+        const void* add_to = nullptr;  // where the gradient so far is read from: the buffer written, or one that has to stay as it is
+        Storage& gx = g.grad_for_write(x, &acc, &add_to);
         Tensor& tw = g.at(w);
-        if (!tw.is_param) g.materialize_grad(w);
+        if (!tw.is_param) g.apply_pending_zero(w);
         if (!tw.grad.valid() || tw.grad.dtype != EISEN_F32) throw Error("rms_norm backward: the gain needs an f32 gradient buffer");
         if (tw.is_param) {
             // the gain gradient stays in partial rows until the end of the backward pass (flush_norm_dw)
@@ -1003,11 +1156,16 @@ size_t Graph::rms_norm(size_t x, size_t w, float eps) {
             // a gradient still waiting to be cleared (zero_grad is lazy) is overwritten by the finishing launch
             PendingNormDW e{g.device_alloc((size_t)EISEN_RMS_NORM_PARTIAL_ROWS * dim, EISEN_F32, false), w, 0, dim, tw.grad_zero_pending};
             tw.grad_zero_pending = false;
-            const int rc = eisen_hip_rms_norm_backward_partial(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr, (const float*)g.at(rr).data.ptr,
-                                                               go.ptr, gx.ptr, (float*)e.partial.ptr, &e.nrows, go.dtype, rows, dim, acc);
+            const int rc = acc ? eisen_hip_rms_norm_backward_partial_add(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr,
+                                                                         (const float*)g.at(rr).data.ptr, go.ptr, add_to, gx.ptr, (float*)e.partial.ptr,
+                                                                         &e.nrows, go.dtype, rows, dim)
+                               : eisen_hip_rms_norm_backward_partial(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr,
+                                                                     (const float*)g.at(rr).data.ptr, go.ptr, gx.ptr, (float*)e.partial.ptr, &e.nrows,
+                                                                     go.dtype, rows, dim, 0);
             g.pending_norm_dw.push_back(e);  // before the check: the buffer is released with the list
             g.check(rc, "rms_norm backward");
         } else {
+            if (acc && add_to != gx.ptr) g.check(eisen_hip_dtod(g.ctx(), gx.ptr, add_to, gx.numel * (gx.dtype == EISEN_BF16 ? 2 : 4)), "gradient copy");
             g.check(eisen_hip_rms_norm_backward(g.ctx(), g.compute_data(x).ptr, (const float*)tw.data.ptr, (const float*)g.at(rr).data.ptr, go.ptr, gx.ptr,
                                                 (float*)tw.grad.ptr, go.dtype, rows, dim, acc),
                     "rms_norm backward");

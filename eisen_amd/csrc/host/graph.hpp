@@ -12,6 +12,7 @@
 #include <functional>
 #include <stdexcept>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "eisen_hip.h"
@@ -155,11 +156,16 @@ class Graph {
 
     // ---- helpers for optimisers and backward closures -----------------------------------------
     Tensor& at(size_t id);
-    // Gradient buffer of `id` for a store; *accumulate tells the kernel whether to add.
-    Storage& grad_for_write(size_t id, int* accumulate);
+    // Gradient buffer of `id` for a store; *accumulate tells the kernel whether to add.  add_from: a caller that can read
+    // what it adds to from another buffer than the one it writes passes this; it receives that buffer (the returned one
+    // itself unless the gradient's present content has to stay as it is for a weight-gradient GEMM that has not run yet,
+    // see set_weight_gradient_window: then the store goes to a fresh buffer, and a caller without add_from gets the old
+    // content copied there first).
+    Storage& grad_for_write(size_t id, int* accumulate, const void** add_from = nullptr);
     // Gradient as an input (must have been written).
     const Storage& grad_for_read(size_t id);
-    void materialize_grad(size_t id);      // apply a pending zero_grad
+    void materialize_grad(size_t id);      // before a gradient is read: run what the weight-gradient window holds, apply a pending zero_grad
+    void apply_pending_zero(size_t id);    // the pending zero_grad alone (for a store that touches part of the buffer)
     void request_zero_grad(size_t id);     // AdamW::zero_grad, lazily
     const Storage& compute_data(size_t id);   // what kernels read: bf16 shadow for mixed-mode params
     void refresh_shadow(size_t id);           // re-cast the master weight into the bf16 copy
@@ -188,10 +194,37 @@ class Graph {
     void flush_norm_dw(bool compute);
     void side_join();
 
+    // ---- weight gradients over a window of micro-batches ---------------------------------------------------
+    // The reference forms a Linear layer's weight gradient in the backward pass of every micro-batch and adds it to the
+    // f32 gradient (src/graph/ops/linear.rs:279-287; examples/train_llm.rs:386-477 runs 8 such passes per optimizer step).
+    // With a window of n > 1 backward passes the product is left for later instead (bf16 graphs, weights of whole
+    // 256 x 256 tiles): the activations and the output gradient stay where the passes left them -- their buffers outlive
+    // clear_activations, and a gradient buffer that a later node would add to in place is replaced by a fresh one -- and
+    // one launch per group of equally shaped weights contracts over all the micro-batches of the window
+    // (eisen_hip_gemm_grouped_ksegments): each gradient is read and written once per window.  The launches run when
+    // the n-th pass ends, and before anything reads, clears or scales a parameter's gradient; what a caller can observe
+    // is the reference's sum in a different rounding order (one f32 accumulation over all tokens of the window).
+    // The price is memory: the operands of every windowed product of every pass in the window stay allocated.
+    void set_weight_gradient_window(size_t backward_passes);
+    size_t weight_gradient_window() const { return window_; }
+    void flush_weight_gradients();
+    struct WindowDW {
+        size_t weight, rows, in, out;
+        std::vector<const void*> x, dy;  // one pair per piece, in the order the passes ran
+    };
+    std::vector<WindowDW> window_dw;
+
    private:
     eisen_ctx* ctx_;
     size_t backward_root_ = (size_t)-1;
     size_t backward_epoch_ = 0;
+    size_t window_ = 0, window_passes_ = 0;
+    // buffers a windowed weight-gradient GEMM will read -> whether their owner has released them (then the flush frees them)
+    std::unordered_map<const void*, bool> retained_;
+    // the product x^T dy joins the window when it can; false: the caller forms it now
+    bool window_take(size_t weight, const void* x, const void* dy, int dtype, size_t rows, size_t in, size_t out);
+    bool window_fits(size_t weight, int dtype, size_t rows, size_t in, size_t out);
+    void free_buffer(void* ptr);  // eisen_hip_free unless the buffer is retained
     size_t push_tensor(const std::vector<size_t>& shape, int dtype, bool pooled);
     Storage device_alloc(size_t numel, int dtype, bool zero);
     void device_free(Storage& s);

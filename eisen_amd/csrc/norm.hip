@@ -62,9 +62,10 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_fwd_kernel(const T* __re
 template <typename T, int MAXP>
 __global__ __launch_bounds__(kBwdThreads) void rms_norm_bwd_kernel(const T* __restrict__ x, const float* __restrict__ w,
                                                                    const float* __restrict__ rrms_in,
-                                                                   const T* __restrict__ go, T* __restrict__ gx,
-                                                                   float* __restrict__ partial, size_t rows, int dim,
-                                                                   int accumulate_x) {
+                                                                   const T* __restrict__ go, const T* gx_old, T* gx,
+                                                                   float* __restrict__ partial, size_t rows, int dim) {
+    // gx_old: what dx is added to (gx itself for an in-place accumulation, another buffer of the same layout, or null to assign)
+    const bool accumulate_x = gx_old != nullptr;
     constexpr int N = Pack<T>::N;
     extern __shared__ float lds[];  // [kBwdWaves][dim]
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(kBwdThreads) void rms_norm_bwd_kernel(const T* __re
             if (c < dim) {
                 xd[p] = load_pack(x + row * dim + c);
                 gd[p] = load_pack(go + row * dim + c);
-                if (accumulate_x) od[p] = load_pack(gx + row * dim + c);
+                if (accumulate_x) od[p] = load_pack(gx_old + row * dim + c);
             }
         }
     };
@@ -194,8 +195,8 @@ __global__ __launch_bounds__(256) void rms_norm_dw_reduce_kernel(FinishSlots slo
 template <typename T>
 __global__ __launch_bounds__(kRowThreads) void rms_norm_bwd_scalar_kernel(const T* __restrict__ x, const float* __restrict__ w,
                                                                           const float* __restrict__ rrms_in,
-                                                                          const T* __restrict__ go, T* __restrict__ gx,
-                                                                          size_t rows, int dim, int accumulate_x) {
+                                                                          const T* __restrict__ go, const T* gx_old, T* gx,
+                                                                          size_t rows, int dim) {
     const int lane = threadIdx.x & 63;
     const size_t row = (size_t)blockIdx.x * kRowWaves + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(kRowThreads) void rms_norm_bwd_scalar_kernel(const 
     const float rrc_d = rrms * rrms * rrms / (float)dim;
     for (int c = lane; c < dim; c += kWave) {
         const float dx = rrms * (to_f32(gr[c]) * w[c]) - to_f32(xr[c]) * rrc_d * gdxw;
-        gxr[c] = from_f32<T>(accumulate_x ? to_f32(gxr[c]) + dx : dx);
+        gxr[c] = from_f32<T>(gx_old ? to_f32(gx_old[row * dim + c]) + dx : dx);
     }
 }
 // dw for the scalar fallback: one thread per column walks the rows in order.
@@ -277,21 +278,22 @@ int rms_norm_fwd(eisen_ctx* ctx, const void* x, const float* w, void* out, float
 constexpr unsigned kMaxPartialRows = EISEN_RMS_NORM_PARTIAL_ROWS;
 
 template <typename T, int MAXP>
-int rms_norm_bwd_vec(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* partial, unsigned blocks,
-                     size_t rows, size_t dim, int accumulate_x) {
+int rms_norm_bwd_vec(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, const void* gx_old, void* gx, float* partial,
+                     unsigned blocks, size_t rows, size_t dim) {
     const size_t lds = (size_t)kBwdWaves * dim * sizeof(float);
-    rms_norm_bwd_kernel<T, MAXP><<<blocks, kBwdThreads, lds, ctx->stream>>>((const T*)x, w, rrms, (const T*)go, (T*)gx, partial, rows, (int)dim,
-                                                                            accumulate_x);
+    rms_norm_bwd_kernel<T, MAXP><<<blocks, kBwdThreads, lds, ctx->stream>>>((const T*)x, w, rrms, (const T*)go, (const T*)gx_old, (T*)gx, partial, rows,
+                                                                            (int)dim);
     EISEN_LAUNCH_CHECK(ctx, "rms_norm_bwd_kernel");
     return 0;
 }
 
 // dx, and the gain gradient as rows of `partial` ([kMaxPartialRows][dim]); *nrows = rows written.
 template <typename T>
-int rms_norm_bwd_partial(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx, float* partial, size_t* nrows,
-                         size_t rows, size_t dim, int accumulate_x) {
+int rms_norm_bwd_partial(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, const void* gx_old, void* gx, float* partial,
+                         size_t* nrows, size_t rows, size_t dim) {
     constexpr int N = Pack<T>::N;
-    const bool vec = dim % N == 0 && eisen_aligned(x, 16) && eisen_aligned(go, 16) && eisen_aligned(gx, 16) && eisen_aligned(w, 16) &&
+    const bool accumulate_x = gx_old != nullptr;
+    const bool vec = dim % N == 0 && eisen_aligned(x, 16) && eisen_aligned(go, 16) && eisen_aligned(gx, 16) && eisen_aligned(gx_old, 16) && eisen_aligned(w, 16) &&
                      dim <= (size_t)kWave * N * 8 && (size_t)kBwdWaves * dim * sizeof(float) <= 64 * 1024;
     // algorithmic bytes: x and dy read, dx written (and read first when the call accumulates), one rrms per row
     EisenProfScope prof(ctx, sizeof(T) == 2 ? "rms_norm_bwd_bf16" : "rms_norm_bwd_f32",
@@ -301,13 +303,13 @@ int rms_norm_bwd_partial(eisen_ctx* ctx, const void* x, const float* w, const fl
         const unsigned blocks = (unsigned)std::min<size_t>(eisen_ceil_div(rows, kBwdWaves), kMaxPartialRows);
         *nrows = blocks;
         const size_t packs = eisen_ceil_div(dim, (size_t)kWave * N);
-        if (packs <= 1) return rms_norm_bwd_vec<T, 1>(ctx, x, w, rrms, go, gx, partial, blocks, rows, dim, accumulate_x);
-        if (packs <= 2) return rms_norm_bwd_vec<T, 2>(ctx, x, w, rrms, go, gx, partial, blocks, rows, dim, accumulate_x);
-        if (packs <= 4) return rms_norm_bwd_vec<T, 4>(ctx, x, w, rrms, go, gx, partial, blocks, rows, dim, accumulate_x);
-        return rms_norm_bwd_vec<T, 8>(ctx, x, w, rrms, go, gx, partial, blocks, rows, dim, accumulate_x);
+        if (packs <= 1) return rms_norm_bwd_vec<T, 1>(ctx, x, w, rrms, go, gx_old, gx, partial, blocks, rows, dim);
+        if (packs <= 2) return rms_norm_bwd_vec<T, 2>(ctx, x, w, rrms, go, gx_old, gx, partial, blocks, rows, dim);
+        if (packs <= 4) return rms_norm_bwd_vec<T, 4>(ctx, x, w, rrms, go, gx_old, gx, partial, blocks, rows, dim);
+        return rms_norm_bwd_vec<T, 8>(ctx, x, w, rrms, go, gx_old, gx, partial, blocks, rows, dim);
     }
     rms_norm_bwd_scalar_kernel<T><<<(unsigned)eisen_ceil_div(rows, kRowWaves), kRowThreads, 0, ctx->stream>>>(
-        (const T*)x, w, rrms, (const T*)go, (T*)gx, rows, (int)dim, accumulate_x);
+        (const T*)x, w, rrms, (const T*)go, (const T*)gx_old, (T*)gx, rows, (int)dim);
     EISEN_LAUNCH_CHECK(ctx, "rms_norm_bwd_scalar_kernel");
     *nrows = 1;  // one thread per column adds its rows in order into a zeroed row
     int rc = eisen_hip_fill(ctx, partial, EISEN_F32, 0.0f, dim);
@@ -362,8 +364,9 @@ extern "C" int eisen_hip_rms_norm_backward(eisen_ctx* ctx, const void* x, const 
     int rc = eisen_workspace(ctx, (size_t)kMaxPartialRows * dim * sizeof(float), &ws);
     if (rc) return rc;
     size_t nrows = 0;
-    rc = dtype == EISEN_F32 ? rms_norm_bwd_partial<float>(ctx, x, w, rrms, go, gx, (float*)ws, &nrows, rows, dim, accumulate_x)
-                            : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx, (float*)ws, &nrows, rows, dim, accumulate_x);
+    const void* gx_old = accumulate_x ? gx : nullptr;
+    rc = dtype == EISEN_F32 ? rms_norm_bwd_partial<float>(ctx, x, w, rrms, go, gx_old, gx, (float*)ws, &nrows, rows, dim)
+                            : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx_old, gx, (float*)ws, &nrows, rows, dim);
     if (rc) return rc;
     const float* p = (const float*)ws;
     return rms_norm_dw_finish(ctx, 1, &p, &gw, &nrows, dim, nullptr);
@@ -377,8 +380,21 @@ extern "C" int eisen_hip_rms_norm_backward_partial(eisen_ctx* ctx, const void* x
     EISEN_REQUIRE(ctx, dim > 0 && dim < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_rms_norm_backward_partial: dim %zu out of range", dim);
     *nrows_out = 0;
     if (rows == 0) return 0;
-    return dtype == EISEN_F32 ? rms_norm_bwd_partial<float>(ctx, x, w, rrms, go, gx, partial, nrows_out, rows, dim, accumulate_x)
-                              : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx, partial, nrows_out, rows, dim, accumulate_x);
+    const void* gx_old = accumulate_x ? gx : nullptr;
+    return dtype == EISEN_F32 ? rms_norm_bwd_partial<float>(ctx, x, w, rrms, go, gx_old, gx, partial, nrows_out, rows, dim)
+                              : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx_old, gx, partial, nrows_out, rows, dim);
+}
+
+extern "C" int eisen_hip_rms_norm_backward_partial_add(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, const void* gx_in,
+                                                       void* gx, float* partial, size_t* nrows_out, int dtype, size_t rows, size_t dim) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, x && w && rrms && go && gx_in && gx && partial && nrows_out, EISEN_E_ARG, "eisen_hip_rms_norm_backward_partial_add: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_rms_norm_backward_partial_add: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, dim > 0 && dim < (size_t(1) << 30), EISEN_E_SHAPE, "eisen_hip_rms_norm_backward_partial_add: dim %zu out of range", dim);
+    *nrows_out = 0;
+    if (rows == 0) return 0;
+    return dtype == EISEN_F32 ? rms_norm_bwd_partial<float>(ctx, x, w, rrms, go, gx_in, gx, partial, nrows_out, rows, dim)
+                              : rms_norm_bwd_partial<bf16_t>(ctx, x, w, rrms, go, gx_in, gx, partial, nrows_out, rows, dim);
 }
 
 extern "C" int eisen_hip_rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim,

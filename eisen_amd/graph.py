@@ -88,6 +88,9 @@ class Graph:
     def set_no_grad(self, v): self._call("eisen_graph_set_no_grad", _i(int(v)))
     def restore_save_point(self, sp): self._call("eisen_graph_restore_save_point", _sz(sp))
 
+    def set_weight_gradient_window(self, backward_passes): self._call("eisen_graph_set_weight_gradient_window", _sz(backward_passes))
+    def flush_weight_gradients(self): self._call("eisen_graph_flush_weight_gradients")
+
     def restore_save_point_keep(self, sp, keep):
         out = _sz()
         self._call("eisen_graph_restore_save_point_keep", _sz(sp), _sz(keep), C.byref(out))

@@ -257,6 +257,13 @@ class Context:
                    _sz(rows), _sz(dim), _i(accumulate_x))
         return n.value
 
+    def rms_norm_backward_partial_add(self, x, w, rrms, go, gx_in, gx, partial, dtype, rows, dim):
+        """rms_norm_backward_partial with gx = gx_in + dx (gx_in may be gx)."""
+        n = C.c_size_t(0)
+        self._call("eisen_hip_rms_norm_backward_partial_add", _ptr(x), _ptr(w), _ptr(rrms), _ptr(go), _ptr(gx_in), _ptr(gx), _ptr(partial), C.byref(n),
+                   _i(dtype), _sz(rows), _sz(dim))
+        return n.value
+
     def rms_norm_dw_finish(self, partials, gws, nrows, dim, assign=None):
         """gw_i (+)= column sums of the first nrows_i rows of partial_i, all in one launch; assign[i]: overwrite gw_i."""
         n = len(partials)
@@ -317,6 +324,16 @@ class Context:
         pc = (_vp * n)(*[_ptr(c) for c in Cs])
         pn = (C.c_size_t * n)(*Ns)
         self._call("eisen_hip_gemm_grouped", _sz(n), pa, pb, pc, pn, _i(dtype_ab), _i(dtype_c), _i(trans_a), _i(trans_b), _sz(M), _sz(K), _i(accumulate))
+
+    def gemm_grouped_ksegments(self, As, Bs, Cs, Ms, Ns, seg_k, accumulate=0):
+        """C_p (+)= sum_s As[p][s]^T Bs[p][s]: bf16 pieces [seg_k, M_p] and [seg_k, N_p], f32 results."""
+        n, ns = len(Cs), len(As[0])
+        pa = (_vp * (n * ns))(*[_ptr(a) for row in As for a in row])
+        pb = (_vp * (n * ns))(*[_ptr(b) for row in Bs for b in row])
+        pc = (_vp * n)(*[_ptr(c) for c in Cs])
+        pm = (C.c_size_t * n)(*Ms)
+        pn = (C.c_size_t * n)(*Ns)
+        self._call("eisen_hip_gemm_grouped_ksegments", _sz(n), _sz(ns), pa, pb, pc, pm, pn, _sz(seg_k), _i(accumulate))
 
     def gemm_swiglu_forward(self, X, Wg, Wu, G, U, H, dtype, M, N, K):
         """G = X Wg, U = X Wu, H = silu(G) * U."""

@@ -48,6 +48,15 @@ int eisen_graph_restore_save_point(eisen_graph* g, size_t save_point);
  * (its new id is returned), everything else above the save point goes back to the pool.  The reference's test of the
  * primitives (tests/gpu_kernels.rs:560-610) copies the block output to the host instead; recompute block by block
  * needs it to stay on the device. */
+/* Weight gradients over a window of backward passes (no counterpart in the reference, whose Linear backward adds
+ * A^T dC to the gradient in every pass, src/graph/ops/linear.rs:279-287).  With backward_passes = n in 2..8 the weight
+ * gradients of bf16 Linear layers of at least 16 tiles of 256 x 256 are not formed by the pass that produces their
+ * operands: the operands stay allocated (they outlive clear_activations) and one launch per group of equally shaped
+ * weights contracts over all passes of the window (eisen_hip_gemm_grouped_ksegments) when the n-th pass ends, or as
+ * soon as a parameter's gradient is read, cleared or handed to the optimizer.  The sums are the reference's in another
+ * rounding order.  0 or 1 (the default): every pass forms its own.  _flush runs what the window holds now. */
+int eisen_graph_set_weight_gradient_window(eisen_graph* g, size_t backward_passes);
+int eisen_graph_flush_weight_gradients(eisen_graph* g);
 int eisen_graph_restore_save_point_keep(eisen_graph* g, size_t save_point, size_t keep, size_t* new_id_out);
 int eisen_graph_clear_activations(eisen_graph* g);
 int eisen_graph_reinterpret_shape(eisen_graph* g, size_t id, const size_t* shape, int rank);

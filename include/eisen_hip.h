@@ -193,6 +193,10 @@ int eisen_hip_rms_norm_backward(eisen_ctx* ctx, const void* x, const float* w, c
 #define EISEN_RMS_NORM_PARTIAL_ROWS 256
 int eisen_hip_rms_norm_backward_partial(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, void* gx,
                                         float* partial, size_t* nrows_out, int dtype, size_t rows, size_t dim, int accumulate_x);
+/* eisen_hip_rms_norm_backward_partial whose input gradient is gx = gx_in + dx: what it adds to is read from another
+ * buffer than the one it writes (gx_in may also be gx itself).  For a caller that must keep gx_in as it is. */
+int eisen_hip_rms_norm_backward_partial_add(eisen_ctx* ctx, const void* x, const float* w, const float* rrms, const void* go, const void* gx_in,
+                                            void* gx, float* partial, size_t* nrows_out, int dtype, size_t rows, size_t dim);
 int eisen_hip_rms_norm_dw_finish(eisen_ctx* ctx, size_t n, const float* const* partial, float* const* gw, const size_t* nrows, size_t dim,
                                  const int* assign);
 /* rope_f32 / rope_backward_f32 (kernels/ops_f32.cu:724-760; Graph::rope,
@@ -259,6 +263,18 @@ int eisen_hip_gemm_residual(eisen_ctx* ctx, const void* A, const void* B, const 
  * transformer block; they run as one grid when that fills the chip better than the separate launches. */
 int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* const* A, const void* const* B, void* const* C, const size_t* N,
                            int dtype_ab, int dtype_c, int trans_a, int trans_b, size_t M, size_t K, int accumulate);
+
+/* C_p (+)= sum_{s < n_segments} A_ps^T B_ps for p < n_products: the dB += A^T dC of the matmul backward
+ * (src/graph/ops/linear.rs:279-287) for several weights and several micro-batches of a gradient-accumulation
+ * window at once.  A[p * n_segments + s] is bf16 [seg_k, M_p] (the activations weight p multiplied in micro-batch s),
+ * B[p * n_segments + s] bf16 [seg_k, N_p] (the gradient of that product), C[p] f32 [M_p, N_p].  The reference adds one
+ * micro-batch at a time, in f32; here the pieces of a product are summed in the MFMA accumulators of one launch (any
+ * number of products of up to 8 pieces, every M_p and N_p a multiple of 256, seg_k of 128, at least 176 tiles of
+ * 256 x 256 in all), which reads and writes each gradient once per window instead of once per micro-batch.  Other
+ * shapes run one accumulating GEMM per product and piece, in piece order. */
+#define EISEN_GEMM_MAX_KSEGMENTS 8
+int eisen_hip_gemm_grouped_ksegments(eisen_ctx* ctx, size_t n_products, size_t n_segments, const void* const* A, const void* const* B,
+                                     void* const* C, const size_t* M, const size_t* N, size_t seg_k, int accumulate);
 
 /* G = X Wg, U = X Wu, H = silu(G) * U: the gate and up projections of the feed-forward block and their SwiGLU
  * (src/nn/transformer.rs:41-46: `ffn_gate.forward`, `g.silu`, `ffn1.forward`, `g.mul`) as one kernel.  X [M, K],

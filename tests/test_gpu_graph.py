@@ -193,6 +193,58 @@ def test_per_block_recompute_gives_the_same_bits_and_a_lower_high_water_mark(ctx
     assert peak1 < 0.6 * peak0, (peak0, peak1)
 
 
+@pytest.mark.parametrize("fused,checkpointing", [(True, False), (False, False), (True, True)], ids=["fused", "chain", "fused-recompute"])
+def test_weight_gradient_window_sums_over_micro_batches(ctx, fused, checkpointing):
+    # Graph::set_weight_gradient_window: the dB += A^T dC of every Linear layer (src/graph/ops/linear.rs:279-287) waits
+    # for the end of a window of backward passes and runs as one contraction over all of them.  Against the same passes
+    # without a window: losses and every gradient the window does not touch (norm gains, embedding) bit-identical -- the
+    # chain of activation gradients must not notice that its buffers are kept -- and the windowed gradients equal up to
+    # the rounding order of an f32 sum.  A full window (3 passes, gradients assigned), then a partial one that a gradient
+    # read ends (2 passes, gradients added to); nothing stays allocated afterwards.
+    cfg = dict(vocab=1024, hidden=1024, heads=8, kv_heads=8, ffn=2048, layers=2, tie=False)
+    mb, seq = 2, 128
+    batches = [gen.lm_batch(950 + i, mb, seq, cfg["vocab"]) for i in range(5)]
+    results = []
+    for window in (0, 3):
+        gg = G.Graph(ctx, G.BF16_MIXED)
+        lm = G.TransformerLM(gg, **cfg)
+        names = []
+        for pid, (name, w) in enumerate(gen.lm_weights(34, perturb_norm=0.1, **cfg)):
+            gg.load_tensor_data(pid, w)
+            names.append(name)
+        gg.mark_params()
+        lm.set_fused(fused)
+        lm.set_checkpointing(checkpointing)
+        gg.set_weight_gradient_window(window)
+        params = lm.params()
+        opt = G.AdamW(gg, params, 1e-3)
+        opt.zero_grad()
+        ctx.sync()
+        base = ctx.pool_stats()[0]
+        ctx.profile_start()
+        losses = [lm.micro_step(x, y) for x, y in batches]
+        grads = [gg.sync_grad_to_cpu(p) for p in params]
+        prof = ctx.profile_stop()
+        assert gg.num_tensors() == gg.num_params() and gg.tape_len() == 0
+        ctx.sync()
+        assert ctx.pool_stats()[0] == base, "buffers kept for the window were not given back"
+        launches = sum(e["launches"] for k, e in prof.items() if k.endswith("_window"))
+        assert launches == (2 if window else 0), prof.keys()
+        results.append((losses, grads, [names[p] for p in params]))
+        gg.close()
+    (l0, g0, names), (l1, g1, _) = results
+    assert l0 == l1
+    windowed = 0
+    for name, a, b in zip(names, g0, g1):
+        assert a.any(), name
+        if a.ndim == 2 and "embed" not in name:
+            assert_close(b, a, 1e-4, f"windowed gradient of {name}")
+            windowed += 1
+        else:
+            assert np.array_equal(a, b), f"gradient of {name} differs although the window does not hold it"
+    assert windowed == 7 * cfg["layers"] + 1
+
+
 # ---- composed training step against the oracle ---------------------------------------------------
 
 def _build_pair(ctx, cfg, weights, precision):

@@ -257,7 +257,17 @@ def test_rms_norm_backward_in_two_parts(ctx, dtype, dim):
         assert 1 <= n <= ctx.RMS_NORM_PARTIAL_ROWS
         assert_close(dn(ctx, gx, x.shape, dtype), egx, tol_for(dtype), f"dx {i}")
         parts.append(part); gws.append(gw); nrows.append(n); exp.append(gw0 + egw)
-        keep += [dx, dw, dgo, rr, gx]
+        # the input gradient added to what another buffer holds, which stays as it was; and in place: the same bits
+        old = prep(gen.normal(640 + i, (rows, dim)), dtype)
+        d_old, gx2, part2 = up(ctx, old, dtype), ctx.malloc(x.nbytes), ctx.malloc(ctx.RMS_NORM_PARTIAL_ROWS * dim * 4)
+        assert ctx.rms_norm_backward_partial_add(dx, dw, rr, dgo, d_old, gx2, part2, dtype, rows, dim) == n
+        got2 = dn(ctx, gx2, x.shape, dtype)
+        assert_close(got2, old.astype(np.float64) + egx, tol_for(dtype), f"dx {i} added to another buffer")
+        assert np.array_equal(dn(ctx, d_old, x.shape, dtype), old)
+        assert np.array_equal(dn(ctx, part2, (n, dim), F32), dn(ctx, part, (n, dim), F32))
+        ctx.rms_norm_backward_partial(dx, dw, rr, dgo, d_old, part2, dtype, rows, dim, 1)
+        assert np.array_equal(dn(ctx, d_old, x.shape, dtype), got2)
+        keep += [dx, dw, dgo, rr, gx, d_old, gx2, part2]
     ctx.rms_norm_dw_finish(parts, gws, nrows, dim)
     for i in range(len(row_counts)):
         assert_close(dn(ctx, gws[i], (dim,), F32), exp[i], tol_for(dtype) if dtype == BF16 else 2e-4, f"dw {i}")
@@ -821,6 +831,38 @@ def test_gemm_grouped_weight_gradients(ctx, M, K, Ns, accumulate):
         exp = xs[i].astype(np.float64).T @ dys[i].astype(np.float64) + (c0[i] if accumulate else 0)
         assert_close(dn(ctx, dC[i], (M, n), F32), exp, 1e-3, f"product {i}")
     for x in dA + dB + dC:
+        x.free()
+
+
+@pytest.mark.parametrize("shapes,seg_k,nseg", [(((1024, 2048), (2048, 4096), (512, 2048)), 256, 3),   # 176 tiles of 256x256: one launch
+                                               (((2048, 5632), (256, 256)), 128, 8),                   # the most pieces a launch takes
+                                               (tuple([(256, 512)] * 40 + [(512, 256)] * 48), 128, 2), # many products, one launch
+                                               (((128, 64), (256, 192)), 96, 2),                       # one GEMM per product and piece
+                                               (((256, 256),), 128, 9)])                               # too many pieces for one launch
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_gemm_grouped_ksegments_weight_gradients_over_micro_batches(ctx, shapes, seg_k, nseg, accumulate):
+    # dW_p (+)= sum_s X_ps^T dY_ps: X_ps [seg_k, M_p], dY_ps [seg_k, N_p] stored piece by piece (one per micro-batch)
+    xs = [[prep(gen.normal(600 + 16 * p + s, (seg_k, m), 0.5), BF16) for s in range(nseg)] for p, (m, n) in enumerate(shapes)]
+    dys = [[prep(gen.normal(800 + 16 * p + s, (seg_k, n), 0.5), BF16) for s in range(nseg)] for p, (m, n) in enumerate(shapes)]
+    c0 = [gen.normal(1000 + p, (m, n)).astype(np.float32) for p, (m, n) in enumerate(shapes)]
+    dA = [[up(ctx, x, BF16) for x in row] for row in xs]
+    dB = [[up(ctx, d, BF16) for d in row] for row in dys]
+    dC = [up(ctx, c, F32) for c in c0]
+    Ms, Ns = [m for m, n in shapes], [n for m, n in shapes]
+    ctx.gemm_grouped_ksegments(dA, dB, dC, Ms, Ns, seg_k, accumulate)
+    got = [dn(ctx, dC[p], shapes[p], F32) for p in range(len(shapes))]
+    for p, (m, n) in enumerate(shapes):
+        exp = sum(xs[p][s].astype(np.float64).T @ dys[p][s].astype(np.float64) for s in range(nseg)) + (c0[p] if accumulate else 0)
+        assert_close(got[p], exp, 1e-3, f"product {p}")
+    # the same contraction stored in one piece: the kernel walks the same slabs in the same order, so the bits agree
+    catA = [[up(ctx, np.concatenate(xs[p], axis=0), BF16)] for p in range(len(shapes))]
+    catB = [[up(ctx, np.concatenate(dys[p], axis=0), BF16)] for p in range(len(shapes))]
+    dC2 = [up(ctx, c, F32) for c in c0]
+    if nseg <= 8 and all(m % 256 == 0 and n % 256 == 0 for m, n in shapes):
+        ctx.gemm_grouped_ksegments(catA, catB, dC2, Ms, Ns, seg_k * nseg, accumulate)
+        for p in range(len(shapes)):
+            assert np.array_equal(dn(ctx, dC2[p], shapes[p], F32), got[p]), f"product {p}: pieces and one piece differ"
+    for x in [t for row in dA + dB + catA + catB for t in row] + dC + dC2:
         x.free()
 
 
