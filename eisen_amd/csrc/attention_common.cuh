@@ -69,14 +69,6 @@ __device__ __forceinline__ bf16x8 lds_tr_operand(const bf16_t* tile, int pitch, 
     return concat4(lds_read_tr(p), lds_read_tr(p + 8 * pitch));
 }
 
-// Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  This
-// renumbering gives XCD j the contiguous id range [j*total/8, (j+1)*total/8), in dispatch order, so
-// workgroups that are neighbours in the renumbered order (and share operands) also share an L2.
-__device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
-    const int per = total / 8;
-    return linear < per * 8 ? (linear % 8) * per + linear / 8 : linear;
-}
-
 // 2^x as the bare hardware instruction: results below 2^-126 flush to zero, which is what a softmax
 // weight that small should be; the library exp2f spends four more instructions per value on them.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -105,3 +105,11 @@ __device__ __forceinline__ int lds_swz(int row) {
     if (ROW_BYTES == 128) return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1);  // two rows per bank span
     return ((row & 3) << 2) | ((row >> 2) & 3);                                                          // a row is one or two bank spans
 }
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  This
+// renumbering gives XCD j the contiguous id range [j*total/8, (j+1)*total/8), in dispatch order, so
+// workgroups that are neighbours in the renumbered order (and share operands) also share an L2.
+__device__ __forceinline__ int xcd_contiguous_id(int linear, int total) {
+    const int per = total / 8;
+    return linear < per * 8 ? (linear % 8) * per + linear / 8 : linear;
+}

@@ -52,6 +52,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, std::conditi
     int t = blockIdx.x, mt, nt;
     int prod = 0;
     if constexpr (WIN) {
+        // an XCD (its own L2) works through a contiguous range of the tile order, 32 tiles at a time: with the order below
+        // those are a compact block of one product's tiles, which share their operand panels in that L2
+        t = xcd_contiguous_id(t, gridDim.x);
         // the first product whose tiles end after t (the table is the same for every lane: scalar loads)
         int lo = 0, hi = w.nprod - 1;
         while (lo < hi) {
@@ -67,7 +70,6 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, std::conditi
         g.A = uniform_pointer(row.A[0]); g.B = uniform_pointer(row.B[0]);
         g.lda = g.M; g.ldb = g.N; g.ldc = g.N;
         g.K = w.nseg * w.seg_slabs * WBK;
-        g.tile_group = g.N / WBN >= 32 ? 16 : 0;
     } else if (g.ngroup > 0) {
         int first = 0;
         g.A = g.grp_A[0]; g.B = g.grp_B[0]; g.C = g.grp_C[0]; g.N = g.grp_N[0];
@@ -81,7 +83,18 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, std::conditi
         g.ldc = g.N;
         if (!B_KC) g.ldb = g.N;
     }
-    {
+    if constexpr (WIN) {
+        // blocks of about 32 tiles: every M tile of a few N tiles, or (a tall product of few N tiles) every N tile of a few M tiles
+        const int n_tiles = g.N / WBN, m_tiles = g.M / WBM;
+        const bool along_m = m_tiles > 8 && n_tiles <= 8;
+        const int inner = along_m ? n_tiles : m_tiles, outer = along_m ? m_tiles : n_tiles;
+        const int width_max = max(1, 32 / inner);
+        const int per_group = width_max * inner, grp = t / per_group, within = t % per_group;
+        const int width = min(width_max, outer - grp * width_max);
+        const int in_i = within / width, out_i = grp * width_max + within % width;
+        mt = along_m ? out_i : in_i;
+        nt = along_m ? in_i : out_i;
+    } else {
         const int n_tiles = g.N / WBN, m_tiles = g.M / WBM;
         if (g.tile_group > 0) {  // all M tiles of a group of N tiles before the next group
             const int per_group = g.tile_group * m_tiles, grp = t / per_group, within = t % per_group;
