@@ -212,7 +212,9 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
     // compact block of C, so that the A and B panels they stream fit the caches together: C is walked in groups
     // of g.tile_group N tiles, all M tiles of a group before the next group, N index fastest inside a group.
     int mt = blockIdx.y, nt = blockIdx.x;
-    if (g.tile_group > 0) {
+    if (g.tile_group < 0) {
+        xcd_block_tile<4, 8>(blockIdx.y * gridDim.x + blockIdx.x, gridDim.y, gridDim.x, mt, nt);
+    } else if (g.tile_group > 0) {
         const int m_tiles = gridDim.y, n_tiles = gridDim.x;
         const int lin = blockIdx.y * n_tiles + blockIdx.x, per_group = g.tile_group * m_tiles;
         const int grp = lin / per_group, within = lin % per_group;
@@ -673,6 +675,9 @@ void launch_mfma_direct(eisen_ctx* ctx, GemmArgs g, bool a_kc, bool b_kc, int ba
     // grids many N tiles wide walk C in groups of 32 N tiles (measured on the 32000-column lm_head GEMMs: 4 % and
     // 10 % faster than row-major order); narrower grids are a few rounds of workgroups anyway
     g.tile_group = g.N / BN >= 64 ? 32 : 0;
+    // 256-row tiles of narrower grids: blocks of 4 x 8 tiles per XCD (tile_group < 0, see xcd_block_tile; 1-5 % faster on the
+    // products of a 4096-token step with contractions of 2048 to 32000)
+    if (g.tile_group == 0 && g.ngroup == 0 && BM == 256) g.tile_group = -1;
     // reading step st+1's operand registers between step st's MFMAs gains 2-4 % except in the slab-32 kernels of the
     // dW shapes (two steps per slab, two or three workgroups per CU already overlapping), where it loses
     const bool pipe = a_kc || b_kc || BK == 64;

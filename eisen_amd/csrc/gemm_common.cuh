@@ -34,7 +34,7 @@ struct GemmArgs {
     int grp_N[kMaxGroup];
     int grp_tile_end[kMaxGroup];
     long long grp_partial_off[kMaxGroup];  // grouped launch with split > 1: where product p's partial results start inside `partial`
-    int tile_group;                    // direct kernel: > 0 = N tiles per group of the tile order (see the kernel), 0 = row-major order
+    int tile_group;                    // direct kernel: > 0 = N tiles per group of the tile order (see the kernel), 0 = row-major order, < 0 = blocks per XCD
     int vec_c;                         // C rows are 16-byte aligned at every 8th column: the epilogue may use 16-byte accesses
     // K made of up to three segments with their own operands, C (+)= sum_s op(A_s) op(B_s): segment 0 is A/B/lda/ldb,
     // seg_end[s] is the contraction offset at which segment s ends (multiples of 64); nseg <= 1 means plain
@@ -86,6 +86,21 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 
 typedef bf16x4 __attribute__((address_space(3))) * lds_bf16x4_ptr;
+
+// Tile (mt, nt) of workgroup `lin` in an order that keeps the tiles an XCD works on at one time (a contiguous range of
+// the order, see xcd_contiguous_id; about one tile per CU, 32 per XCD) inside a block of BMT x BNT tiles, which share
+// BMT + BNT operand panels in that XCD's L2.  Block rows of BMT tile rows, blocks left to right, row-major inside a
+// block; the last block of a row and the last row of blocks may be smaller.
+template <int BMT, int BNT>
+__device__ __forceinline__ void xcd_block_tile(int lin, int m_tiles, int n_tiles, int& mt, int& nt) {
+    lin = xcd_contiguous_id(lin, m_tiles * n_tiles);
+    const int row_block = BMT * n_tiles, bi = lin / row_block, rem = lin % row_block;
+    const int h = min(BMT, m_tiles - BMT * bi);
+    const int bj = rem / (h * BNT), rem2 = rem % (h * BNT);
+    const int wdt = min(BNT, n_tiles - BNT * bj);
+    mt = BMT * bi + rem2 / wdt;
+    nt = BNT * bj + rem2 % wdt;
+}
 
 // d(silu(gate) * up) for one element, given dh (src/graph/ops/elementwise.rs:442-455 for silu, :294-331 for mul)
 __device__ __forceinline__ void swiglu_backward_elem(float gate, float up, float dh, float& dgate, float& dup) {
