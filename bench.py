@@ -159,7 +159,7 @@ def cpu_baseline_lm(c, seq, mb=1):
 # workloads
 # ---------------------------------------------------------------------------------------------
 
-def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True):
+def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True, beside=True):
     from eisen_amd import graph as G
     from eisen_amd import hip
     c = CONFIGS[name]
@@ -176,6 +176,7 @@ def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True):
     # weight gradients over the whole accumulation window in one contraction (Graph::set_weight_gradient_window): the sums
     # of train_llm.rs:386-477's micro-batch loop, each gradient read and written once per optimizer step
     g.set_weight_gradient_window(c["accum"] if window and 2 <= c["accum"] <= 8 else 0)
+    g.set_weight_gradients_beside(beside)   # the library's default; off = every GEMM in tape order on the one stream
     opt = G.AdamW(g, lm.params(), 1e-3)
     opt.config(1e-3, 0.9, 0.95, 1e-8, 0.1, 1.0)      # train_llm.rs:266-270 + grad clip 1.0
     opt.init_moments()
@@ -338,6 +339,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
     ap.add_argument("--no-window", action="store_true", help="c5: form every micro-batch's weight gradients in its own backward pass, as the reference does, "
                     "instead of once per optimizer step over the whole accumulation window")
+    ap.add_argument("--no-beside", action="store_true", help="c4: keep the weight-gradient GEMMs of narrow layers on the main stream, in tape order")
     ap.add_argument("--recompute", action="store_true", help="c5 / c4: per-block recompute (lower activation memory, one more forward pass per block)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -345,11 +347,11 @@ def main():
         sys.exit(2)
     w = args.workload
     if w in ("all", "c5"):
-        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute, not args.no_window)
+        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside)
         if w == "all":
             out["other_configs"] = dict(c4=brief(bench_lm("c4", 20, 3, not args.no_cpu)), c3=brief(bench_c3(20, 3)), c2=brief(bench_c2(20, 3)))
     elif w == "c4":
-        out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute, not args.no_window)
+        out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside)
     elif w == "c3":
         out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3)
     else:

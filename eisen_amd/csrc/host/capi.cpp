@@ -94,6 +94,9 @@ int eisen_graph_reinterpret_shape(eisen_graph* g, size_t id, const size_t* shape
 int eisen_graph_set_weight_gradient_window(eisen_graph* g, size_t backward_passes) {
     return guarded(g, [&](Graph& G) { G.set_weight_gradient_window(backward_passes); });
 }
+int eisen_graph_set_weight_gradients_beside(eisen_graph* g, int on) {
+    return guarded(g, [&](Graph& G) { G.set_weight_gradients_beside(on != 0); });
+}
 int eisen_graph_flush_weight_gradients(eisen_graph* g) {
     return guarded(g, [&](Graph& G) { G.flush_weight_gradients(); });
 }

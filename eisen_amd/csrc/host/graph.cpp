@@ -202,6 +202,9 @@ void Graph::reinterpret_shape(size_t id, const std::vector<size_t>& shape) {
 // back to the size-keyed pool inside the runtime.
 void Graph::restore_save_point(size_t save_point) {
     if (!side_guards.empty()) side_join();  // a backward pass that threw may have left side-stream work reading these buffers
+    // buffers kept for side-stream GEMMs (no window): given back now, so that a block-by-block recompute keeps its low
+    // high-water mark (the main stream waits for the side stream here; after a whole backward pass it already has)
+    if (window_dw.empty() && !retained_.empty()) side_join();
     flush_norm_dw(false);                   // ... and partial rows nobody will finish
     while (tensors.size() > save_point) {
         release(tensors.back());
@@ -230,6 +233,7 @@ void Graph::record(std::vector<size_t> inputs, size_t output, std::function<void
 Storage& Graph::grad_for_write(size_t id, int* accumulate, const void** add_from) {
     Tensor& t = at(id);
     if (t.is_param) {
+        if (!in_beside_ && !side_written_.empty() && std::find(side_written_.begin(), side_written_.end(), id) != side_written_.end()) side_join();
         *accumulate = t.grad_zero_pending ? 0 : 1;
         t.grad_zero_pending = false;
         if (add_from) *add_from = t.grad.ptr;
@@ -376,16 +380,53 @@ void Graph::flush_weight_gradients() {
         if (rc) break;
     }
     // the operands go back to the pool (stream order keeps them intact until the launches above have read them)
-    std::unordered_map<const void*, bool> held;
-    held.swap(retained_);
-    for (auto& kv : held)
-        if (kv.second) (void)eisen_hip_free(ctx_, const_cast<void*>(kv.first));
+    release_retained();
     check(rc, "weight gradients of the window");
 }
 
 void Graph::side_join() {
     check(eisen_hip_side_wait(ctx_), "side stream join");
     side_guards.clear();
+    side_written_.clear();
+    if (window_dw.empty()) release_retained();  // operands of side-stream GEMMs: what the main stream does next is ordered after them
+}
+
+void Graph::release_retained() {
+    if (retained_.empty()) return;
+    std::unordered_map<const void*, bool> held;
+    held.swap(retained_);
+    for (auto& kv : held)
+        if (kv.second) (void)eisen_hip_free(ctx_, const_cast<void*>(kv.first));
+}
+
+// a weight gradient of fewer 128 x 128 tiles than the chip has CUs, formed by its own backward pass (no window)
+bool Graph::beside_fits(size_t in, size_t out) const {
+    return beside_ && window_ < 2 && precision_mode == PrecisionMode::Bf16Mixed && ((in + 127) / 128) * ((out + 127) / 128) < 256;
+}
+
+void Graph::run_beside(bool beside, const std::vector<const void*>& reads, const std::vector<size_t>& weights, const std::function<int()>& launch,
+                       const char* what) {
+    if (!beside) {
+        check(launch(), what);
+        return;
+    }
+    check(eisen_hip_side_begin(ctx_), "side stream");
+    in_beside_ = true;
+    int rc = 0;
+    try {
+        rc = launch();
+    } catch (...) {
+        in_beside_ = false;
+        (void)eisen_hip_side_end(ctx_);
+        throw;
+    }
+    in_beside_ = false;
+    const int rc_end = eisen_hip_side_end(ctx_);  // back on the main stream whatever the launch returned
+    for (const void* p : reads) retained_.emplace(p, false);
+    for (size_t w : weights)
+        if (std::find(side_written_.begin(), side_written_.end(), w) == side_written_.end()) side_written_.push_back(w);
+    check(rc, what);
+    check(rc_end, "side stream");
 }
 
 const Storage& Graph::grad_for_read(size_t id) {
@@ -408,6 +449,7 @@ void Graph::materialize_grad(size_t id) {
 }
 
 void Graph::apply_pending_zero(size_t id) {
+    if (!side_written_.empty() && std::find(side_written_.begin(), side_written_.end(), id) != side_written_.end()) side_join();
     Tensor& t = at(id);
     if (t.grad_zero_pending) {
         check(eisen_hip_memset_zero(ctx_, t.grad.ptr, t.grad.numel * sizeof(float)), "zero_grad");
@@ -568,8 +610,12 @@ size_t Graph::matmul(size_t a, size_t b) {
         Storage& ga = g.grad_for_write(a, &acc);
         g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 1, M, K, N, acc), "matmul backward dA");
         if (g.window_take(b, g.compute_data(a).ptr, go.ptr, go.dtype, M, K, N)) return;
-        Storage& gb = g.grad_for_write(b, &acc);
-        g.check(eisen_hip_gemm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul backward dB");
+        const void* xa = g.compute_data(a).ptr;
+        g.run_beside(g.at(b).is_param && g.beside_fits(K, N), {xa, go.ptr}, {b}, [&]() {
+            int accb = 0;
+            Storage& gb = g.grad_for_write(b, &accb);
+            return eisen_hip_gemm(g.ctx(), xa, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, accb);
+        }, "matmul backward dB");
     });
     return out;
 }
@@ -612,8 +658,12 @@ size_t Graph::matmul_residual(size_t a, size_t b, size_t r, bool defer_dw) {
             // dOut's buffer (now also dR's) is only added to by nodes that run after the collecting group
             g.pending_dw.push_back(PendingDW{b, g.compute_data(a).ptr, go.ptr, M, K, N});
         } else {
-            Storage& gb = g.grad_for_write(b, &acc);
-            g.check(eisen_hip_gemm(g.ctx(), g.compute_data(a).ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "matmul_residual backward dB");
+            const void* xa = g.compute_data(a).ptr;
+            g.run_beside(g.at(b).is_param && g.beside_fits(K, N), {xa, go.ptr}, {b}, [&]() {
+                int accb = 0;
+                Storage& gb = g.grad_for_write(b, &accb);
+                return eisen_hip_gemm(g.ctx(), xa, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, accb);
+            }, "matmul_residual backward dB");
         }
     });
     return out;
@@ -684,8 +734,12 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r,
             g.device_free(dh);
         }
         if (!side && !windowed) {
-            Storage& gb = g.grad_for_write(b, &acc);
-            g.check(eisen_hip_gemm(g.ctx(), g.at(h).data.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, acc), "swiglu_matmul_residual backward dB");
+            const void* xh = g.at(h).data.ptr;
+            g.run_beside(g.at(b).is_param && g.beside_fits(K, N), {xh, go.ptr}, {b}, [&]() {
+                int accb = 0;
+                Storage& gb = g.grad_for_write(b, &accb);
+                return eisen_hip_gemm(g.ctx(), xh, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N, M, accb);
+            }, "swiglu_matmul_residual backward dB");
         }
     });
     return out;
@@ -844,18 +898,30 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
                 m++;
             }
             for (size_t i = 1; i < m; i++) same = same && accs[i] == accs[0];
-            if (same) {
-                g.check(eisen_hip_gemm_grouped(g.ctx(), m, As, Bs, Cs, Ns, EISEN_BF16, EISEN_F32, 1, 0, K, M, accs[0]), "matmul_group backward dW");
-            } else {  // same work, one launch per product (grad_for_write has already been consumed above)
-                for (size_t i = 0; i < m; i++)
-                    g.check(eisen_hip_gemm(g.ctx(), As[i], Bs[i], Cs[i], EISEN_BF16, dts[i], 1, 0, K, Ns[i], M, accs[i]), "matmul_group backward dW");
+            // narrow products: beside the chain (the gradients were fetched above: a weight the side stream is still writing
+            // has made the main stream wait there, which is safe and rare)
+            std::vector<const void*> reads(As, As + m);
+            reads.insert(reads.end(), Bs, Bs + m);
+            std::vector<size_t> written;
+            size_t tiles = 0;
+            for (size_t i = 0; i < m; i++) {
+                written.push_back(i < n ? ws[i] : extras[i - n].weight);
+                tiles += ((K + 127) / 128) * ((Ns[i] + 127) / 128);
             }
+            g.run_beside(tiles < 256 && g.beside_fits(K, 128), reads, written, [&]() {
+                if (same) return eisen_hip_gemm_grouped(g.ctx(), m, As, Bs, Cs, Ns, EISEN_BF16, EISEN_F32, 1, 0, K, M, accs[0]);
+                int rc = 0;  // same work, one launch per product (grad_for_write has already been consumed above)
+                for (size_t i = 0; i < m && !rc; i++) rc = eisen_hip_gemm(g.ctx(), As[i], Bs[i], Cs[i], EISEN_BF16, dts[i], 1, 0, K, Ns[i], M, accs[i]);
+                return rc;
+            }, "matmul_group backward dW");
             done = true;
         } else {
             for (const PendingDW& e : extras) {
                 int acc = 0;
                 Storage& gw = g.grad_for_write(e.weight, &acc);
-                g.check(eisen_hip_gemm(g.ctx(), e.x, e.dy, gw.ptr, EISEN_BF16, gw.dtype, 1, 0, e.in, e.out, e.rows, acc), "deferred dW");
+                g.run_beside(g.beside_fits(e.in, e.out), {e.x, e.dy}, {e.weight}, [&]() {
+                    return eisen_hip_gemm(g.ctx(), e.x, e.dy, gw.ptr, EISEN_BF16, gw.dtype, 1, 0, e.in, e.out, e.rows, acc);
+                }, "deferred dW");
             }
         }
         for (size_t i = 0; i < n && !done; i++) {
@@ -867,19 +933,22 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
                 Storage& g2 = g.grad_for_write(ws[i + 1], &acc2);
                 const size_t gs = g1.dtype == EISEN_BF16 ? 2 : 4;
                 const ptrdiff_t gd = (const char*)g2.ptr - (const char*)g1.ptr, od = (const char*)go2.ptr - (const char*)go1.ptr;
-                if (acc1 == acc2 && g1.dtype == g2.dtype && gd % 16 == 0 && od % 16 == 0) {
-                    g.check(eisen_hip_gemm_strided_batched(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, 2, K, N[i], M, 0, od / 2,
-                                                           gd / (ptrdiff_t)gs, acc1), "matmul_group backward dW");
-                } else {
-                    g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, K, N[i], M, acc1), "matmul_group backward dW");
-                    g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go2.ptr, g2.ptr, go2.dtype, g2.dtype, 1, 0, K, N[i + 1], M, acc2), "matmul_group backward dW");
-                }
+                const bool beside = g.at(ws[i]).is_param && g.at(ws[i + 1]).is_param && g.beside_fits(K, 2 * N[i]);
+                g.run_beside(beside, {xa.ptr, go1.ptr, go2.ptr}, {ws[i], ws[i + 1]}, [&]() {
+                    if (acc1 == acc2 && g1.dtype == g2.dtype && gd % 16 == 0 && od % 16 == 0)
+                        return eisen_hip_gemm_strided_batched(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, 2, K, N[i], M, 0, od / 2,
+                                                              gd / (ptrdiff_t)gs, acc1);
+                    const int rc = eisen_hip_gemm(g.ctx(), xa.ptr, go1.ptr, g1.ptr, go1.dtype, g1.dtype, 1, 0, K, N[i], M, acc1);
+                    return rc ? rc : eisen_hip_gemm(g.ctx(), xa.ptr, go2.ptr, g2.ptr, go2.dtype, g2.dtype, 1, 0, K, N[i + 1], M, acc2);
+                }, "matmul_group backward dW");
                 i++;
             } else if (has[i]) {
                 const Storage& go = g.grad_for_read(outs[i]);
                 int acc = 0;
                 Storage& gb = g.grad_for_write(ws[i], &acc);
-                g.check(eisen_hip_gemm(g.ctx(), xa.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N[i], M, acc), "matmul_group backward dW");
+                g.run_beside(g.at(ws[i]).is_param && g.beside_fits(K, N[i]), {xa.ptr, go.ptr}, {ws[i]}, [&]() {
+                    return eisen_hip_gemm(g.ctx(), xa.ptr, go.ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, K, N[i], M, acc);
+                }, "matmul_group backward dW");
             }
         }
         (void)all;
@@ -906,8 +975,12 @@ size_t Graph::matmul_trans_b(size_t a, size_t b) {
         int acc = 0;
         Storage& ga = g.grad_for_write(a, &acc);
         g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(b).ptr, ga.ptr, go.dtype, ga.dtype, 0, 0, M, K, N, acc), "matmul_trans_b backward dA");
-        Storage& gb = g.grad_for_write(b, &acc);
-        g.check(eisen_hip_gemm(g.ctx(), go.ptr, g.compute_data(a).ptr, gb.ptr, go.dtype, gb.dtype, 1, 0, N, K, M, acc), "matmul_trans_b backward dB");
+        const void* xa = g.compute_data(a).ptr;
+        g.run_beside(g.at(b).is_param && g.beside_fits(N, K), {go.ptr, xa}, {b}, [&]() {
+            int accb = 0;
+            Storage& gb = g.grad_for_write(b, &accb);
+            return eisen_hip_gemm(g.ctx(), go.ptr, xa, gb.ptr, go.dtype, gb.dtype, 1, 0, N, K, M, accb);
+        }, "matmul_trans_b backward dB");
     });
     return out;
 }

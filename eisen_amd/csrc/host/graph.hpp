@@ -205,6 +205,11 @@ class Graph {
     // the n-th pass ends, and before anything reads, clears or scales a parameter's gradient; what a caller can observe
     // is the reference's sum in a different rounding order (one f32 accumulation over all tokens of the window).
     // The price is memory: the operands of every windowed product of every pass in the window stay allocated.
+    // Without a window, the weight-gradient GEMMs of narrow layers (each too small to fill the chip) run on the context's
+    // side stream beside the chain of input gradients, which never waits for them: their operands are kept as above
+    // (a gradient buffer that a later node adds to in place is replaced by a fresh one) until the backward pass ends
+    // and the main stream has waited for the side stream.  Same kernels, same bits.  On by default.
+    void set_weight_gradients_beside(bool on) { beside_ = on; }
     void set_weight_gradient_window(size_t backward_passes);
     size_t weight_gradient_window() const { return window_; }
     void flush_weight_gradients();
@@ -219,6 +224,13 @@ class Graph {
     size_t backward_root_ = (size_t)-1;
     size_t backward_epoch_ = 0;
     size_t window_ = 0, window_passes_ = 0;
+    bool beside_ = true, in_beside_ = false;
+    std::vector<size_t> side_written_;  // parameters whose gradients the side stream is writing: the main stream waits before it touches them
+    // Runs `launch` (weight-gradient GEMMs reading `reads`, writing the gradients of `weights`) on the side stream when
+    // the products are small and no window is set, on the current stream otherwise.
+    bool beside_fits(size_t in, size_t out) const;
+    void run_beside(bool beside, const std::vector<const void*>& reads, const std::vector<size_t>& weights, const std::function<int()>& launch, const char* what);
+    void release_retained();
     // buffers a windowed weight-gradient GEMM will read -> whether their owner has released them (then the flush frees them)
     std::unordered_map<const void*, bool> retained_;
     // the product x^T dy joins the window when it can; false: the caller forms it now

@@ -61,6 +61,8 @@ struct eisen_ctx {
     // grow-only device workspace for two-stage reductions and tables
     void* ws = nullptr;
     size_t ws_bytes = 0;
+    void* ws_side = nullptr;  // the same for launches on the side stream, which run beside main-stream kernels that use `ws`
+    size_t ws_side_bytes = 0;
     std::vector<eisen_rope_table> rope_tables;
     float* attn_scratch = nullptr;  // this device's copy of the file-scope scratch array in attention.hip (never freed)
     eisen_prof prof;

@@ -89,6 +89,8 @@ extern "C" int eisen_hip_destroy(eisen_ctx* ctx) {
     for (auto& kv : ctx->live) (void)hipFreeAsync(kv.first, ctx->stream);
     for (auto& t : ctx->rope_tables) (void)hipFreeAsync(t.cos_sin, ctx->stream);
     if (ctx->ws) (void)hipFreeAsync(ctx->ws, ctx->stream);
+    if (ctx->ws_side) (void)hipFreeAsync(ctx->ws_side, ctx->side_stream);
+    (void)hipStreamSynchronize(ctx->side_stream);
     (void)hipStreamSynchronize(ctx->stream);
     for (auto& sl : ctx->stage) {
         if (sl.ptr) (void)hipHostFree(sl.ptr);
@@ -216,18 +218,21 @@ extern "C" int eisen_hip_pool_stats(eisen_ctx* ctx, size_t* in_use_bytes, size_t
 }
 
 int eisen_workspace(eisen_ctx* ctx, size_t bytes, void** out) {
-    if (bytes > ctx->ws_bytes) {
+    // one block per stream: each is allocated, used and freed in the order of its own stream
+    void*& ws = ctx->side_active ? ctx->ws_side : ctx->ws;
+    size_t& ws_bytes = ctx->side_active ? ctx->ws_side_bytes : ctx->ws_bytes;
+    if (bytes > ws_bytes) {
         // stream order makes the old block safe to free while earlier kernels still read it
-        if (ctx->ws) EISEN_HIP_TRY(ctx, hipFreeAsync(ctx->ws, ctx->stream));
-        ctx->ws = nullptr;
-        ctx->ws_bytes = 0;
+        if (ws) EISEN_HIP_TRY(ctx, hipFreeAsync(ws, ctx->stream));
+        ws = nullptr;
+        ws_bytes = 0;
         size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
-        hipError_t e = hipMallocAsync(&ctx->ws, want, ctx->stream);
+        hipError_t e = hipMallocAsync(&ws, want, ctx->stream);
         if (e != hipSuccess)
             return eisen_set_error(ctx, EISEN_E_NOMEM, "workspace of %zu bytes: %s", want, hipGetErrorString(e));
-        ctx->ws_bytes = want;
+        ws_bytes = want;
     }
-    *out = ctx->ws;
+    *out = ws;
     return 0;
 }
 

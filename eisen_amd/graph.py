@@ -89,6 +89,7 @@ class Graph:
     def restore_save_point(self, sp): self._call("eisen_graph_restore_save_point", _sz(sp))
 
     def set_weight_gradient_window(self, backward_passes): self._call("eisen_graph_set_weight_gradient_window", _sz(backward_passes))
+    def set_weight_gradients_beside(self, on): self._call("eisen_graph_set_weight_gradients_beside", _i(int(on)))
     def flush_weight_gradients(self): self._call("eisen_graph_flush_weight_gradients")
 
     def restore_save_point_keep(self, sp, keep):

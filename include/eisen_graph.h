@@ -56,6 +56,11 @@ int eisen_graph_restore_save_point(eisen_graph* g, size_t save_point);
  * soon as a parameter's gradient is read, cleared or handed to the optimizer.  The sums are the reference's in another
  * rounding order.  0 or 1 (the default): every pass forms its own.  _flush runs what the window holds now. */
 int eisen_graph_set_weight_gradient_window(eisen_graph* g, size_t backward_passes);
+/* 1 (the default): without a window, the weight-gradient GEMMs of narrow layers (fewer 128 x 128 tiles than the chip has
+ * CUs; bf16 graphs) run on the context's side stream beside the chain of input gradients, their operands kept until
+ * the backward pass has ended and the main stream has waited for the side stream.  Same kernels and bits as 0, where
+ * every GEMM runs in tape order on the one stream, as in the reference (src/graph/mod.rs:670-796). */
+int eisen_graph_set_weight_gradients_beside(eisen_graph* g, int on);
 int eisen_graph_flush_weight_gradients(eisen_graph* g);
 int eisen_graph_restore_save_point_keep(eisen_graph* g, size_t save_point, size_t keep, size_t* new_id_out);
 int eisen_graph_clear_activations(eisen_graph* g);

@@ -245,6 +245,43 @@ def test_weight_gradient_window_sums_over_micro_batches(ctx, fused, checkpointin
     assert windowed == 7 * cfg["layers"] + 1
 
 
+@pytest.mark.parametrize("tie,checkpointing", [(True, False), (False, False), (True, True)], ids=["tied", "untied", "tied-recompute"])
+def test_weight_gradients_beside_the_chain_give_the_same_bits(ctx, tie, checkpointing):
+    # Graph::set_weight_gradients_beside (the default): the weight-gradient GEMMs of narrow layers run on the side stream
+    # while the main stream goes on with the input gradients.  Same kernels on the same operands => every loss and
+    # gradient bit-identical to the run that keeps the reference's tape order on one stream (src/graph/mod.rs:670-796),
+    # over two accumulated micro-batches; with tied embeddings the lm_head gradient (side stream) and the embedding
+    # scatter (main stream) meet in one buffer.  Nothing stays allocated afterwards.
+    cfg = dict(vocab=512, hidden=256, heads=4, kv_heads=2, ffn=512, layers=3, tie=tie)
+    mb, seq = 4, 128
+    batches = [gen.lm_batch(970 + i, mb, seq, cfg["vocab"], "zipf") for i in range(2)]
+    results = []
+    for beside in (False, True):
+        gg = G.Graph(ctx, G.BF16_MIXED)
+        lm = G.TransformerLM(gg, **cfg)
+        for pid, (_, w) in enumerate(gen.lm_weights(35, perturb_norm=0.1, **cfg)):
+            gg.load_tensor_data(pid, w)
+        gg.mark_params()
+        lm.set_checkpointing(checkpointing)
+        gg.set_weight_gradients_beside(beside)
+        params = lm.params()
+        opt = G.AdamW(gg, params, 1e-3)
+        opt.zero_grad()
+        ctx.sync()
+        base = ctx.pool_stats()[0]
+        losses = [lm.micro_step(x, y) for x, y in batches]
+        grads = [gg.sync_grad_to_cpu(p) for p in params]
+        assert gg.num_tensors() == gg.num_params() and gg.tape_len() == 0
+        ctx.sync()
+        assert ctx.pool_stats()[0] == base, "buffers kept for the side stream were not given back"
+        results.append((losses, grads))
+        gg.close()
+    (l0, g0), (l1, g1) = results
+    assert l0 == l1
+    for i, (a, b) in enumerate(zip(g0, g1)):
+        assert a.any() and np.array_equal(a, b), f"gradient of parameter {i} differs when the weight gradients run beside the chain"
+
+
 # ---- composed training step against the oracle ---------------------------------------------------
 
 def _build_pair(ctx, cfg, weights, precision):
