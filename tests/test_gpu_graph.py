@@ -245,6 +245,56 @@ def test_weight_gradient_window_sums_over_micro_batches(ctx, fused, checkpointin
     assert windowed == 7 * cfg["layers"] + 1
 
 
+def test_weight_gradient_window_flushes_when_a_gradient_is_read_cleared_or_outgrows_it(ctx):
+    # The corners of Graph::set_weight_gradient_window on a two-matmul graph whose weight is used twice per pass: a
+    # gradient read in the middle of a window sees every pass so far; zero_grad in the middle of a window discards what
+    # the window held (added, then cleared, as the reference's order of calls would); more passes than the window fit
+    # in any number of launches; turning the window off finishes what it holds.  Against the same calls without a window.
+    hidden, rows = 1024, 128
+    w0 = gen.normal(41, (hidden, hidden), 0.03)
+    xs = [gen.normal(42 + i, (rows, hidden)) for i in range(7)]
+    tg = [gen.uniform_ids(60 + i, (rows,), hidden) for i in range(7)]
+
+    def run(window):
+        g = G.Graph(ctx, G.BF16_MIXED)
+        w = g.alloc(w0.shape, w0)
+        g.mark_params()
+        g.set_weight_gradient_window(window)
+        opt = G.AdamW(g, [w], 1e-3)
+        opt.zero_grad()
+        ctx.sync()
+        base = ctx.pool_stats()[0]
+        seen = []
+
+        def one_pass(i):
+            x = g.input(xs[i])
+            loss = g.cross_entropy(g.matmul(g.matmul(x, w), w), tg[i])
+            g.backward(loss)
+            g.clear_activations()
+
+        one_pass(0)
+        seen.append(g.sync_grad_to_cpu(w))            # read after one pass of a window of three
+        one_pass(1)
+        one_pass(2)
+        one_pass(3)                                     # the fourth pass since zero_grad: the window has been through one flush by now
+        seen.append(g.sync_grad_to_cpu(w))
+        one_pass(4)
+        opt.zero_grad()                                 # one pass pending: it must not come back after the clearing
+        one_pass(5)
+        g.set_weight_gradient_window(0)                 # finishes pass 5
+        one_pass(6)                                     # formed by its own backward pass
+        seen.append(g.sync_grad_to_cpu(w))
+        ctx.sync()
+        assert g.num_tensors() == g.num_params() and ctx.pool_stats()[0] == base
+        g.close()
+        return seen
+
+    plain, windowed = run(0), run(3)
+    for i, (a, b) in enumerate(zip(plain, windowed)):
+        assert a.any()
+        assert_close(b, a, 1e-4, f"weight gradient at read {i}")
+
+
 @pytest.mark.parametrize("tie,checkpointing", [(True, False), (False, False), (True, True)], ids=["tied", "untied", "tied-recompute"])
 def test_weight_gradients_beside_the_chain_give_the_same_bits(ctx, tie, checkpointing):
     # Graph::set_weight_gradients_beside (the default): the weight-gradient GEMMs of narrow layers run on the side stream
