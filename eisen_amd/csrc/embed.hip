@@ -226,16 +226,42 @@ __global__ __launch_bounds__(kThreads) void scatter_runs_kernel(const T* __restr
 }
 
 // The device route takes batches whose keys fit 32 bits and whose rows are whole column pairs.
-bool scatter_on_device(const void* go, const float* gw, int dtype, size_t n_ids, size_t vocab, size_t hidden, int* n_pow2, int* shift) {
+bool scatter_index_on_device(size_t n_ids, size_t vocab, int* n_pow2, int* shift) {
     if (n_ids == 0 || n_ids > (size_t)kSortMax) return false;
     int p = kSortThreads, sh = 10;  // the sort works on whole multiples of its 1024 threads
     while ((size_t)p < n_ids) { p <<= 1; sh++; }
     if ((unsigned long long)vocab << sh >= 0xffffffffull) return false;
-    (void)dtype;
-    if (hidden % 2 != 0 || !eisen_aligned(go, 8) || !eisen_aligned(gw, 8)) return false;
     *n_pow2 = p;
     *shift = sh;
     return true;
+}
+bool scatter_on_device(const void* go, const float* gw, int dtype, size_t n_ids, size_t vocab, size_t hidden, int* n_pow2, int* shift) {
+    (void)dtype;
+    if (hidden % 2 != 0 || !eisen_aligned(go, 8) || !eisen_aligned(gw, 8)) return false;
+    return scatter_index_on_device(n_ids, vocab, n_pow2, shift);
+}
+
+// index = [sorted ids | positions in sorted order | run ends], n_ids ints each
+void scatter_launch_sort(eisen_ctx* ctx, const int32_t* ids_dev, size_t n_ids, size_t vocab, int n_pow2, int shift, int32_t* index) {
+    int32_t* sorted_ids = index;
+    int32_t* order = sorted_ids + n_ids;
+    int32_t* run_end = order + n_ids;
+    switch (n_pow2 / kSortThreads) {
+        case 1: scatter_sort_kernel<1><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+        case 2: scatter_sort_kernel<2><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+        case 4: scatter_sort_kernel<4><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+        case 8: scatter_sort_kernel<8><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+        default: scatter_sort_kernel<16><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
+    }
+}
+void scatter_launch_runs(eisen_ctx* ctx, const int32_t* index, const void* go, float* gw, int dtype, size_t n_ids, size_t hidden) {
+    const int32_t* sorted_ids = index;
+    const int32_t* order = sorted_ids + n_ids;
+    const int32_t* run_end = order + n_ids;
+    const int slabs = (int)eisen_ceil_div(hidden, (size_t)kWave * 2);
+    const unsigned blocks = (unsigned)eisen_ceil_div(n_ids * slabs, (size_t)(kThreads / kWave));
+    if (dtype == EISEN_F32) scatter_runs_kernel<float><<<blocks, kThreads, 0, ctx->stream>>>((const float*)go, gw, sorted_ids, order, run_end, (int)n_ids, (int)hidden, slabs);
+    else scatter_runs_kernel<bf16_t><<<blocks, kThreads, 0, ctx->stream>>>((const bf16_t*)go, gw, sorted_ids, order, run_end, (int)n_ids, (int)hidden, slabs);
 }
 
 int scatter_device_route(eisen_ctx* ctx, const int32_t* ids_dev, const void* go, float* gw, int dtype, size_t n_ids, size_t vocab, size_t hidden,
@@ -243,25 +269,13 @@ int scatter_device_route(eisen_ctx* ctx, const int32_t* ids_dev, const void* go,
     void* dev = nullptr;
     int rc = eisen_hip_malloc(ctx, 3 * n_ids * sizeof(int32_t), &dev);
     if (rc) return rc;
-    int32_t* sorted_ids = (int32_t*)dev;
-    int32_t* order = sorted_ids + n_ids;
-    int32_t* run_end = order + n_ids;
     {
         // algorithmic bytes: every row of dOut read once, every touched row of the f32 gradient read and written once; the
         // touched rows are not known on the host here, so the entry counts dOut and the index only (a lower bound)
         EisenProfScope prof(ctx, dtype == EISEN_BF16 ? "scatter_rows_bf16" : "scatter_rows_f32",
                             (double)n_ids * (double)hidden * eisen_dtype_size(dtype) + 16.0 * (double)n_ids);
-        switch (n_pow2 / kSortThreads) {
-            case 1: scatter_sort_kernel<1><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
-            case 2: scatter_sort_kernel<2><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
-            case 4: scatter_sort_kernel<4><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
-            case 8: scatter_sort_kernel<8><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
-            default: scatter_sort_kernel<16><<<1, kSortThreads, 0, ctx->stream>>>(ids_dev, (int)n_ids, shift, (int)vocab, sorted_ids, order, run_end); break;
-        }
-        const int slabs = (int)eisen_ceil_div(hidden, (size_t)kWave * 2);
-        const unsigned blocks = (unsigned)eisen_ceil_div(n_ids * slabs, (size_t)(kThreads / kWave));
-        if (dtype == EISEN_F32) scatter_runs_kernel<float><<<blocks, kThreads, 0, ctx->stream>>>((const float*)go, gw, sorted_ids, order, run_end, (int)n_ids, (int)hidden, slabs);
-        else scatter_runs_kernel<bf16_t><<<blocks, kThreads, 0, ctx->stream>>>((const bf16_t*)go, gw, sorted_ids, order, run_end, (int)n_ids, (int)hidden, slabs);
+        scatter_launch_sort(ctx, ids_dev, n_ids, vocab, n_pow2, shift, (int32_t*)dev);
+        scatter_launch_runs(ctx, (const int32_t*)dev, go, gw, dtype, n_ids, hidden);
     }
     hipError_t e = hipGetLastError();
     const int rc_free = eisen_hip_free(ctx, dev);  // stream-ordered: the block is reused only by later work
@@ -387,4 +401,37 @@ extern "C" int eisen_hip_gather_backward_dev(eisen_ctx* ctx, const int32_t* ids_
     int rc = eisen_hip_dtoh(ctx, host.data(), ids_dev, n_ids * sizeof(int32_t));
     if (rc) return rc;
     return eisen_hip_gather_backward(ctx, host.data(), go, gw, dtype, n_ids, vocab, hidden);
+}
+
+// The two halves of eisen_hip_gather_backward_dev for a caller that knows the ids long before the gradient exists (the token ids
+// of a training step are known when its forward pass starts): the index depends on the ids alone.
+extern "C" int eisen_hip_gather_index_dev(eisen_ctx* ctx, const int32_t* ids_dev, size_t n_ids, size_t vocab, int32_t* index) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, ids_dev && index, EISEN_E_ARG, "gather_index_dev: null pointer");
+    EISEN_REQUIRE(ctx, vocab > 0 && vocab < (size_t(1) << 31), EISEN_E_SHAPE, "gather_index_dev: vocab out of range");
+    if (n_ids == 0) return 0;
+    int n_pow2 = 0, shift = 0;
+    EISEN_REQUIRE(ctx, scatter_index_on_device(n_ids, vocab, &n_pow2, &shift), EISEN_E_SHAPE,
+                  "gather_index_dev: %zu ids of a vocabulary of %zu are more than the device-side index takes", n_ids, vocab);
+    EisenProfScope prof(ctx, "scatter_index", 16.0 * (double)n_ids);
+    scatter_launch_sort(ctx, ids_dev, n_ids, vocab, n_pow2, shift, index);
+    EISEN_LAUNCH_CHECK(ctx, "scatter_sort_kernel");
+    return 0;
+}
+
+extern "C" int eisen_hip_gather_backward_indexed(eisen_ctx* ctx, const int32_t* index, const void* go, float* gw, int dtype, size_t n_ids,
+                                                 size_t vocab, size_t hidden) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, index && go && gw, EISEN_E_ARG, "gather_backward_indexed: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "gather_backward_indexed: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, vocab > 0 && vocab < (size_t(1) << 31) && hidden > 0 && hidden < (size_t(1) << 30), EISEN_E_SHAPE,
+                  "gather_backward_indexed: vocab/hidden out of range");
+    if (n_ids == 0) return 0;
+    int n_pow2 = 0, shift = 0;
+    EISEN_REQUIRE(ctx, scatter_on_device(go, gw, dtype, n_ids, vocab, hidden, &n_pow2, &shift), EISEN_E_SHAPE,
+                  "gather_backward_indexed: rows of %zu values at these addresses need eisen_hip_gather_backward_dev", hidden);
+    EisenProfScope prof(ctx, dtype == EISEN_BF16 ? "scatter_rows_bf16" : "scatter_rows_f32", (double)n_ids * (double)hidden * eisen_dtype_size(dtype) + 16.0 * (double)n_ids);
+    scatter_launch_runs(ctx, index, go, gw, dtype, n_ids, hidden);
+    EISEN_LAUNCH_CHECK(ctx, "scatter_runs_kernel");
+    return 0;
 }

@@ -1155,6 +1155,19 @@ size_t Graph::gather(size_t weights, size_t indices) {
     const size_t out = push_tensor(os, dw.dtype, true);
     check(eisen_hip_htod(ctx_, at(dids).data.ptr, ids.data(), n * sizeof(int32_t)), "gather ids");
     check(eisen_hip_gather(ctx_, dw.ptr, (const int32_t*)at(dids).data.ptr, at(out).data.ptr, dw.dtype, n, vocab, hidden), "gather");
+    // The position index of the backward scatter depends on the ids alone: it is built now, on the side stream beside the
+    // forward pass (one workgroup sorting for tens of microseconds), instead of in front of the last kernel of the backward pass.
+    size_t didx = (size_t)-1;
+    if (!no_grad && !tape_paused && beside_) {
+        didx = push_tensor({3 * n}, EISEN_F32, true);  // int32 payload
+        check(eisen_hip_side_begin(ctx_), "side stream");
+        const int rc = eisen_hip_gather_index_dev(ctx_, (const int32_t*)at(dids).data.ptr, n, vocab, (int32_t*)at(didx).data.ptr);
+        const int rc_end = eisen_hip_side_end(ctx_);  // back on the main stream whatever the call returned
+        side_guards.push_back(at(didx).data.ptr);     // a restore_save_point before any backward pass waits for the sort
+        if (rc == EISEN_E_SHAPE) didx = (size_t)-1;   // a batch the device-side index does not take: backward builds it its own way
+        else check(rc, "gather index");
+        check(rc_end, "side stream");
+    }
     record({weights, indices}, out, [=](Graph& g) {
         const Storage& go = g.grad_for_read(out);
         g.apply_pending_zero(weights);  // the scatter touches only the rows that occur
@@ -1165,8 +1178,14 @@ size_t Graph::gather(size_t weights, size_t indices) {
             if (!acc) g.check(eisen_hip_memset_zero(g.ctx(), gw0.ptr, gw0.numel * (gw0.dtype == EISEN_BF16 ? 2 : 4)), "gather backward");
         }
         if (w.grad.dtype != EISEN_F32) throw Error("gather backward: the embedding gradient must be f32");
-        g.check(eisen_hip_gather_backward_dev(g.ctx(), (const int32_t*)g.at(dids).data.ptr, go.ptr, (float*)w.grad.ptr, go.dtype, n, vocab, hidden),
-                "gather backward");
+        int rc = EISEN_E_SHAPE;
+        if (didx != (size_t)-1) {
+            g.side_join();  // the index (and whatever else the side stream was given) is complete
+            rc = eisen_hip_gather_backward_indexed(g.ctx(), (const int32_t*)g.at(didx).data.ptr, go.ptr, (float*)w.grad.ptr, go.dtype, n, vocab, hidden);
+        }
+        if (rc == EISEN_E_SHAPE)  // no index, or rows the indexed kernel does not take
+            rc = eisen_hip_gather_backward_dev(g.ctx(), (const int32_t*)g.at(dids).data.ptr, go.ptr, (float*)w.grad.ptr, go.dtype, n, vocab, hidden);
+        g.check(rc, "gather backward");
     });
     return out;
 }

@@ -391,6 +391,14 @@ class Context:
         """The scatter with int32 ids already on the device."""
         self._call("eisen_hip_gather_backward_dev", _ptr(ids_dev), _ptr(go), _ptr(gw), _i(dtype), _sz(n_ids), _sz(vocab), _sz(hidden))
 
+    def gather_index_dev(self, ids_dev, n_ids, vocab, index):
+        """The position index of the ordered scatter (3 * n_ids int32, device) from int32 ids on the device."""
+        self._call("eisen_hip_gather_index_dev", _ptr(ids_dev), _sz(n_ids), _sz(vocab), _ptr(index))
+
+    def gather_backward_indexed(self, index, go, gw, dtype, n_ids, vocab, hidden):
+        """The scatter with an index built by gather_index_dev."""
+        self._call("eisen_hip_gather_backward_indexed", _ptr(index), _ptr(go), _ptr(gw), _i(dtype), _sz(n_ids), _sz(vocab), _sz(hidden))
+
     # ---- loss -------------------------------------------------------------------------
     def cross_entropy(self, logits, targets, dlogits, row_loss, loss_out, dtype, rows, classes, normalizer, grad_scale=1.0,
                       argmax_out=None, target_logit_out=None):

@@ -362,6 +362,15 @@ int eisen_hip_gather_backward(eisen_ctx* ctx, const int32_t* ids_host, const voi
  * skipped on the device route. */
 int eisen_hip_gather_backward_dev(eisen_ctx* ctx, const int32_t* ids_dev, const void* go, float* gw, int dtype,
                                   size_t n_ids, size_t vocab, size_t hidden);
+/* eisen_hip_gather_backward_dev in two halves, for a caller that knows the ids long before the gradient exists (the token
+ * ids of a training step are known when its forward pass starts).  _index_dev builds the position index of the ordered
+ * scatter from the ids alone: `index` receives 3 * n_ids int32 (device memory); EISEN_E_SHAPE when the batch is more
+ * than the device-side index takes (more than 16384 ids, or vocab * ids beyond 32 bits): then use _backward_dev.
+ * _backward_indexed adds the rows of dOut into the f32 gradient in ascending position with that index, the result of
+ * eisen_hip_gather_backward_dev bit for bit (src/graph/ops/transform.rs:306-315 is the order it keeps). */
+int eisen_hip_gather_index_dev(eisen_ctx* ctx, const int32_t* ids_dev, size_t n_ids, size_t vocab, int32_t* index);
+int eisen_hip_gather_backward_indexed(eisen_ctx* ctx, const int32_t* index, const void* go, float* gw, int dtype, size_t n_ids,
+                                      size_t vocab, size_t hidden);
 
 /* ---- loss ------------------------------------------------------------------------------ */
 

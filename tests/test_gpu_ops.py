@@ -443,7 +443,19 @@ def test_scatter_index_on_device_and_on_host(ctx, n, vocab, hidden):
         got = dn(ctx, gw, (vocab, hidden), F32)
         assert np.array_equal(got, exp), entry
         gw.free()
-    for b in (dids, dgo):
+    # the index built ahead of the gradient (the ids are known when the forward pass starts), then the indexed scatter:
+    # the same bits where the device-side index takes the batch, a clear refusal where it does not
+    index = ctx.malloc(3 * n * 4)
+    if n <= 16384 and vocab < 2 ** 31 // 16384 and hidden % 2 == 0:
+        ctx.gather_index_dev(dids, n, vocab, index)
+        gw = ctx.upload(gw0)
+        ctx.gather_backward_indexed(index, dgo, gw, BF16, n, vocab, hidden)
+        assert np.array_equal(dn(ctx, gw, (vocab, hidden), F32), exp), "indexed"
+        gw.free()
+    elif n > 16384:
+        with pytest.raises(hip.EisenHipError):
+            ctx.gather_index_dev(dids, n, vocab, index)
+    for b in (dids, dgo, index):
         b.free()
 
 
