@@ -328,7 +328,11 @@ bool Graph::window_take(size_t weight, const void* x, const void* dy, int dtype,
 
 void Graph::flush_weight_gradients() {
     window_passes_ = 0;
-    if (window_dw.empty() && retained_.empty()) return;
+    if (window_dw.empty()) {
+        // nothing waits for a launch; buffers kept for side-stream GEMMs go back once the main stream has waited for them
+        if (!retained_.empty()) side_join();
+        return;
+    }
     std::vector<WindowDW> list;
     list.swap(window_dw);
     // One launch per set of products with the same shape, number of pieces and accumulate state (equal tiles, and for a
