@@ -114,12 +114,31 @@ def test_config5_full_model_micro_step(ctx):
     print(f"\nconfig 5, 4 x 1024 tokens: activation high-water mark {peak_plain / 2**30:.2f} GiB plain, {peak_ck / 2**30:.2f} GiB with per-block recompute")
     assert peak_ck < 0.5 * peak_plain, (peak_plain, peak_ck)
 
+    # ---- the weight-gradient window at full size: the same micro-batch twice in a window of two.  Adding a gradient to
+    # itself in f32 is exact, so the gain gradients, which the window does not hold, double to the bit; the windowed gradients (one
+    # contraction over both passes: five launches, one per shape of weight) double up to the rounding order of an f32 sum
+    gg.set_weight_gradient_window(2)
+    opt.zero_grad()
+    ctx.profile_start()
+    assert lm.micro_step(x, y) == loss and lm.micro_step(x, y) == loss
+    prof = ctx.profile_stop()
+    assert sum(e["launches"] for k, e in prof.items() if k.endswith("_window")) == 5, sorted(prof)
+    shapes = gen.lm_param_shapes(**C5)
+    for p, gr, (name, shape) in zip(params, grads, shapes):
+        got = gg.sync_grad_to_cpu(p)
+        if len(shape) == 2:   # (the embedding's rows are added to occurrence by occurrence in both passes: not an exact doubling either)
+            assert_close(got, 2.0 * gr.astype(np.float64), 1e-4, f"config 5, window of two passes: grad {name}")
+        else:
+            assert np.array_equal(got, 2.0 * gr), f"gradient of {name} is not twice the single pass although the window does not hold it"
+    gg.set_weight_gradient_window(0)
+    ctx.sync()
+    assert ctx.pool_stats()[0] == in_use, "buffers kept for the window were not given back"
+
     # ---- the fused path against the reference's op-by-op chain, all 16 layers (separately oracle-checked kernels)
     lm.set_fused(False)
     opt.zero_grad()
     loss3 = lm.micro_step(x, y)
     assert abs(loss3 - loss) <= 2e-3 * abs(loss), (loss3, loss)
-    shapes = gen.lm_param_shapes(**C5)
     worst = 0.0
     for p, gr, (name, _) in zip(params, grads, shapes):
         un = gg.sync_grad_to_cpu(p)
