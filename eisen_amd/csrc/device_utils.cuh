@@ -106,6 +106,14 @@ __device__ __forceinline__ int lds_swz(int row) {
     return ((row & 3) << 2) | ((row >> 2) & 3);                                                          // a row is one or two bank spans
 }
 
+// Forward rotary embedding of one interleaved pair by the angle whose (cos, sin) is cs: y0 = x0 c - x1 s, y1 = x0 s + x1 c
+// (src/graph/ops/transform.rs:562-566).  The fused multiply-adds are written out so that every kernel that rotates gets
+// the same bits, whatever the compiler would contract elsewhere.
+__device__ __forceinline__ void rope_rotate_forward(float a, float b, float2 cs, float& y0, float& y1) {
+    y0 = __builtin_fmaf(a, cs.x, -(b * cs.y));
+    y1 = __builtin_fmaf(a, cs.y, b * cs.x);
+}
+
 // Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  This
 // renumbering gives XCD j the contiguous id range [j*total/8, (j+1)*total/8), in dispatch order, so
 // workgroups that are neighbours in the renumbered order (and share operands) also share an L2.

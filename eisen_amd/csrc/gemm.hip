@@ -729,11 +729,14 @@ struct SwigluBackwardEpilogue {  // see GemmArgs::gate
     const void* up;
     void* dup;
 };
+struct RopeEpilogue {  // see GemmArgs::rope
+    size_t members, seq, head_dim;
+};
 constexpr int kEpilogueNotFusable = -7001;  // internal: the shape takes a kernel without the fused epilogue
 static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype_ab, int dtype_c, int trans_a,
                        int trans_b, size_t M, size_t N, size_t K, size_t batch, long long sA, long long sB, long long sC,
                        int accumulate, const char* who, const KSegments* segs = nullptr, const void* residual = nullptr,
-                       const SwigluBackwardEpilogue* swiglu = nullptr) {
+                       const SwigluBackwardEpilogue* swiglu = nullptr, const RopeEpilogue* rope = nullptr) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, A && B && C, EISEN_E_ARG, "%s: null pointer", who);
     EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype_ab) && eisen_dtype_ok(dtype_c), EISEN_E_ARG, "%s: unknown dtype", who);
@@ -828,7 +831,25 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
                         (wide_tiles >= 512 || (wide_tiles >= 300 && !wide));
     // 256 x 256 tiles (the gate/up kernel's main loop: an A operand register feeds twice the MFMAs) where the grid still
     // has three rounds of them: the lm_head forward (1035 against 980 TFLOP/s at 4096 x 32000 x 2048)
-    const bool wide256 = mfma_ok && split == 1 && n_more == 0 && a_kc && !b_kc && batch == 1 && dtype_c == EISEN_BF16 && !residual && !swiglu &&
+    if (rope) {
+        // the rotation lives in the staged epilogue of the whole-tile kernels; any other shape is the caller's to rotate
+        // (256x128x64 and 128x128x64 direct-to-LDS kernels, the 64x64x32 kernel without bounds checks: all three stage C through
+        // the LDS, where gemm_store_tile rotates)
+        const bool whole128 = big_tile && M % 128 == 0 && N % 128 == 0 && K % 64 == 0;
+        const bool whole64 = !big_tile && M % 64 == 0 && N % 64 == 0 && K % 32 == 0;
+        static_assert(2 * (OperandTile<64, true, 32, 256>::ELEMS + OperandTile<64, false, 32, 256>::ELEMS) * sizeof(bf16_t) >= 4 * 32 * (32 + 4) * sizeof(float),
+                      "the 64x64x32 kernel's LDS must hold its staged C bands");
+        const bool fits = mfma_ok && split == 1 && n_more == 0 && dtype_c == EISEN_BF16 && !residual && !swiglu && !accumulate && g.vec_c && a_kc && !b_kc &&
+                          (wide || whole128 || whole64) && rope->head_dim % 8 == 0 && N % rope->head_dim == 0 && rope->seq > 0 && rope->seq < (size_t(1) << 24) &&
+                          rope->head_dim < (size_t(1) << 24);
+        if (!fits) return kEpilogueNotFusable;
+        int rc = eisen_rope_table_get(ctx, rope->seq, rope->head_dim, &g.rope);
+        if (rc) return rc;
+        g.rope_seq = (int)rope->seq;
+        g.rope_head_dim = (int)rope->head_dim;
+        g.rope_members = (int)std::min<size_t>(rope->members, batch);
+    }
+    const bool wide256 = mfma_ok && split == 1 && n_more == 0 && a_kc && !b_kc && batch == 1 && dtype_c == EISEN_BF16 && !residual && !swiglu && !rope &&
                          !accumulate && M % 256 == 0 && N % 256 == 0 && K % 32 == 0 && (M / 256) * (N / 256) >= 768 && eisen_aligned(C, 16);
     if (wide256) {
         SwigluForwardArgs a{static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(B), static_cast<const bf16_t*>(B) + 128, static_cast<bf16_t*>(C),
@@ -854,7 +875,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
     }
     const char* tile = !mfma_ok ? "fma64x64" : wide32 ? "256x128x32" : wide ? "256x128x64" : (big_tile || split128) ? (K % 64 == 0 && !(!a_kc && !b_kc && M % 128 == 0 && N % 128 == 0 && tiles128 * split >= 512) ? "128x128x64" : "128x128x32") : "64x64x32";
     snprintf(pname, sizeof(pname), "gemm_%s%s_%s_%s_%s%s", trans_a ? "t" : "n", trans_b ? "t" : "n", dtype_ab == EISEN_BF16 ? "bf16" : "f32",
-             dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : swiglu ? "_swiglu_bwd" : "");
+             dtype_c == EISEN_BF16 ? "bf16out" : "f32out", tile, split > 1 ? "_splitk" : swiglu ? "_swiglu_bwd" : rope ? "_rope" : "");
     EisenProfScope prof(ctx, pname, 2.0 * (double)M * (double)N * (double)K * (double)batch, true);
     if (mfma_ok) {
         if (split > 1) {
@@ -925,6 +946,30 @@ extern "C" int eisen_hip_gemm_strided_batched(eisen_ctx* ctx, const void* A, con
                                               long long stride_b, long long stride_c, int accumulate) {
     return gemm_common(ctx, A, B, C, dtype_ab, dtype_c, trans_a, trans_b, M, N, K, batch, stride_a, stride_b, stride_c, accumulate,
                        "eisen_hip_gemm_strided_batched");
+}
+
+extern "C" int eisen_hip_gemm_rope(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype, size_t batch, size_t M, size_t N, size_t K,
+                                   long long stride_b, long long stride_c, size_t rope_members, size_t seq, size_t head_dim) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, A && B && C, EISEN_E_ARG, "eisen_hip_gemm_rope: null pointer");
+    EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_gemm_rope: unknown dtype %d", dtype);
+    EISEN_REQUIRE(ctx, rope_members <= batch, EISEN_E_ARG, "eisen_hip_gemm_rope: %zu rotated members of %zu", rope_members, batch);
+    EISEN_REQUIRE(ctx, seq > 0 && M % seq == 0, EISEN_E_SHAPE, "eisen_hip_gemm_rope: %zu rows are not whole sequences of %zu", M, seq);
+    EISEN_REQUIRE(ctx, head_dim >= 2 && head_dim % 2 == 0 && N % head_dim == 0, EISEN_E_SHAPE,
+                  "eisen_hip_gemm_rope: %zu columns must be a multiple of an even head_dim (%zu)", N, head_dim);
+    if (batch == 0 || M == 0 || N == 0) return 0;
+    const RopeEpilogue rope{rope_members, seq, head_dim};
+    int rc = kEpilogueNotFusable;
+    if (rope_members > 0 && K > 0)
+        rc = gemm_common(ctx, A, B, C, dtype, dtype, 0, 0, M, N, K, batch, 0, stride_b, stride_c, 0, "eisen_hip_gemm_rope", nullptr, nullptr, nullptr, &rope);
+    if (rc != kEpilogueNotFusable) return rc;
+    // the product, then the rotation in place, member by member
+    rc = gemm_common(ctx, A, B, C, dtype, dtype, 0, 0, M, N, K, batch, 0, stride_b, stride_c, 0, "eisen_hip_gemm_rope");
+    for (size_t b = 0; b < rope_members && !rc; b++) {
+        void* Cb = static_cast<char*>(C) + (long long)b * stride_c * (long long)eisen_dtype_size(dtype);
+        rc = eisen_hip_rope(ctx, Cb, Cb, dtype, M / seq, seq, N, head_dim);
+    }
+    return rc;
 }
 
 extern "C" int eisen_hip_gemm_ksegments(eisen_ctx* ctx, size_t n_segments, const void* const* A, const void* const* B, const size_t* K,

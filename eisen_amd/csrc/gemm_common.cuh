@@ -43,6 +43,10 @@ struct GemmArgs {
     const void* B_seg[2];
     int lda_seg[2], ldb_seg[2];
     int seg_end[2];
+    // Rotary-embedding epilogue (rope != nullptr; bf16 C, whole tiles, no accumulation, residual or split): the batch members
+    // below rope_members leave as rope(A*B), row m at position m % rope_seq, heads of rope_head_dim columns (a multiple of 8)
+    const float2* rope;                // cos/sin table [>= rope_seq][rope_head_dim / 2]
+    int rope_seq, rope_head_dim, rope_members;
 };
 
 // gemm_wide.hip: 256 x 256 tiles, four waves of 128 x 128 (plain products, whole tiles only)
@@ -178,6 +182,21 @@ __device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)
                 } else {
                     TC* dst = C + (long long)m * g.ldc + n;
                     Pack<TC> o[8 / Pack<TC>::N];
+                    if constexpr (sizeof(TC) == 2) {
+                        if (g.rope && bz < g.rope_members) {
+                            // the product rounded to bf16 and then rotated, as the separate rotary kernel would find it
+                            const float4* cs = reinterpret_cast<const float4*>(g.rope + (long long)(m % g.rope_seq) * (g.rope_head_dim >> 1) +
+                                                                               ((n % g.rope_head_dim) >> 1));
+#pragma unroll
+                            for (int q = 0; q < 2; q++) {
+                                const float4 t = cs[q];
+                                const float a0 = to_f32(from_f32<TC>(val[4 * q])), b0 = to_f32(from_f32<TC>(val[4 * q + 1]));
+                                const float a1 = to_f32(from_f32<TC>(val[4 * q + 2])), b1 = to_f32(from_f32<TC>(val[4 * q + 3]));
+                                rope_rotate_forward(a0, b0, make_float2(t.x, t.y), val[4 * q], val[4 * q + 1]);
+                                rope_rotate_forward(a1, b1, make_float2(t.z, t.w), val[4 * q + 2], val[4 * q + 3]);
+                            }
+                        }
+                    }
                     if (add_old) {
                         const TC* src = Rsrc + (long long)m * g.ldc + n;
 #pragma unroll

@@ -754,9 +754,11 @@ size_t Graph::swiglu_matmul_residual(size_t gate, size_t up, size_t b, size_t r,
 // fewer launches: equally shaped neighbours (K and V, gate and up) run as a batch of two whose "stride" is the
 // distance between the two tensors, forward and for dW; the input gradient of the whole group is one GEMM
 // whose contraction runs over the outputs of all members, written once.
-std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws, const std::vector<size_t>& collect_dw, size_t* swiglu_h, bool defer_dw) {
+std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws, const std::vector<size_t>& collect_dw, size_t* swiglu_h, bool defer_dw,
+                                        size_t rope_members, size_t rope_head_dim, bool* rotated) {
     const std::vector<size_t> sa = at(a).shape;
     const size_t n = ws.size();
+    if (rotated) *rotated = false;
     const Storage da = compute_data(a);
     bool ok = n >= 2 && n <= 3 && !sa.empty() && da.dtype == EISEN_BF16;
     for (size_t i = 0; i < n && ok; i++)
@@ -789,13 +791,25 @@ std::vector<size_t> Graph::matmul_group(size_t a, const std::vector<size_t>& ws,
         check(eisen_hip_gemm_swiglu_forward(ctx_, da.ptr, compute_data(ws[0]).ptr, compute_data(ws[1]).ptr, at(outs[0]).data.ptr, at(outs[1]).data.ptr,
                                             at(*swiglu_h).data.ptr, da.dtype, M, N[0], K),
               "matmul_group");
+    // rotary embedding of the first outputs by the kernel that forms them ([batch, seq, hidden] inputs, whole heads)
+    size_t rope_n = (rotated && !swiglu_h && sa.size() == 3 && sa[1] > 0 && rope_head_dim >= 8 && rope_head_dim % 8 == 0) ? std::min(rope_members, n) : 0;
+    for (size_t i = 0; i < rope_n; i++)
+        if (N[i] % rope_head_dim) rope_n = 0;
+    if (rope_n > 0) *rotated = true;
+    const size_t seq = sa.size() == 3 ? sa[1] : 0;
     for (size_t i = 0; i < n && !with_h; i++) {
         const Storage w = compute_data(ws[i]);
         if (pair[i]) {
             const ptrdiff_t wd = ((const char*)compute_data(ws[i + 1]).ptr - (const char*)w.ptr) / 2;
             const ptrdiff_t od = ((const char*)at(outs[i + 1]).data.ptr - (const char*)at(outs[i]).data.ptr) / 2;
-            check(eisen_hip_gemm_strided_batched(ctx_, da.ptr, w.ptr, at(outs[i]).data.ptr, da.dtype, da.dtype, 0, 0, 2, M, N[i], K, 0, wd, od, 0), "matmul_group");
+            const size_t members = (i < rope_n ? 1 : 0) + (i + 1 < rope_n ? 1 : 0);
+            if (members > 0)
+                check(eisen_hip_gemm_rope(ctx_, da.ptr, w.ptr, at(outs[i]).data.ptr, da.dtype, 2, M, N[i], K, wd, od, members, seq, rope_head_dim), "matmul_group");
+            else
+                check(eisen_hip_gemm_strided_batched(ctx_, da.ptr, w.ptr, at(outs[i]).data.ptr, da.dtype, da.dtype, 0, 0, 2, M, N[i], K, 0, wd, od, 0), "matmul_group");
             i++;
+        } else if (i < rope_n) {
+            check(eisen_hip_gemm_rope(ctx_, da.ptr, w.ptr, at(outs[i]).data.ptr, da.dtype, 1, M, N[i], K, 0, 0, 1, seq, rope_head_dim), "matmul_group");
         } else {
             check(eisen_hip_gemm(ctx_, da.ptr, w.ptr, at(outs[i]).data.ptr, da.dtype, da.dtype, 0, 0, M, N[i], K, 0), "matmul_group");
         }
@@ -1330,7 +1344,7 @@ size_t Graph::attention_gqa(size_t q, size_t k, size_t v, size_t heads, size_t k
 // `g.rope(q)`, `g.rope(k)` and the attention chain (src/nn/attention.rs:316-375) as one node.  Forward: the two
 // rotary kernels into internal tensors, then the fused attention.  Backward: one attention backward whose
 // kernels un-rotate dQ and dK as they store them, so the gradients land directly on the projections.
-size_t Graph::attention_gqa_rope(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal) {
+size_t Graph::attention_gqa_rope(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal, bool prerotated) {
     const std::vector<size_t> sq = at(q).shape, sk = at(k).shape;
     if (sq.size() != 3 || sk.size() != 3 || at(v).shape != sk) throw Error("attention_gqa_rope: expects q [B,S,Hq*hd], k/v [B,S,Hkv*hd]");
     if (heads == 0 || kv_heads == 0 || sq[2] % heads || heads % kv_heads) throw Error("attention_gqa_rope: bad head counts");
@@ -1338,8 +1352,12 @@ size_t Graph::attention_gqa_rope(size_t q, size_t k, size_t v, size_t heads, siz
     if (sk[2] != kv_heads * hd || sk[0] != B || sk[1] != S) throw Error("attention_gqa_rope: k/v shape does not match q");
     const Storage dq = compute_data(q), dk = compute_data(k), dv = compute_data(v);
     if (dq.dtype != dk.dtype || dq.dtype != dv.dtype) throw Error("attention_gqa_rope: q, k, v must share an element type");
-    const size_t q_rot = push_tensor(sq, dq.dtype, true), k_rot = push_tensor(sk, dk.dtype, true);  // kept for backward
-    check(eisen_hip_rope_pair(ctx_, dq.ptr, at(q_rot).data.ptr, sq[2], dk.ptr, at(k_rot).data.ptr, sk[2], dq.dtype, B, S, hd), "rope");
+    size_t q_rot = q, k_rot = k;
+    if (!prerotated) {
+        q_rot = push_tensor(sq, dq.dtype, true);  // kept for backward
+        k_rot = push_tensor(sk, dk.dtype, true);
+        check(eisen_hip_rope_pair(ctx_, dq.ptr, at(q_rot).data.ptr, sq[2], dk.ptr, at(k_rot).data.ptr, sk[2], dq.dtype, B, S, hd), "rope");
+    }
     const size_t out = alloc_pooled_dtype(sq, dq.dtype);
     const size_t lse = alloc_pooled_dtype({B, heads, S}, EISEN_F32);
     check(eisen_hip_attention_forward(ctx_, at(q_rot).data.ptr, at(k_rot).data.ptr, dv.ptr, at(out).data.ptr, (float*)at(lse).data.ptr, dq.dtype, B, S,

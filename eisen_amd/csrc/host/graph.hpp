@@ -126,8 +126,12 @@ class Graph {
     // collect_dw: weights whose deferred gradient GEMMs join this group's dW launch; defer_dw: this group's own weight
     // gradients are left for a later group that names them; swiglu_h: receives the id of silu(out0) * out1 when the
     // kernel that forms it with the two products ran, (size_t)-1 otherwise
+    // rope_members / rope_head_dim / rotated: the first rope_members outputs may leave rotary-embedded (`rope` applied to
+    // a [batch, seq, hidden] product by the kernel that forms it); *rotated says whether they did.  Such an output stands for
+    // rope(a w): its consumer (attention_gqa_rope with prerotated) leaves the gradient of the un-rotated product a w in its
+    // gradient buffer, which is what this group's backward multiplies.
     std::vector<size_t> matmul_group(size_t a, const std::vector<size_t>& weights, const std::vector<size_t>& collect_dw = {}, size_t* swiglu_h = nullptr,
-                                     bool defer_dw = false);
+                                     bool defer_dw = false, size_t rope_members = 0, size_t rope_head_dim = 0, bool* rotated = nullptr);
     size_t matmul_bf16(size_t a, size_t b) { return matmul(a, b); }
     size_t matmul_trans_b(size_t a, size_t b);
     size_t bmm(size_t a, size_t b, bool trans_b);
@@ -146,7 +150,8 @@ class Graph {
     // q [B,S,Hq*hd], k/v [B,S,Hkv*hd] straight from the projections -> [B,S,Hq*hd].
     size_t attention_gqa(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal);
     // the same with the rotary embedding of q and k inside: rope(q), rope(k) -> attention; backward stores d q, d k un-rotated
-    size_t attention_gqa_rope(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal);
+    // prerotated: q and k already are rope(q0), rope(k0) (matmul_group with *rotated); d q0, d k0 are stored all the same
+    size_t attention_gqa_rope(size_t q, size_t k, size_t v, size_t heads, size_t kv_heads, float scale, bool causal, bool prerotated = false);
 
     // src/graph/mod.rs:670-796
     void backward(size_t loss_id);

@@ -89,13 +89,16 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
     if (xs.size() != 3) throw Error("GQA requires [Batch, Seq, Dim]");
     const size_t batch = xs[0], seq = xs[1];
     size_t q, k, v;
+    bool rotated = false;  // q and k left their projection kernels rotary-embedded
     if (collects()) {
         // the three projections read the same input: K and V as one launch, one input-gradient GEMM for all
         // (the group also collects the output projection's weight gradient when that projection defers it: four dW GEMMs, one launch)
         const bool defer_out = residual != (size_t)-1 && !out_proj.has_bias;
         std::vector<size_t> collect = collect_dw;
         if (defer_out) collect.insert(collect.begin(), out_proj.weight_id);
-        const std::vector<size_t> qkv = g.matmul_group(x_id, {q_proj.weight_id, k_proj.weight_id, v_proj.weight_id}, collect);
+        const bool kernel_attention = fused && (!g.uses_bf16_mixed_precision() || head_dim == 32 || head_dim == 64 || head_dim == 128);
+        const std::vector<size_t> qkv = g.matmul_group(x_id, {q_proj.weight_id, k_proj.weight_id, v_proj.weight_id}, collect, nullptr, false,
+                                                       kernel_attention ? 2 : 0, head_dim, &rotated);
         q = qkv[0]; k = qkv[1]; v = qkv[2];
         for (size_t t : qkv) g.reinterpret_shape(t, {batch, seq, g.at(t).shape.back()});
     } else {
@@ -111,7 +114,7 @@ size_t GroupedQueryAttention::forward_with_mask(Graph& g, size_t x_id, bool caus
     size_t ctx_flat;
     if (fused_attention) {
         // one op for the rotary embedding and steps 3-11: head split, GQA repeat, scores, scale, mask, softmax, P V, merge
-        ctx_flat = g.attention_gqa_rope(q, k, v, num_heads, num_kv_heads, scale, causal);
+        ctx_flat = g.attention_gqa_rope(q, k, v, num_heads, num_kv_heads, scale, causal, rotated);
     } else {
         const size_t q_rope = g.rope(q, head_dim), k_rope = g.rope(k, head_dim);
         const size_t q4 = g.reshape(q_rope, {batch, seq, num_heads, head_dim});

@@ -65,8 +65,7 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ in
                 r0 = a * cs.x + b * cs.y;
                 r1 = -a * cs.y + b * cs.x;
             } else {
-                r0 = a * cs.x - b * cs.y;
-                r1 = a * cs.y + b * cs.x;
+                rope_rotate_forward(a, b, cs, r0, r1);
             }
             o.set(2 * j, accumulate ? o.get(2 * j) + r0 : r0);
             o.set(2 * j + 1, accumulate ? o.get(2 * j + 1) + r1 : r1);
@@ -99,8 +98,10 @@ __global__ __launch_bounds__(kThreads) void rope_pair_kernel(const T* __restrict
         for (int j = 0; j < N / 2; j++) {
             const float2 cs = table[(size_t)pos * half + pair0 + j];
             const float a = v.get(2 * j), b = v.get(2 * j + 1);
-            o.set(2 * j, a * cs.x - b * cs.y);
-            o.set(2 * j + 1, a * cs.y + b * cs.x);
+            float r0, r1;
+            rope_rotate_forward(a, b, cs, r0, r1);
+            o.set(2 * j, r0);
+            o.set(2 * j + 1, r1);
         }
         store_pack(out + pk * N, o);
     }

@@ -279,6 +279,10 @@ class Context:
     def rope_pair(self, q, q_out, hidden_q, k, k_out, hidden_k, dtype, batch, seq, head_dim):
         self._call("eisen_hip_rope_pair", _ptr(q), _ptr(q_out), _sz(hidden_q), _ptr(k), _ptr(k_out), _sz(hidden_k), _i(dtype), _sz(batch), _sz(seq), _sz(head_dim))
 
+    def gemm_rope(self, A, B, Cm, dtype, batch, M, N, K, stride_b, stride_c, rope_members, seq, head_dim):
+        self._call("eisen_hip_gemm_rope", _ptr(A), _ptr(B), _ptr(Cm), _i(dtype), _sz(batch), _sz(M), _sz(N), _sz(K), C.c_longlong(stride_b),
+                   C.c_longlong(stride_c), _sz(rope_members), _sz(seq), _sz(head_dim))
+
     def rope_backward(self, go, gx, dtype, batch, seq, hidden, head_dim, accumulate=0):
         self._call("eisen_hip_rope_backward", _ptr(go), _ptr(gx), _i(dtype), _sz(batch), _sz(seq), _sz(hidden), _sz(head_dim), _i(accumulate))
 

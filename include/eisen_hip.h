@@ -207,6 +207,16 @@ int eisen_hip_rope(eisen_ctx* ctx, const void* x, void* out, int dtype, size_t b
 int eisen_hip_rope_backward(eisen_ctx* ctx, const void* go, void* gx, int dtype, size_t batch, size_t seq,
                             size_t hidden, size_t head_dim, int accumulate);
 
+/* rope(x W) as one kernel: a projection of GroupedQueryAttention::forward_with_mask with the `g.rope` that follows it
+ * (src/nn/attention.rs:300-305, :316-317; Graph::matmul, src/graph/ops/linear.rs:235-259, then Graph::rope,
+ * src/graph/ops/transform.rs:467-610).  A [M, K] (M = batches of `seq` rows) is shared by `batch` products with their own
+ * B [K, N] (stride_b elements apart) and C [M, N] (stride_c apart); the first `rope_members` of them leave rotated
+ * (heads of `head_dim` columns, row m at position m % seq), the others as plain products (the v projection beside k).
+ * The product is rounded to the element type before it is rotated: the same bits as eisen_hip_gemm followed by
+ * eisen_hip_rope, which is also what shapes outside the fused kernel's tiles run. */
+int eisen_hip_gemm_rope(eisen_ctx* ctx, const void* A, const void* B, void* C, int dtype, size_t batch, size_t M, size_t N, size_t K,
+                        long long stride_b, long long stride_c, size_t rope_members, size_t seq, size_t head_dim);
+
 /* eisen_hip_rope of two tensors that share batch, seq and head_dim in one launch: the q and k projections of
  * GroupedQueryAttention::forward_with_mask (src/nn/attention.rs:304-305, two `g.rope` calls). */
 int eisen_hip_rope_pair(eisen_ctx* ctx, const void* q, void* q_out, size_t hidden_q, const void* k, void* k_out, size_t hidden_k, int dtype,

@@ -313,6 +313,48 @@ def test_rope_pair(ctx, dtype):
         t.free()
 
 
+@pytest.mark.parametrize("case", [
+    # dtype, batch, rotated members, rows (sequences of seq), N, K, seq, head_dim
+    (BF16, 1, 1, 4096, 2048, 256, 1024, 64),   # 256 tiles of 256 x 128: the rotation runs in the product's epilogue
+    (BF16, 2, 1, 1024, 512, 128, 256, 64),     # a K|V pair of 128 x 128 tiles: K rotated, V plain
+    (BF16, 2, 2, 512, 256, 64, 128, 32),       # a Q|K pair, both rotated
+    (BF16, 2, 1, 512, 64, 256, 256, 32),       # a narrow K|V pair on 64 x 64 tiles
+    (BF16, 2, 1, 96, 64, 40, 32, 16),          # ragged: the product, then the rotation in place
+    (BF16, 1, 0, 256, 128, 64, 64, 32),        # nothing to rotate
+    (F32, 2, 1, 64, 32, 24, 16, 8),
+], ids=["256x128", "kv_pair", "qk_pair", "kv_pair_64", "ragged", "plain", "f32"])
+def test_gemm_rope_is_the_product_followed_by_the_rotation(ctx, case):
+    # rope(x W) from one call = eisen_hip_gemm followed by eisen_hip_rope, bit for bit (the product is rounded to the
+    # element type before it is rotated), and matches the oracle's matmul + rope
+    dtype, batch, members, M, N, K, seq, hd = case
+    x = prep(gen.normal(650, (M, K)) * 0.5, dtype)
+    w = prep(gen.normal(651, (batch, K, N)) * 0.2, dtype)
+    es = 2 if dtype == BF16 else 4
+    dx, dw = up(ctx, x, dtype), up(ctx, w, dtype)
+    got, ref = ctx.malloc(batch * M * N * es), ctx.malloc(batch * M * N * es)
+    ctx.profile_start()
+    ctx.gemm_rope(dx, dw, got, dtype, batch, M, N, K, K * N, M * N, members, seq, hd)
+    names = list(ctx.profile_stop())
+    # whole tiles of a kernel that stages C: one launch, no separate rotation
+    one_kernel = dtype == BF16 and members > 0 and M % 64 == 0 and N % 64 == 0 and K % 32 == 0
+    assert any(n.endswith("_rope") for n in names) == one_kernel and (not one_kernel or len(names) == 1), names
+    ctx.gemm_strided_batched(dx, dw, ref, dtype, dtype, 0, 0, batch, M, N, K, 0, K * N, M * N, 0)
+    plain = dn(ctx, ref, (batch, M, N), dtype)
+    for b in range(members):
+        part = ref.ptr + b * M * N * es
+        ctx.rope(part, part, dtype, M // seq, seq, N, hd)
+    a, e = dn(ctx, got, (batch, M, N), dtype), dn(ctx, ref, (batch, M, N), dtype)
+    assert np.array_equal(a, e)
+    for b in range(members, batch):
+        assert np.array_equal(a[b], plain[b])
+    for b in range(members):
+        want = R.rope_fwd(R.matmul_fwd(x, w[b]).reshape(M // seq, seq, N), hd).reshape(M, N)
+        assert_close(a[b], want, tol_for(dtype), "gemm_rope member %d" % b)
+        assert not np.array_equal(a[b], plain[b])
+    for t in (dx, dw, got, ref):
+        t.free()
+
+
 def test_rope_reference_vector(ctx):
     # tests/gpu_kernels.rs:485-513
     x = np.ones((1, 2, 4), np.float32)
