@@ -225,6 +225,9 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
         const int q0 = (qblk * QS + qsub) * 32, q = q0 + c;
         const bool valid_q = q < a.S;
         const long long qoff = b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
+        // the first K / V tile travels with the rows of Q, dO and O, not behind the reduction that waits for them
+        kv_tile.load(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
+        kv_tile.load(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
 
         bf16x8 qf[KSTEPS], dof[KSTEPS];
         float dpart = 0.f;
@@ -255,8 +258,6 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
         const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
         const int my_qmax = q0 < a.S ? q0 + 31 : -1;
 
-        kv_tile.load(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
-        kv_tile.load(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
         auto tile = [&](int kt, auto masked_c) {
             constexpr bool MASKED = decltype(masked_c)::value;  // false: no key of the tile is masked for this wave
             const bf16_t* Ks = Ksb[kt & 1];
