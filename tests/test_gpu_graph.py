@@ -430,6 +430,16 @@ def test_config5_block_shape_bf16_mixed_step(ctx):
     _train_steps(ctx, cfg, G.BF16_MIXED, 2, 128, steps=1, accum=1, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
 
 
+def test_equal_query_and_kv_heads_bf16_mixed_step(ctx):
+    """No GQA (4 query heads, 4 K/V heads, head_dim 64): Q and K have one shape, so they leave one batched launch, both
+    rotary-embedded by its epilogue, and V a plain one; and head_dim 32 with 512 tokens, where the three projections are
+    whole 128 x 128 tiles."""
+    cfg = dict(vocab=512, hidden=256, heads=4, kv_heads=4, ffn=512, layers=2, tie=False)
+    _train_steps(ctx, cfg, G.BF16_MIXED, 2, 128, steps=1, accum=2, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
+    cfg = dict(vocab=512, hidden=256, heads=8, kv_heads=8, ffn=512, layers=1, tie=False)
+    _train_steps(ctx, cfg, G.BF16_MIXED, 2, 256, steps=1, accum=1, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
+
+
 def test_wide_ffn_bf16_mixed_step(ctx):
     """2048 tokens through a 128 -> 4096 -> 128 feed-forward block: large enough for the kernel that forms gate, up and
     silu(gate) * up in one launch and for the wide-tile GEMMs behind it; head_dim 64, 2:1 GQA."""
