@@ -306,6 +306,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
     using I0 = std::integral_constant<int, 0>;
     using IN = std::integral_constant<int, NLOADS>;
     const int nk = (k_hi - k_lo) / BK;
+    // One workgroup per CU (slabs of 64) and bf16 C: what the epilogue adds to or multiplies with travels with the first slabs.
+    constexpr bool kPrefetch = sizeof(TC) == 2 && BK == 64;
+    using Pre = std::conditional_t<kPrefetch, TileEpilogueReads<BM, BN, WGM, WGN, SWIGLU_BWD>, NoEpilogueReads>;
+    Pre pre;
+    if constexpr (kPrefetch) pre.fetch(g, reinterpret_cast<const bf16_t*>(Rsrc), add_old, bz, part, m0, n0, wm, wn, lane);
     issue(locate(0, 0), I0{}, IN{});
     if (nk > 1) issue(locate(1, 1), I0{}, IN{});
     int stage = 0;
@@ -378,8 +383,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
     for (; kt + 2 < nk; kt++) slab(kt, std::true_type{});
     for (; kt < nk; kt++) slab(kt, std::false_type{});
     barrier_no_fence();  // the staging epilogue reuses the operand LDS
-    gemm_store_tile<BM, BN, WGM, WGN, false, sizeof(lds), TC>(g, acc, reinterpret_cast<float*>(&lds[0][0]), C, Rsrc, add_old, bz, split, part,
-                                                              m0, n0, wave, wm, wn, lane);
+    gemm_store_tile<BM, BN, WGM, WGN, false, sizeof(lds), TC, Pre>(g, acc, reinterpret_cast<float*>(&lds[0][0]), C, Rsrc, add_old, bz, split, part,
+                                                                   m0, n0, wave, wm, wn, lane, pre);
 }
 
 // ---- gate and up projections with the SwiGLU in the epilogue ----------------------------------------

@@ -114,13 +114,61 @@ __device__ __forceinline__ void swiglu_backward_elem(float gate, float up, float
     dup = dh * silu;
 }
 
+// What the staged epilogue of gemm_store_tile reads back from memory (the old C or the residual it adds to; gate and up of
+// the SwiGLU-backward epilogue), requested when the kernel starts instead of band by band behind the epilogue's fences,
+// where every pass of every band waits a memory latency of its own with nothing else running on the CU.  One 16-byte
+// packet per band, pass and tensor: bf16 C only.  SECOND: the kernel also holds the `up` packets (the instantiations for
+// the SwiGLU backward).  Every member is written on every path, so the packets stay in registers.
+template <int BM, int BN, int WGM, int WGN, bool SECOND>
+struct TileEpilogueReads {
+    static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, LPR = WN / 8, PASSES = 32 * LPR / 64;
+    static constexpr bool kSecond = SECOND;
+    Pack<bf16_t> first[TM][PASSES];
+    Pack<bf16_t> second[SECOND ? TM : 1][SECOND ? PASSES : 1];
+    bool have_first, have_second;
+    __device__ __forceinline__ void fetch(const GemmArgs& g, const bf16_t* Rsrc, bool add_old, int bz, int part, int m0, int n0, int wm, int wn, int lane) {
+        const bool gate = g.gate != nullptr && SECOND;
+        // partial sums of a split contraction read nothing; unaligned C takes the scalar epilogue
+        const bool need = part == 0 && g.vec_c && (gate || (add_old && g.gate == nullptr));
+        have_first = need;
+        have_second = need && gate;
+        Pack<bf16_t> zero;
+#pragma unroll
+        for (int e = 0; e < 8; e++) zero.set(e, 0.f);
+        second[0][0] = zero;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ps++) {
+                const int idx = ps * 64 + lane, r = idx / LPR, cg = idx % LPR;
+                const int m = m0 + wm * WM + i * 32 + r, n = n0 + wn * WN + cg * 8;
+                Pack<bf16_t> v1 = zero, v2 = zero;
+                if (need) {
+                    if (gate) {
+                        const long long at = (long long)bz * g.sC + (long long)m * g.ldc + n;
+                        v1 = load_pack(static_cast<const bf16_t*>(g.gate) + at);
+                        v2 = load_pack(static_cast<const bf16_t*>(g.up) + at);
+                    } else {
+                        v1 = load_pack(Rsrc + (long long)m * g.ldc + n);
+                    }
+                }
+                first[i][ps] = v1;
+                if constexpr (SECOND) second[i][ps] = v2;
+            }
+    }
+};
+struct NoEpilogueReads {
+    static constexpr bool kSecond = false;
+};
+
 // Epilogue shared by the MFMA kernels.  Accumulator register v of lane l holds
 // C[8*(v/4) + 4*(l/32) + v%4][l%32] of its 32x32 tile.  `lds_f32` is the operand LDS (LDS_BYTES bytes), idle by now
 // and used as a staging area.
-template <int BM, int BN, int WGM, int WGN, bool EDGE, size_t LDS_BYTES, typename TC>
+template <int BM, int BN, int WGM, int WGN, bool EDGE, size_t LDS_BYTES, typename TC, typename PRE = NoEpilogueReads>
 __device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], float* lds_f32, TC* C,
                                                 const TC* Rsrc, bool add_old, int bz, int split, int part, int m0, int n0, int wave,
-                                                int wm, int wn, int lane) {
+                                                int wm, int wn, int lane, const PRE& pre = PRE{}) {
+    constexpr bool kPre = !std::is_same<PRE, NoEpilogueReads>::value;  // pre.first / pre.second may hold what the staged epilogue reads
     constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     float* P = part > 0 ? g.partial + ((long long)bz * (split - 1) + (part - 1)) * g.M * g.N : nullptr;
     constexpr int SP = WN + 4;  // staging pitch in floats
@@ -160,10 +208,20 @@ __device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)
                     const TC* gsrc = static_cast<const TC*>(g.gate) + at;
                     const TC* usrc = static_cast<const TC*>(g.up) + at;
                     Pack<TC> og[8 / Pack<TC>::N], ou[8 / Pack<TC>::N];
+                    bool loaded = false;
+                    if constexpr (kPre && PRE::kSecond && sizeof(TC) == 2) {
+                        if (pre.have_second) {
+                            og[0] = pre.first[i][ps];
+                            ou[0] = pre.second[i][ps];
+                            loaded = true;
+                        }
+                    }
+                    if (!loaded) {
 #pragma unroll
-                    for (int k = 0; k < 8 / Pack<TC>::N; k++) {
-                        og[k] = load_pack(gsrc + k * Pack<TC>::N);
-                        ou[k] = load_pack(usrc + k * Pack<TC>::N);
+                        for (int k = 0; k < 8 / Pack<TC>::N; k++) {
+                            og[k] = load_pack(gsrc + k * Pack<TC>::N);
+                            ou[k] = load_pack(usrc + k * Pack<TC>::N);
+                        }
                     }
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
@@ -198,9 +256,18 @@ __device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)
                         }
                     }
                     if (add_old) {
-                        const TC* src = Rsrc + (long long)m * g.ldc + n;
+                        bool loaded = false;
+                        if constexpr (kPre && sizeof(TC) == 2) {
+                            if (pre.have_first) {  // (never set together with a gate: that epilogue is the branch above)
+                                o[0] = pre.first[i][ps];
+                                loaded = true;
+                            }
+                        }
+                        if (!loaded) {
+                            const TC* src = Rsrc + (long long)m * g.ldc + n;
 #pragma unroll
-                        for (int k = 0; k < 8 / Pack<TC>::N; k++) o[k] = load_pack(src + k * Pack<TC>::N);
+                            for (int k = 0; k < 8 / Pack<TC>::N; k++) o[k] = load_pack(src + k * Pack<TC>::N);
+                        }
 #pragma unroll
                         for (int e = 0; e < 8; e++) val[e] += o[e / Pack<TC>::N].get(e % Pack<TC>::N);
                     }
