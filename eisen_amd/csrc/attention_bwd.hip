@@ -72,27 +72,24 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
     Loader loader;
     loader.init(a.q_ss, 0, lane);
 
+    // K and V rows of this lane's key of key block kb_, as they are stored
+    bf16x8 kraw[KSTEPS], vraw[KSTEPS];
+    auto load_kv = [&](int kb_) {
+        const int key_ = kb_ * 32 + c;
+        const long long koff = b * a.k_sb + kvh * a.k_sh + (long long)key_ * a.k_ss;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; st++) {
+            const int d = st * 16 + 8 * g;
+            kraw[st] = key_ < a.S ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.K) + koff + d) : zero8;
+            vraw[st] = key_ < a.S ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.V) + koff + d) : zero8;
+        }
+    };
+
     for (int pass = 0; pass < 2; pass++) {
         const int kb = pass == 0 ? pair : n_qt - 1 - pair;
         if (pass == 1 && kb <= pair) break;  // odd block count: the middle block has no mirror
         const int k0 = kb * 32, key = k0 + c;
-        bf16x8 kf[KSTEPS], vn[KSTEPS];  // K and -V of the 32 keys, MFMA B operands
-        {
-            const long long koff = b * a.k_sb + kvh * a.k_sh + (long long)key * a.k_ss;
-#pragma unroll
-            for (int st = 0; st < KSTEPS; st++) {
-                const int d = st * 16 + 8 * g;
-                kf[st] = key < a.S ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.K) + koff + d) : zero8;
-                vn[st] = key < a.S ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.V) + koff + d) : zero8;
-                typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-                u32x4 bits = __builtin_bit_cast(u32x4, vn[st]) ^ 0x80008000u;  // sign flip of the eight bf16 values
-                vn[st] = __builtin_bit_cast(bf16x8, bits);
-                // the flip is done here, once, not again at every use; and both operands have arrived before the loop (a
-                // pending load of theirs would make the compiler wait for every outstanding load at their first use in it,
-                // the prefetched tile's included)
-                asm volatile("" : "+v"(vn[st]), "+v"(kf[st]));
-            }
-        }
+        if (pass == 0) load_kv(kb);  // the second pass's rows were requested before the first pass's reduction
         f32x16 dk[DT], dv[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
@@ -133,6 +130,18 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
         };
 
         if (n_mine > 0) issue(0);
+        bf16x8 kf[KSTEPS], vn[KSTEPS];  // K and -V of the 32 keys, MFMA B operands (requested before the first tile, used after it is)
+#pragma unroll
+        for (int st = 0; st < KSTEPS; st++) {
+            typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+            kf[st] = kraw[st];
+            u32x4 bits = __builtin_bit_cast(u32x4, vraw[st]) ^ 0x80008000u;  // sign flip of the eight bf16 values
+            vn[st] = __builtin_bit_cast(bf16x8, bits);
+            // the flip is done here, once, not again at every use; and both operands have arrived before the loop (a
+            // pending load of theirs would make the compiler wait for every outstanding load at their first use in it,
+            // the prefetched tile's included)
+            asm volatile("" : "+v"(vn[st]), "+v"(kf[st]));
+        }
         for (int i = 0; i < n_mine; i++) {
             // the other stage was read by tile i - 1, whose operand reads have all returned (its MFMAs were issued)
             if (i + 1 < n_mine) {
@@ -202,6 +211,8 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
                 }
         }
 
+        // the mirror block's K and V rows travel while this block's partial results are summed
+        if (pass == 0 && n_qt - 1 - pair > pair) load_kv(n_qt - 1 - pair);
         // Sum the four waves' partial results through the (now idle) rings, dK then dV, and store.
         float* red = reinterpret_cast<float*>(lds);  // [wave][32 keys][HD]
         bf16_t* outs[2] = {static_cast<bf16_t*>(a.dK) + b * a.k_sb + kvh * a.k_sh, static_cast<bf16_t*>(a.dV) + b * a.k_sb + kvh * a.k_sh};
