@@ -274,7 +274,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                 if (MASKED && (k0 >= a.S || my_qmax < 0 || (a.causal && k0 > my_qmax))) continue;
                 f32x16 s, dp;
 #pragma unroll
-                for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = 0.f; }
+                for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = -Dq; }  // the MFMA chain delivers dP - D
 #pragma unroll
                 for (int st = 0; st < KSTEPS; st++) {
                     const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + tile_at<HD>(sub * 32 + c, st * 16 + 8 * g));
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                         if (acc_row(v, g) > rel) p[v] = 0.f;
                 }
 #pragma unroll
-                for (int v = 0; v < 16; v++) dsf[v >> 3][v & 7] = (bf16_t)(p[v] * (dp[v] - Dq));
+                for (int v = 0; v < 16; v++) dsf[v >> 3][v & 7] = (bf16_t)(p[v] * dp[v]);
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
