@@ -138,12 +138,17 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                     for (int v = 0; v < 16; v++)
                         if (sub * 32 + acc_row(v, g) > lim) s[sub][v] = -INFINITY;
             }
-            float mx = -INFINITY;  // of the raw scores; the (positive) scale is folded into the exponent's fma
+            // maximum of the raw scores (the positive scale is folded into the exponent's fma): four chains, not one of 16
+            float mx4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
-            for (int v = 0; v < 16; v++) mx = fmaxf(mx, fmaxf(s[0][v], s[1][v]));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * a.scale_log2e;
-            const bool grow = mx > m + 8.0f;
-            if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+            for (int v = 0; v < 16; v++) mx4[v & 3] = fmaxf(mx4[v & 3], fmaxf(s[0][v], s[1][v]));
+            float mx = fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3]));
+            mx *= a.scale_log2e;
+            // mx is the maximum over this lane's half of the tile's keys; the two lanes of a query exchange theirs only when
+            // one of them has outgrown the reference point (then both take the same new one)
+            if (__builtin_amdgcn_ballot_w64(mx > m + 8.0f) != 0) {
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const bool grow = mx > m + 8.0f;
                 const float alpha = grow ? fast_exp2(m - mx) : 1.0f;
                 m = grow ? mx : m;
                 l *= alpha;
@@ -153,15 +158,16 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                     for (int v = 0; v < 16; v++) o[dt][v] *= alpha;
             }
             const float m_use = m == -INFINITY ? 0.f : m;
-            float rowsum = 0.f;
+            float rs4[4] = {0.f, 0.f, 0.f, 0.f};  // four chains of eight additions, not one of 32
 #pragma unroll
             for (int sub = 0; sub < 2; sub++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     s[sub][v] = fast_exp2(fmaf(s[sub][v], a.scale_log2e, -m_use));
-                    rowsum += s[sub][v];
+                    rs4[v & 3] += s[sub][v];
                 }
-            l += rowsum + __shfl_xor(rowsum, 32, 64);
+            const float rowsum = (rs4[0] + rs4[1]) + (rs4[2] + rs4[3]);
+            l += rowsum;  // this lane's half of the row sum; the halves meet after the last tile
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
                 if (sub == 1 && !two) break;
@@ -184,6 +190,7 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
         int kt = 0;
         for (; kt < n_plain; kt++) tile(kt, std::false_type{});
         for (; kt < n_kt; kt++) tile(kt, std::true_type{});
+        l += __shfl_xor(l, 32, 64);
         if (valid_q) {
             const float inv = l > 0.f ? 1.0f / l : 0.f;
             bf16_t* Op = static_cast<bf16_t*>(a.Out) + b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
