@@ -310,6 +310,17 @@ def bench_c2(steps, warmup):
         step()
     prof = ctx.profile_stop()
     roofline = pick_dominant(prof, "c2")
+    # What a plain copy of the same bytes (logits read, gradient written) reaches on this GPU, in this run: the practical
+    # ceiling of a kernel that streams 524 MB in and 524 MB out, next to the published 8 TB/s the fraction is quoted against.
+    for _ in range(warmup):
+        ctx.cast(dx, hip.BF16, dl, hip.BF16, rows * V)
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ctx.cast(dx, hip.BF16, dl, hip.BF16, rows * V)
+    ctx.sync()
+    copy_gbs = steps * 2.0 * rows * V * 2 / (time.perf_counter() - t0) / 1e9
+    roofline["copy_of_same_bytes"] = dict(achieved=round(copy_gbs, 1), unit="GB/s", frac=round(copy_gbs / 8000.0, 4))
     ctx.close()
     R.set_threads(1)
     sample = 64
