@@ -143,13 +143,7 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
             asm volatile("" : "+v"(vn[st]), "+v"(kf[st]));
         }
         for (int i = 0; i < n_mine; i++) {
-            // the other stage was read by tile i - 1, whose operand reads have all returned (its MFMAs were issued)
-            if (i + 1 < n_mine) {
-                issue(i + 1);
-                wait_vmcnt<LOADS>();
-            } else {
-                wait_vmcnt<0>();
-            }
+            wait_vmcnt<0>();  // tile i was requested in the middle of tile i - 1
             const int item = wave + 4 * i;
             const int q0 = (qt_start + item % per_head) * 32;
             const bf16_t* Qs = reinterpret_cast<const bf16_t*>(stage_of(i));
@@ -186,6 +180,9 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
                     dotr[dt][t] = lds_tr_operand_swz<HD>(dOs, 0, dt * 32, t, lane);
                     qtr[dt][t] = lds_tr_operand_swz<HD>(Qs, 0, dt * 32, t, lane);
                 }
+            // the next tile's loads go out while the score MFMAs run (the other stage was read by tile i - 1, whose operand reads
+            // have all returned)
+            if (i + 1 < n_mine) issue(i + 1);
             float p[16];
 #pragma unroll
             for (int v = 0; v < 16; v++) p[v] = fast_exp2(s[v] * a.scale_log2e);
