@@ -9,7 +9,11 @@ heads, head_dim 64, SiLU-gated MLP 5632, untied lm_head), seq 1024, micro-batch 
 Zipf(1.1) token ids, N(0, 0.02) weights.  One "step" = zero_grad, 8 x (upload ids, forward, fused cross entropy,
 loss read-back, backward), gradient-norm clip, fused AdamW -- the loop of examples/train_llm.rs:386-477, the
 per-micro-batch loss read-back of :450 included (the copy is queued before the backward pass and collected
-after it, so reading it does not drain the device).
+after it, so reading it does not drain the device).  One departure from that loop in the headline run, stated in the
+line's `config.weight_gradient_window`: the weight gradients dW = X^T dY of the 8 micro-batches are formed once per
+optimizer step, as one contraction over the 32,768 tokens of the window, instead of 8 products added in f32 (the same
+sums in another rounding order, equal to 1e-4); `other_configs.c5_per_pass_weight_gradients` carries the same step with
+the reference's order (`--no-window`), window 0.
 
 Prints one JSON line.  `value` is tokens/s over K timed steps (inputs resident in host memory, weights and
 optimiser state resident in HBM).  `roofline` describes the kernel symbol that takes the largest share of the
@@ -175,7 +179,8 @@ def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True, b
     lm.set_checkpointing(recompute)   # per-block recompute: off in the headline run (the reference's train_llm.rs does not use it)
     # weight gradients over the whole accumulation window in one contraction (Graph::set_weight_gradient_window): the sums
     # of train_llm.rs:386-477's micro-batch loop, each gradient read and written once per optimizer step
-    g.set_weight_gradient_window(c["accum"] if window and 2 <= c["accum"] <= 8 else 0)
+    win_passes = c["accum"] if window and 2 <= c["accum"] <= 8 else 0
+    g.set_weight_gradient_window(win_passes)
     g.set_weight_gradients_beside(beside)   # the library's default; off = every GEMM in tape order on the one stream
     opt = G.AdamW(g, lm.params(), 1e-3)
     opt.config(1e-3, 0.9, 0.95, 1e-8, 0.1, 1.0)      # train_llm.rs:266-270 + grad clip 1.0
@@ -218,6 +223,7 @@ def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True, b
                ms_per_step=round(1e3 * elapsed / steps, 3), higher_is_better=True, scaling="weak", vs_baseline=None, dtype="bf16",
                data="synthetic",
                config=dict(workload=c["label"] + (", per-block recompute" if recompute else ""), tokens_per_step=tokens_per_step, parallelism="single GPU",
+                           weight_gradient_window=win_passes, weight_gradients_beside=bool(beside), recompute=bool(recompute),
                            step_model_tflops=round(step_flops / 1e12, 4),
                            mfma_frac_of_step=round(step_flops / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 4), last_loss=round(float(last_loss), 4)),
                roofline=pick_dominant(prof, name), kernels=kernel_table(prof))
@@ -361,6 +367,9 @@ def main():
         out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside)
         if w == "all":
             out["other_configs"] = dict(c4=brief(bench_lm("c4", 20, 3, not args.no_cpu)), c3=brief(bench_c3(20, 3)), c2=brief(bench_c2(20, 3)))
+            if not args.no_window:   # the same step in the reference's accumulation order: every pass forms and adds its own dW
+                ref_order = brief(bench_lm("c5", 3, 1, False, args.recompute, False, not args.no_beside))
+                out["other_configs"]["c5_per_pass_weight_gradients"] = {k: ref_order[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup", "config")}
     elif w == "c4":
         out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside)
     elif w == "c3":

@@ -130,6 +130,14 @@ int eisen_graph_sync_grad_to_cpu(eisen_graph* g, size_t id, float* out, size_t n
         std::memcpy(out, v.data(), n * sizeof(float));
     });
 }
+int eisen_graph_sync_compute_copy_to_cpu(eisen_graph* g, size_t id, float* out, size_t n) {
+    return guarded(g, [&](Graph& G) {
+        if (n != G.at(id).size()) throw Error("sync_compute_copy_to_cpu: element count mismatch");
+        if (n) need(out, "out");
+        const std::vector<float> v = G.sync_compute_copy_to_cpu(id);
+        std::memcpy(out, v.data(), n * sizeof(float));
+    });
+}
 int eisen_graph_synchronize(eisen_graph* g) { return guarded(g, [&](Graph& G) { G.synchronize(); }); }
 
 #define OP_OUT(expr) return guarded(g, [&](Graph& G) { need(out, "out"); *out = (expr); })

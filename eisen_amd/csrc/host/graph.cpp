@@ -181,6 +181,7 @@ static std::vector<float> download(Graph& g, const Storage& s) {
 
 // Tensor::sync_to_cpu / Graph::sync_grad_to_cpu (src/tensor.rs:177-223, src/graph/mod.rs:629-668).
 std::vector<float> Graph::sync_to_cpu(size_t id) { return download(*this, at(id).data); }
+std::vector<float> Graph::sync_compute_copy_to_cpu(size_t id) { return download(*this, compute_data(id)); }
 std::vector<float> Graph::sync_grad_to_cpu(size_t id) {
     Tensor& t = at(id);
     materialize_grad(id);

@@ -106,6 +106,7 @@ class Graph {
     void load_tensor_data(size_t id, const float* host, size_t n);
     std::vector<float> sync_to_cpu(size_t id);
     std::vector<float> sync_grad_to_cpu(size_t id);
+    std::vector<float> sync_compute_copy_to_cpu(size_t id);   // the bf16 copy kernels read (mixed-mode parameters), widened
     void reinterpret_shape(size_t id, const std::vector<size_t>& shape);
     void synchronize();
 

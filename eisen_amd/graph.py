@@ -133,6 +133,12 @@ class Graph:
         self._call("eisen_graph_sync_grad_to_cpu", _sz(tid), _fp(out), _sz(out.size))
         return out
 
+    def sync_compute_copy_to_cpu(self, tid):
+        """The values the kernels read for this tensor (a mixed-mode parameter's bf16 copy), widened to f32."""
+        out = np.empty(self.shape(tid), np.float32)
+        self._call("eisen_graph_sync_compute_copy_to_cpu", _sz(tid), _fp(out), _sz(out.size))
+        return out
+
     # ---- ops --------------------------------------------------------------------------
     def add(self, a, b): return self._op("eisen_graph_add", _sz(a), _sz(b))
     def mul(self, a, b): return self._op("eisen_graph_mul", _sz(a), _sz(b))

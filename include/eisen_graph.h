@@ -74,6 +74,10 @@ int eisen_graph_tensor_shape(eisen_graph* g, size_t id, size_t* shape_out, int* 
  * n must equal the element count; bf16 storage is widened to f32. */
 int eisen_graph_sync_to_cpu(eisen_graph* g, size_t id, float* out, size_t n);
 int eisen_graph_sync_grad_to_cpu(eisen_graph* g, size_t id, float* out, size_t n);
+/* What the kernels read for tensor `id`, widened to f32: in Bf16Mixed mode the bf16 copy of a parameter that AdamW
+ * refreshes next to the f32 master weight (the reference keeps its bf16 weights themselves, alloc_param_bf16,
+ * src/graph/mod.rs:567-598); for every other tensor the same values as eisen_graph_sync_to_cpu. */
+int eisen_graph_sync_compute_copy_to_cpu(eisen_graph* g, size_t id, float* out, size_t n);
 int eisen_graph_synchronize(eisen_graph* g);
 
 /* Ops: one per `impl Graph` method under src/graph/ops/ (file:line at each definition in

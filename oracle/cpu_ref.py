@@ -138,6 +138,10 @@ def set_threads(n):
     _lib.ref_set_threads(int(n))
 
 
+def get_threads():
+    return int(_lib.ref_get_threads())
+
+
 def fp(a):
     """float32 C-contiguous numpy array -> float*."""
     assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]

@@ -41,13 +41,16 @@ def _record(name, kind, rtol, a_size, rel_l2, frac_outside, worst_ratio):
                          worst_ratio=float(worst_ratio)))
 
 
-def assert_close(actual, expected, rtol, name="", row_scale=False, l2=None, step=False, step_outliers=0.0):
+def assert_close(actual, expected, rtol, name="", row_scale=False, l2=None, step=False, step_outliers=0.0, row_floor=0.0, outliers=1e-4, worst_cap=2.0):
     """step: the composed-step criterion above (scale = max|e| instead of rms(e), no outlier allowance,
     relative L2 <= rtol).  step_outliers: fraction of the elements that may exceed the step bound, by at most 4x -- only
     for comparisons of two bf16 results with each other (both sides carry rounding noise), never against the oracle.
     row_scale: take rms(e) per last-dim row instead of over the whole tensor -- for tensors whose
     rows differ by orders of magnitude (an embedding gradient: untouched rows are exactly zero, hot
-    rows are large), where one global RMS is not the scale of any element.  l2: bound on the
+    rows are large), where one global RMS is not the scale of any element; row_floor: with row_scale, a row's
+    scale is never taken below this fraction of the tensor's RMS (for rows whose exact value is zero but whose
+    computed value is a rounding residue).  outliers / worst_cap: the bf16-kernel allowance (fraction of the elements
+    that may pass the per-element bound, and by how much at most); a test that widens them says why.  l2: bound on the
     relative L2 error for the bf16 check (default 1e-2).
     Every failure message carries the observed relative L2 error, the fraction of elements outside the
     per-element bound and the worst error as a multiple of that bound."""
@@ -74,7 +77,10 @@ def assert_close(actual, expected, rtol, name="", row_scale=False, l2=None, step
         assert rel_l2 <= bound, f"{name}: relative L2 error {rel_l2:.3g} > {bound:g}; {seen}"
         return
     if row_scale and e.ndim >= 2:
-        rms_el = np.broadcast_to(np.sqrt(np.mean(e * e, axis=-1, keepdims=True)), e.shape).reshape(-1)
+        rms_el = np.sqrt(np.mean(e * e, axis=-1, keepdims=True))
+        if row_floor > 0.0:
+            rms_el = np.maximum(rms_el, row_floor * np.sqrt(np.mean(e * e)))
+        rms_el = np.broadcast_to(rms_el, e.shape).reshape(-1)
     else:
         rms_el = None
     a, e, err = a.reshape(-1), e.reshape(-1), err.reshape(-1)
@@ -87,8 +93,8 @@ def assert_close(actual, expected, rtol, name="", row_scale=False, l2=None, step
     loose = rtol >= RTOL_BF16          # bf16: allow 1e-4 of the elements up to 2x the bound
     _record(name, "bf16 kernel" if loose else "f32 kernel", rtol, a.size, rel_l2, frac, worst)
     seen = f"observed: relative L2 {rel_l2:.3g}, {frac:.3g} of the elements outside the bound, worst error {worst:.3g} x bound"
-    allowed = int(1e-4 * a.size) + 1 if loose else 0
-    if bad.sum() > allowed or (loose and worst > 2):
+    allowed = int(outliers * a.size) + 1 if loose else 0
+    if bad.sum() > allowed or (loose and worst > worst_cap):
         i = int(np.argmax(ratio))
         raise AssertionError(f"{name}: {int(bad.sum())}/{a.size} elements outside rtol {rtol:g}; worst at {i}: "
                              f"got {a[i]:.8g}, expected {e[i]:.8g}, rms {rms:.4g}; {seen}")

@@ -164,3 +164,99 @@ def test_config4_real_micro_batch_against_the_oracle(ctx):
     """Config 4 exactly as BASELINE states it: 6 layers, tied embeddings, Zipf ids, micro-batch 32 x seq 256 (8192 tokens, so
     the tile and split-K choices of M = 8192 are the ones checked), bf16 mixed step against the f32 oracle at rtol 2e-2."""
     _train_steps(ctx, C4, G.BF16_MIXED, 32, 256, steps=1, accum=1, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True)
+
+
+@pytest.mark.timeout(900)
+def test_config5_whole_model_one_sequence_against_the_oracle(ctx):
+    """The whole config-5 model (16 layers, vocab 32000, 852,559,872 parameters) on one sequence of 1024 tokens, the largest
+    batch the oracle's unfused attention chain finishes in about a minute on the host's threads: loss, every gradient, every
+    AdamW-updated weight and both moments against the CPU oracle (examples/train_llm.rs:386-477 with one micro-batch).
+    Every gradient tensor's relative L2 error stays under 2e-2 (observed: 0.0098 for the embedding, the deepest gradient; 0.0182 for layer 8's K projection, the largest).
+    Sixteen layers of bf16 activations deep, a few elements in a million of the 65.5 M-element embedding gradient pass the
+    per-element bound 2e-2 (|e| + max |row|) (observed 3.9e-6 of them, the worst at 1.95 x): 1e-5 of a tensor's elements
+    may, by at most 4 x."""
+    _train_steps(ctx, C5, G.BF16_MIXED, 1, 1024, steps=1, accum=1, rtol_grad=2e-2, dist="zipf", perturb_norm=0.0, bf16_weights=True,
+                 step_outliers=1e-5)
+
+
+def _host_adamw_first_step(w0, g, coef, lr, b1, b2, eps, wd):
+    """src/nn/optim.rs:336-338,533-542 at t = 1 from zero moments, in f32 with the reference's operation order; the gradient
+    is first scaled by the clip coefficient (optim.rs:114-200)."""
+    f = np.float32
+    g = (g * f(coef)).astype(np.float32)
+    bc1, bc2 = f(1.0) / (f(1.0) - f(b1)), f(1.0) / (f(1.0) - f(b2))
+    m = ((f(1.0) - f(b1)) * g).astype(np.float32)
+    v = (((f(1.0) - f(b2)) * g) * g).astype(np.float32)
+    decayed = (w0 * (f(1.0) - f(lr) * f(wd))).astype(np.float32)
+    w = (decayed - (f(lr) * (m * bc1)) / (np.sqrt(v * bc2) + f(eps))).astype(np.float32)
+    return w, m, v
+
+
+@pytest.mark.timeout(900)
+def test_config5_benched_step_window_of_eight_clip_and_adamw(ctx):
+    """The configuration bench.py times: 8 distinct micro-batches of 4 x 1024 tokens, the weight gradients formed once over
+    the window of 8, gradient clipping at 1.0, then the fused AdamW over all 852,559,872 parameters.  Against the same 8
+    passes with every micro-batch's weight gradients formed and added in its own backward pass (the reference's order,
+    src/graph/ops/linear.rs:279-287): losses identical, gradients to 1e-4, the same norm; and the optimizer's result on
+    sampled tensors (first and last layer, one in the middle, embedding, final norm, lm_head) against a host AdamW fed with
+    the downloaded gradients: master weights, both moments, and the bf16 copy = the master weight rounded to nearest even."""
+    mb, seq, accum = 4, 1024, 8
+    lr, b1, b2, eps, wd, clip = 1e-3, 0.9, 0.95, 1e-8, 0.1, 1.0
+    gg = G.Graph(ctx, G.BF16_MIXED)
+    lm = G.TransformerLM(gg, **C5)
+    shapes = gen.lm_param_shapes(**C5)
+    sampled = [i for i, (name, _) in enumerate(shapes) if name.split(".")[0] in ("embed", "l0", "l7", "l15", "norm_f", "lm_head")]
+    rng = np.random.default_rng(77)
+    w0 = {}
+    for pid, (name, shape) in enumerate(shapes):
+        if len(shape) == 2:
+            w = rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)
+            gg.load_tensor_data(pid, w)
+        else:
+            w = np.ones(shape, np.float32)
+        if pid in sampled:
+            w0[pid] = w
+    gg.mark_params()
+    params = lm.params()
+    assert sorted(params) == list(range(len(shapes)))   # params() lists a block's MLP weights in another order than their ids
+    opt = G.AdamW(gg, params, lr)
+    opt.config(lr, b1, b2, eps, wd, clip)
+    opt.init_moments()
+    batches = [gen.lm_batch(8800 + i, mb, seq, C5["vocab"], "zipf") for i in range(accum)]
+
+    # the reference's order: every pass adds its own weight gradients
+    gg.set_weight_gradient_window(0)
+    opt.zero_grad()
+    losses_ref = [lm.micro_step(x, y) for x, y in batches]
+    norm_ref, _ = opt.clip_grad_norm(1e9)     # the norm only: a bound this large scales nothing
+    grads_ref = {p: gg.sync_grad_to_cpu(p) for p in sampled}
+
+    # the benched order: one contraction per weight shape over the 8 passes, flushed by the optimizer
+    gg.set_weight_gradient_window(accum)
+    opt.zero_grad()
+    ctx.profile_start()
+    losses = [lm.micro_step(x, y) for x, y in batches]
+    opt.step()
+    prof = ctx.profile_stop()
+    assert losses == losses_ref
+    assert sum(e["launches"] for k, e in prof.items() if k.endswith("_window")) == 5, sorted(prof)
+    assert prof["adamw"]["launches"] == 1
+    norm, coef = opt.last_grad_norm()
+    assert abs(norm - norm_ref) <= 1e-5 * norm_ref, (norm, norm_ref)
+    assert abs(coef - min(1.0, clip / (norm + 1e-6))) <= 1e-6 * coef, (norm, coef)   # src/nn/optim.rs:114-200
+    for p in sampled:
+        name, shape = shapes[p]
+        got = gg.sync_grad_to_cpu(p)          # AdamW reads the coefficient on the device: the stored gradient is unscaled
+        assert_close(got, grads_ref[p], 1e-4, f"config 5, window of 8: grad {name}", row_scale=(name == "embed"))
+        ew, em, ev = _host_adamw_first_step(w0[p].reshape(-1), got.reshape(-1), coef, lr, b1, b2, eps, wd)
+        w1 = gg.sync_to_cpu(p).reshape(-1)
+        m1, v1 = opt.moments(params.index(p))
+        # the update of an element is at most ~lr; f32 rounding of its pieces is 1e-7 of that
+        assert np.abs(w1 - ew).max() <= 2e-7 * lr * 1e3, (name, float(np.abs(w1 - ew).max()))
+        assert_close(m1, em, 1e-5, f"config 5, benched step: m of {name}", row_scale=False)
+        assert_close(v1, ev, 1e-5, f"config 5, benched step: v of {name}", row_scale=False)
+        if len(shape) == 2:
+            assert np.array_equal(gg.sync_compute_copy_to_cpu(p).reshape(-1), hip.round_bf16(w1)), f"bf16 copy of {name}"
+        del grads_ref[p]
+    gg.set_weight_gradient_window(0)
+    gg.close()

@@ -350,9 +350,11 @@ def _build_pair(ctx, cfg, weights, precision):
 
 
 def _train_steps(ctx, cfg, precision, mb, seq, steps, accum, rtol_grad, seed=1, fused=True, dist="uniform", clip=0.0, perturb_norm=0.05,
-                 bf16_weights=False, l2=None):
+                 bf16_weights=False, l2=None, step_outliers=0.0):
     """bf16_weights: round the seeded matrices to bf16-representable values first, so the oracle and the
-    GPU's bf16 compute copy start from identical numbers and the comparison isolates the kernels."""
+    GPU's bf16 compute copy start from identical numbers and the comparison isolates the kernels.
+    step_outliers: fraction of a gradient's elements that may pass the per-element step bound (by at most 4x); zero except
+    for the 16-layer model, whose caller says why."""
     from eisen_amd import hip
     weights = gen.lm_weights(seed, std=0.02, perturb_norm=perturb_norm, **cfg)
     if bf16_weights:
@@ -372,7 +374,8 @@ def _train_steps(ctx, cfg, precision, mb, seq, steps, accum, rtol_grad, seed=1, 
             assert gg.num_tensors() == len(weights) and gg.tape_len() == 0
         for pid, (name, _) in enumerate(weights):
             # the embedding gradient is row-sparse (untouched rows exactly zero, Zipf-hot rows large): per-row scale
-            assert_close(gg.sync_grad_to_cpu(pid), og.grad(pid), rtol_grad, f"step {step} grad {name}", row_scale=(name == "embed"), l2=l2, step=(precision != G.FP32))
+            assert_close(gg.sync_grad_to_cpu(pid), og.grad(pid), rtol_grad, f"step {step} grad {name}", row_scale=(name == "embed"), l2=l2, step=(precision != G.FP32),
+                         step_outliers=step_outliers)
         opt.step()
         oopt.step()
         for pid, (name, w) in enumerate(weights):
@@ -388,7 +391,7 @@ def _train_steps(ctx, cfg, precision, mb, seq, steps, accum, rtol_grad, seed=1, 
         for i in range(len(weights)):                                      # and identical moments
             m, v = opt.moments(i)
             om, ov = oopt.moments(i)
-            assert_close(m, om, rtol_grad, f"m[{i}]", row_scale=(i == 0), l2=l2, step=(precision != G.FP32))
+            assert_close(m, om, rtol_grad, f"m[{i}]", row_scale=(i == 0), l2=l2, step=(precision != G.FP32), step_outliers=step_outliers)
             np.ctypeslib.as_array(R.lib.ref_adamw_m(oopt.h, i), (m.size,))[:] = m
             np.ctypeslib.as_array(R.lib.ref_adamw_v(oopt.h, i), (v.size,))[:] = v
     return gg, lm, opt

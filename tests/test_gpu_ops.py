@@ -4,6 +4,7 @@ Run on an MI355X with `pytest -m gpu`.  All calls go through libeisen_hip.so's C
 (eisen_amd.hip is a ctypes mirror of include/eisen_hip.h); the oracle is only the checker.
 """
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -566,10 +567,10 @@ def test_cross_entropy_reference_vector_and_ties(ctx):
         assert ctx.download(am, (2,), np.int32).tolist() == [min(5, 900 % classes), classes - 1]
 
 
-def test_cross_entropy_config2_full_size_properties(ctx):
-    """[8192 x 32000] bf16 (config 2): size-independent properties instead of a full oracle run --
-    gradient rows sum to ~0, loss equals the mean of -ln(p_t + 1e-8) recomputed on sampled rows by
-    the oracle, argmax / target logit bit-exact on every row."""
+def test_cross_entropy_config2_full_size_against_the_oracle(ctx):
+    """[8192 x 32000] bf16 (config 2), every row against the oracle (src/graph/ops/reduction.rs:668-716): the mean loss to
+    1e-3 relative (BASELINE config 2's bar), every row's loss, the gradient of all 8192 rows to 2e-2, argmax and target
+    logit bit-exact on every row, and gradient rows summing to ~0."""
     rows, classes = 8192, 32000
     rng = np.random.default_rng(7)
     x = hip.round_bf16((rng.standard_normal((rows, classes), dtype=np.float32) * 2.0))
@@ -581,14 +582,23 @@ def test_cross_entropy_config2_full_size_properties(ctx):
     assert np.array_equal(ctx.download(am, (rows,), np.int32), x.argmax(-1).astype(np.int32))
     assert np.array_equal(dn(ctx, tl, (rows,), F32), x[np.arange(rows), t])
     row_loss = dn(ctx, rl, (rows,), F32)
-    sample = np.arange(0, rows, 64)
-    _, egl, probs = R.cross_entropy(x[sample], t[sample])
-    exp_rows = -np.log(probs[np.arange(sample.size), t[sample]].astype(np.float64) + 1e-8)
-    assert_close(row_loss[sample], exp_rows, 1e-4, "row loss")
     loss = float(dn(ctx, lo, (1,), F32)[0])
-    assert abs(loss - row_loss.astype(np.float64).mean()) <= 1e-5 * loss
     g = dn(ctx, dl, (rows, classes), BF16)
-    assert_close(g[sample] * rows, egl * sample.size, 2e-2, "dlogits (sampled rows)")
+    # the oracle in blocks of 1024 rows (its loss is the mean over the rows it is given, its gradient carries 1 / rows of the
+    # block: both are brought to the full batch here), row loops on the host's threads with identical results
+    before = R.get_threads()
+    R.set_threads(min(16, os.cpu_count() or 1))
+    oracle_loss, blk = 0.0, 1024
+    for r0 in range(0, rows, blk):
+        sl = slice(r0, r0 + blk)
+        eloss, egl, probs = R.cross_entropy(x[sl], t[sl])
+        oracle_loss += float(eloss) * blk / rows
+        exp_rows = -np.log(probs[np.arange(blk), t[sl]].astype(np.float64) + 1e-8)
+        assert_close(row_loss[sl], exp_rows, 1e-4, f"config 2 row loss, rows {r0}..{r0 + blk - 1}")
+        assert_close(g[sl] * rows, egl * blk, 2e-2, f"config 2 dlogits, rows {r0}..{r0 + blk - 1}")
+    R.set_threads(before)
+    assert abs(loss - oracle_loss) <= 1e-3 * oracle_loss, (loss, oracle_loss)
+    assert abs(loss - row_loss.astype(np.float64).mean()) <= 1e-5 * loss
     assert np.abs(g.astype(np.float64).sum(-1)).max() < 2e-2 / rows
     for b in (dx, dt, dl, rl, lo, am, tl):
         b.free()
@@ -1160,13 +1170,40 @@ def test_attention_rope_backward(ctx, dtype, B, S, Hq, Hkv, hd):
         x.free()
 
 
+_C3_ORACLE = {}
+
+
+def _config3_oracle(q, k, v, do):
+    """The unfused chain on every (batch, KV group) slice of config 3 (32 independent sub-problems of 4 query heads x 1024
+    x 1024 scores each; the row loops run on the host's threads with identical results).  Computed once per session:
+    both layouts are compared with the same numbers."""
+    if not _C3_ORACLE:
+        B, S, Hq, hd = q.shape
+        Hkv = k.shape[2]
+        G_ = Hq // Hkv
+        before = R.get_threads()
+        R.set_threads(min(16, os.cpu_count() or 1))
+        eo, edq = np.empty(q.shape, np.float32), np.empty(q.shape, np.float32)
+        edk, edv = np.empty(k.shape, np.float32), np.empty(k.shape, np.float32)
+        for b in range(B):
+            for grp in range(Hkv):
+                hs = slice(grp * G_, (grp + 1) * G_)
+                o_, dq_, dk_, dv_ = oracle_attention(q[b:b + 1, :, hs], k[b:b + 1, :, grp:grp + 1], v[b:b + 1, :, grp:grp + 1], do[b:b + 1, :, hs],
+                                                     np.float32(0.125))
+                eo[b:b + 1, :, hs], edq[b:b + 1, :, hs] = o_, dq_
+                edk[b:b + 1, :, grp:grp + 1], edv[b:b + 1, :, grp:grp + 1] = dk_, dv_
+        R.set_threads(before)
+        _C3_ORACLE.update(o=eo, dq=edq, dk=edk, dv=edv)
+    return _C3_ORACLE["o"], _C3_ORACLE["dq"], _C3_ORACLE["dk"], _C3_ORACLE["dv"]
+
+
 @pytest.mark.parametrize("layout", ["bhsd", "bshd"])
-def test_attention_config3_full_size_properties(ctx, layout):
+def test_attention_config3_full_size_against_the_oracle(ctx, layout):
     """B8 S1024 Hq16 Hkv4 hd64 bf16 (config 3), in the [B,H,S,hd] layout config 3 states (the reference's q_t layout,
-    addressed through strides) and in the [B,S,H,hd] layout the projections produce: too large for the unfused oracle in
-    seconds, so check one batch element's heads of one KV group against the oracle (S=1024 is kept), and size-independent
-    properties on the whole output: row-stochastic P implies O of a constant V is that constant; the deterministic kernels
-    give identical bits on a second run."""
+    addressed through strides) and in the [B,S,H,hd] layout the projections produce.  O, dQ, dK and dV of all 32
+    (batch, KV group) slices against the oracle's unfused chain (src/nn/attention.rs:338-375), slice by slice, so that a fault
+    tied to one workgroup's block index shows in the slice it belongs to; plus two size-independent properties on the whole
+    output: row-stochastic P implies O of a constant V is that constant, and a second run gives identical bits."""
     B, S, Hq, Hkv, hd = 8, 1024, 16, 4, 64
     sd = 1.0 / 8
     # generated as [B,S,H,hd] (the oracle's layout); `dev` puts a tensor into the layout under test, `host` brings it back
@@ -1186,14 +1223,21 @@ def test_attention_config3_full_size_properties(ctx, layout):
     ctx.attention_forward(dq_, dk_, dv_, out, lse, BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
     ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
     o1, q1, k1, v1 = host(out, q), host(gq, q), host(gk, k), host(gv, k)
-    # slice: batch 3, KV group 2 (query heads 8..11) -> an independent sub-problem
-    b, grp = 3, 2
-    hs = slice(grp * 4, grp * 4 + 4)
-    eo, edq, edk, edv = oracle_attention(q[b:b + 1, :, hs], k[b:b + 1, :, grp:grp + 1], v[b:b + 1, :, grp:grp + 1], do[b:b + 1, :, hs], np.float32(0.125))
-    assert_close(o1[b:b + 1, :, hs], eo, 2e-2, f"config 3 {layout} O slice")
-    assert_close(q1[b:b + 1, :, hs], edq, 2e-2, f"config 3 {layout} dQ slice")
-    assert_close(k1[b:b + 1, :, grp:grp + 1], edk, 2e-2, f"config 3 {layout} dK slice")
-    assert_close(v1[b:b + 1, :, grp:grp + 1], edv, 2e-2, f"config 3 {layout} dV slice")
+    eo, edq, edk, edv = _config3_oracle(q, k, v, do)
+    for b in range(B):
+        for grp in range(Hkv):
+            hs, where = slice(grp * 4, grp * 4 + 4), f"config 3 {layout} batch {b} KV head {grp}"
+            assert_close(o1[b, :, hs], eo[b, :, hs], 2e-2, f"{where} O")
+            # dQ: D = rowsum(dO o O) is formed from the stored bf16 O where the reference's chain keeps O in f32.  Its error
+            # enters dQ as -scale dD (P K), which is largest for the first queries (P K is an average over a handful of keys).
+            # An f64 emulation of exactly the kernels' roundings puts 19 elements of a slice, all in query row 1, outside the
+            # per-element bound, the worst at 2.35 x; with D from the unrounded O none.  Hence 2e-4 of the elements up to 3 x
+            # here, where the other bf16 comparisons allow 1e-4 up to 2 x; the relative L2 bound stays 1e-2.
+            assert_close(q1[b, :, hs], edq[b, :, hs], 2e-2, f"{where} dQ", outliers=2e-4, worst_cap=3.0)
+            # dK / dV: the rows of the first keys are sums over a thousand queries' large probabilities, an order of magnitude
+            # above the tensor's RMS: every key's row is measured against its own RMS
+            assert_close(k1[b, :, grp], edk[b, :, grp], 2e-2, f"{where} dK", row_scale=True)
+            assert_close(v1[b, :, grp], edv[b, :, grp], 2e-2, f"{where} dV", row_scale=True)
     ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
     assert np.array_equal(host(gq, q), q1) and np.array_equal(host(gk, k), k1) and np.array_equal(host(gv, k), v1)
     ones = up(ctx, np.full(k.shape, 0.5, np.float32), BF16)
