@@ -86,10 +86,14 @@ def by_symbol(prof):
     return out
 
 
-def roofline_of(name, e, workload):
+def roofline_of(name, e, workload, strict=False):
     """achieved = algorithmic work of the symbol's launches / their summed duration (= work per launch / average
     launch duration, weighted over the shapes the symbol ran)."""
-    traffic = MEASURED_TRAFFIC.get(workload, {}).get(name)
+    table = MEASURED_TRAFFIC.get(workload, {})
+    traffic = table.get(name)
+    if strict and table and traffic is None:
+        raise KeyError(f"{workload}: the dominant kernel symbol {name!r} has no row in MEASURED_TRAFFIC (table of {TRAFFIC_SOURCE.get(workload)}); "
+                       f"a kernel was renamed or the counter runs are stale")
     src = TRAFFIC_SOURCE.get(workload) if traffic is not None else None
     if e["unit"] == "flop":
         achieved = e["work"] / (e["ms"] * 1e-3) / 1e12
@@ -101,10 +105,17 @@ def roofline_of(name, e, workload):
     return r
 
 
+def mfma_ceiling(ctx):
+    """What this GPU sustains on nothing but bf16 MFMAs, measured now, next to the published peak the fractions use:
+    operands in registers, and re-read from LDS at the ratio of a 128x128 and of a 64x64 wave tile."""
+    return dict(unit="TFLOP/s", registers_only=round(ctx.mfma_ceiling(0), 1), lds_fed_128x128_wave_tile=round(ctx.mfma_ceiling(8), 1),
+                lds_fed_64x64_wave_tile=round(ctx.mfma_ceiling(16), 1))
+
+
 def pick_dominant(prof, workload):
     sym = by_symbol(prof)
     name = max(sym, key=lambda k: sym[k]["ms"])
-    r = roofline_of(name, sym[name], workload)
+    r = roofline_of(name, sym[name], workload, strict=True)
     if len(sym[name]["families"]) > 1:
         r["families"] = sorted(sym[name]["families"])
     return r
@@ -227,19 +238,24 @@ def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True, b
                            step_model_tflops=round(step_flops / 1e12, 4),
                            mfma_frac_of_step=round(step_flops / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 4), last_loss=round(float(last_loss), 4)),
                roofline=pick_dominant(prof, name), kernels=kernel_table(prof))
+    out["roofline"]["mfma_ceiling"] = mfma_ceiling(ctx)
     ctx.close()
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline_lm(c, c["seq"], 1 if name == "c5" else 8)
     return out
 
 
-def bench_c3(steps, warmup):
-    """Config 3: causal GQA flash attention forward + backward, B8 S1024 Hq16 Hkv4 hd64 bf16, layout [B,H,S,hd]."""
+def bench_c3(steps, warmup, hd=64):
+    """Config 3: causal GQA flash attention forward + backward, B8 S1024 Hq16 Hkv4 hd64 bf16, layout [B,H,S,hd].
+    hd = 128 (--head-dim 128) keeps the tokens, the model width (Hq * hd = 1024) and so the algorithmic flops, with 8 query and
+    2 KV heads: the same problem at the head size where a score tile costs half the softmax work per MFMA."""
     from eisen_amd import hip
     from oracle import cpu_ref as R
-    B, S, Hq, Hkv, hd = 8, 1024, 16, 4, 64
+    B, S = 8, 1024
+    Hq, Hkv = 1024 // hd, 256 // hd
     ctx = hip.Context(0)
     sd = 1.0 / 8
+    scale = float(1.0 / np.sqrt(hd))     # 1/8 at config 3's head size
     q, do = gen.normal(600, (B, Hq, S, hd), sd), gen.normal(601, (B, Hq, S, hd), sd)
     k, v = gen.normal(602, (B, Hkv, S, hd), sd), gen.normal(603, (B, Hkv, S, hd), sd)
     dq_, dk_, dv_, ddo = (ctx.upload(t, hip.BF16) for t in (q, k, v, do))
@@ -248,8 +264,8 @@ def bench_c3(steps, warmup):
     qs, ks = (Hq * S * hd, hd, S * hd), (Hkv * S * hd, hd, S * hd)
 
     def step():
-        ctx.attention_forward(dq_, dk_, dv_, out, lse, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
-        ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+        ctx.attention_forward(dq_, dk_, dv_, out, lse, hip.BF16, B, S, Hq, Hkv, hd, scale, True, qs, ks)
+        ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, hip.BF16, B, S, Hq, Hkv, hd, scale, True, qs, ks)
 
     for _ in range(warmup):
         step()
@@ -272,15 +288,18 @@ def bench_c3(steps, warmup):
     # CPU: the unfused chain on one batch element and one KV group (4 query heads), scaled by B*Hkv
     R.set_threads(1)
     t1 = time.perf_counter()
-    R.attention_chain(np.ascontiguousarray(q[:1, :4].transpose(0, 2, 1, 3)), np.ascontiguousarray(k[:1, :1].transpose(0, 2, 1, 3)),
-                       np.ascontiguousarray(v[:1, :1].transpose(0, 2, 1, 3)), np.ascontiguousarray(do[:1, :4].transpose(0, 2, 1, 3)), np.float32(0.125))
+    grp = Hq // Hkv
+    R.attention_chain(np.ascontiguousarray(q[:1, :grp].transpose(0, 2, 1, 3)), np.ascontiguousarray(k[:1, :1].transpose(0, 2, 1, 3)),
+                       np.ascontiguousarray(v[:1, :1].transpose(0, 2, 1, 3)), np.ascontiguousarray(do[:1, :grp].transpose(0, 2, 1, 3)), np.float32(scale))
     cpu_s = (time.perf_counter() - t1) * B * Hkv
     return dict(metric="flash-attention fwd+bwd tokens/sec (config 3)", value=round(steps * tokens / elapsed, 1), unit="tokens/s", n_gpus=1,
                 steps=steps, warmup=warmup, ms_per_step=round(1e3 * elapsed / steps, 4), higher_is_better=True, scaling="weak",
                 vs_baseline=None, dtype="bf16", data="synthetic",
-                config=dict(workload="config3 causal GQA flash attention fwd+bwd, B8 S1024 Hq16 Hkv4 hd64, [B,H,S,hd]"),
+                config=dict(workload=f"config3 causal GQA flash attention fwd+bwd, B8 S1024 Hq{Hq} Hkv{Hkv} hd{hd}, [B,H,S,hd]" +
+                            ("" if hd == 64 else " (config 3's tokens and width at another head size)")),
                 roofline=dict(bound="mfma", achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                              frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC["c3"]["attn_bwd"], traffic_source=TRAFFIC_SOURCE["c3"],
+                              frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC["c3"]["attn_bwd"] if hd == 64 else None,
+                              traffic_source=TRAFFIC_SOURCE["c3"] if hd == 64 else None,
                               kernel="attn_bwd (" + " + ".join(sorted(bwd_keys)) + ")", bwd_us=round(1e3 * bwd_ms, 2),
                               algorithmic_gflop=round(bwd_flops / 1e9, 2)),
                 kernels=kernel_table(prof),
@@ -353,6 +372,7 @@ def main():
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="all", choices=["all", "c5", "c4", "c3", "c2"])
+    ap.add_argument("--head-dim", type=int, default=64, choices=[32, 64, 128], help="c3: head size (the token count and Hq * hd = 1024 stay)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
     ap.add_argument("--no-window", action="store_true", help="c5: form every micro-batch's weight gradients in its own backward pass, as the reference does, "
                     "instead of once per optimizer step over the whole accumulation window")
@@ -373,7 +393,7 @@ def main():
     elif w == "c4":
         out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside)
     elif w == "c3":
-        out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3)
+        out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3, args.head_dim)
     else:
         out = bench_c2(args.steps or 20, args.warmup if args.warmup is not None else 3)
     print(json.dumps(out))

@@ -22,11 +22,14 @@
 //     every query head of the group and every visible query tile; Q/dO tiles go through LDS.
 //     No atomics anywhere: dQ has its own query-stationary pass, so results are reproducible.
 // f32 path (any head_dim): one wave per query row / key row, plain FMA, for small shapes.
+#include <cmath>
+#include <mutex>
+
 #include "attention_common.cuh"
 
 namespace {
 
-// Scratch of eisen_hip_attention_backward_noalloc: D = rowsum(dO o O) and LSE * log2(e), two floats per (batch, query
+// Scratch of eisen_hip_attention_backward_noalloc: D = rowsum(dO o O) and -LSE / scale, two floats per (batch, query
 // head, position).  A file-scope device array instead of a workspace allocation, so that entry point never calls an
 // allocator.  Every GPU the library runs on holds its own 8 MiB copy until the process ends; the name below is only a
 // host-side handle, the device address of each GPU's copy comes from hipGetSymbolAddress (eisen_attention_scratch_init).
@@ -34,6 +37,11 @@ constexpr size_t kNoAllocMaxRows = size_t(1) << 20;
 static __device__ __align__(256) float g_attn_bwd_scratch[2 * kNoAllocMaxRows];
 constexpr int kMaxDevices = 64;
 static float* g_attn_bwd_scratch_ptr[kMaxDevices] = {nullptr};  // per device, filled once
+// Every context and stream of a GPU shares that GPU's array, so calls are put in order: the event is recorded behind the
+// kernels of a call and the next call's stream waits for it first (two contexts on one GPU, or the main and the side
+// stream of one).  The mutex covers the two tables and the wait / launch / record sequence.
+static hipEvent_t g_attn_bwd_scratch_done[kMaxDevices] = {nullptr};
+static std::mutex g_attn_bwd_scratch_mu;
 
 // ---- forward -------------------------------------------------------------------------------
 // Grid of the two query-stationary kernels: one block per (pair of query blocks, GW query heads of a
@@ -665,6 +673,8 @@ int fill_args(eisen_ctx* ctx, AttnArgs& a, int dtype, size_t B, size_t S, size_t
     if (dtype == EISEN_BF16)
         EISEN_REQUIRE(ctx, a.q_sb % 8 == 0 && a.q_ss % 8 == 0 && a.q_sh % 8 == 0 && a.k_sb % 8 == 0 && a.k_ss % 8 == 0 && a.k_sh % 8 == 0,
                       EISEN_E_ALIGN, "%s: strides must be multiples of 8 elements for bf16", who);
+    // the key-stationary backward starts its score accumulators at -LSE / scale; a softmax scale is positive anyway
+    EISEN_REQUIRE(ctx, std::isfinite(scale) && scale >= 1e-30f && scale <= 1e30f, EISEN_E_ARG, "%s: softmax scale %g is not a positive finite number", who, (double)scale);
     a.scale = scale;
     a.scale_log2e = scale * kLog2e;
     a.causal = causal;
@@ -744,6 +754,11 @@ extern "C" int eisen_hip_attention_forward(eisen_ctx* ctx, const void* q, const 
 
 int eisen_attention_scratch_init(eisen_ctx* ctx) {
     EISEN_REQUIRE(ctx, ctx->device >= 0 && ctx->device < kMaxDevices, EISEN_E_ARG, "device index %d beyond the %d this library keeps scratch for", ctx->device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_attn_bwd_scratch_mu);
+    if (!g_attn_bwd_scratch_done[ctx->device]) {
+        EISEN_HIP_TRY(ctx, hipSetDevice(ctx->device));
+        EISEN_HIP_TRY(ctx, hipEventCreateWithFlags(&g_attn_bwd_scratch_done[ctx->device], hipEventDisableTiming));
+    }
     if (!g_attn_bwd_scratch_ptr[ctx->device]) {
         float* p = nullptr;
         EISEN_HIP_TRY(ctx, hipSetDevice(ctx->device));
@@ -818,12 +833,22 @@ extern "C" int eisen_hip_attention_backward_noalloc(eisen_ctx* ctx, const void* 
                            B * Hq <= kNoAllocMaxRows && B * Hq * S <= kNoAllocMaxRows,
                   EISEN_E_SHAPE, "attention_backward_noalloc: batch * query heads * seq = %zu * %zu * %zu exceeds the %zu rows of the fixed scratch",
                   B, Hq, S, kNoAllocMaxRows);
+    // Calls that share this GPU's array run one after the other: this call's stream first waits for the kernels of the
+    // previous one, on whatever context or stream that was.  A stream under graph capture cannot wait for an event recorded
+    // outside its graph: there the caller orders the calls (they are nodes of one graph, or the captures do not overlap).
+    std::lock_guard<std::mutex> lock(g_attn_bwd_scratch_mu);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    EISEN_HIP_TRY(ctx, hipStreamIsCapturing(ctx->stream, &capture));
+    hipEvent_t done = g_attn_bwd_scratch_done[ctx->device];
+    const bool ordered = capture == hipStreamCaptureStatusNone && done != nullptr;
+    if (ordered) EISEN_HIP_TRY(ctx, hipStreamWaitEvent(ctx->stream, done, 0));
     // per-kernel profiling creates events on first use: off for the duration of this call
     const bool prof_was = ctx->prof.enabled;
     ctx->prof.enabled = false;
     const int rc = attention_backward_common(ctx, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, q_strides, kv_strides, scale, causal,
                                              false, ctx->attn_scratch);
     ctx->prof.enabled = prof_was;
+    if (ordered) EISEN_HIP_TRY(ctx, hipEventRecord(done, ctx->stream));
     return rc;
 }
 

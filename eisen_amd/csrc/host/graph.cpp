@@ -312,8 +312,8 @@ bool Graph::window_take(size_t weight, const void* x, const void* dy, int dtype,
     WindowDW* e = nullptr;
     for (WindowDW& c : window_dw)
         if (c.weight == weight) e = &c;
-    if (e && (e->rows != rows || e->x.size() >= (size_t)EISEN_GEMM_MAX_KSEGMENTS)) {  // a piece of another length, or one too many
-        flush_weight_gradients();
+    if (e && (e->rows != rows || e->x.size() >= (size_t)EISEN_GEMM_MAX_KSEGMENTS)) {  // a piece of another length, or one too many:
+        flush_weight_gradients(weight);  // this weight's pieces are contracted now, the other weights and the pass count stay
         e = nullptr;
     }
     if (!e) {
@@ -327,15 +327,28 @@ bool Graph::window_take(size_t weight, const void* x, const void* dy, int dtype,
     return true;
 }
 
-void Graph::flush_weight_gradients() {
-    window_passes_ = 0;
+// only_weight: contract the pieces held for that one weight and leave the window as it is otherwise (the kept operands
+// stay allocated until the whole window is flushed: other weights' pieces may be the same buffers)
+void Graph::flush_weight_gradients(size_t only_weight) {
+    const bool all = only_weight == (size_t)-1;
+    if (all) window_passes_ = 0;
     if (window_dw.empty()) {
         // nothing waits for a launch; buffers kept for side-stream GEMMs go back once the main stream has waited for them
-        if (!retained_.empty()) side_join();
+        if (all && !retained_.empty()) side_join();
         return;
     }
     std::vector<WindowDW> list;
-    list.swap(window_dw);
+    if (all) {
+        list.swap(window_dw);
+    } else {
+        for (size_t i = 0; i < window_dw.size(); i++)
+            if (window_dw[i].weight == only_weight) {
+                list.push_back(std::move(window_dw[i]));
+                window_dw.erase(window_dw.begin() + (ptrdiff_t)i);
+                break;
+            }
+        if (list.empty()) return;
+    }
     // One launch per set of products with the same shape, number of pieces and accumulate state (equal tiles, and for a
     // model of equal blocks a whole number of rounds of the chip); sets of fewer tiles than the chip has CUs share one.
     struct Launch {
@@ -385,7 +398,7 @@ void Graph::flush_weight_gradients() {
         if (rc) break;
     }
     // the operands go back to the pool (stream order keeps them intact until the launches above have read them)
-    release_retained();
+    if (all) release_retained();
     check(rc, "weight gradients of the window");
 }
 

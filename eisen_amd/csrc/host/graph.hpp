@@ -218,7 +218,7 @@ class Graph {
     void set_weight_gradients_beside(bool on) { beside_ = on; }
     void set_weight_gradient_window(size_t backward_passes);
     size_t weight_gradient_window() const { return window_; }
-    void flush_weight_gradients();
+    void flush_weight_gradients(size_t only_weight = (size_t)-1);
     struct WindowDW {
         size_t weight, rows, in, out;
         std::vector<const void*> x, dy;  // one pair per piece, in the order the passes ran

@@ -23,6 +23,7 @@ int eisen_rope_table_get(eisen_ctx* ctx, size_t seq, size_t head_dim, const floa
             host[pos * half + p] = make_float2(cosf(theta), sinf(theta));
         }
     float* dev = nullptr;
+    ctx->driver_allocs++;
     EISEN_HIP_TRY(ctx, hipMallocAsync((void**)&dev, bytes, ctx->stream));
     EISEN_HIP_TRY(ctx, hipMemcpyAsync(dev, host.data(), bytes, hipMemcpyHostToDevice, ctx->stream));
     EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // `host` dies at return

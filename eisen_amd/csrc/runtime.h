@@ -47,6 +47,7 @@ struct eisen_ctx {
     std::unordered_map<void*, size_t> live;
     size_t in_use_bytes = 0, cached_bytes = 0;
     size_t peak_in_use_bytes = 0;  // high-water mark of in_use_bytes since the last reset
+    size_t driver_allocs = 0;      // requests for memory that reached the driver (device pool misses, workspace growth, tables, pinned staging)
     // pinned staging ring for asynchronous uploads: a slot is reused only after its copy's event fired
     struct StageSlot {
         void* ptr = nullptr;

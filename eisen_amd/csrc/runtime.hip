@@ -156,6 +156,7 @@ extern "C" int eisen_hip_malloc(eisen_ctx* ctx, size_t bytes, void** out) {
         it->second.pop_back();
         ctx->cached_bytes -= bytes;
     } else {
+        ctx->driver_allocs++;
         hipError_t e = hipMallocAsync(&p, bytes, ctx->stream);
         if (e != hipSuccess) {
             // out of memory: give cached blocks back and retry once
@@ -210,6 +211,13 @@ extern "C" int eisen_hip_mem_info(eisen_ctx* ctx, size_t* free_bytes, size_t* to
     return 0;
 }
 
+extern "C" int eisen_hip_driver_allocs(eisen_ctx* ctx, size_t* count_out) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, count_out != nullptr, EISEN_E_ARG, "driver_allocs: count_out is null");
+    *count_out = ctx->driver_allocs;
+    return 0;
+}
+
 extern "C" int eisen_hip_pool_stats(eisen_ctx* ctx, size_t* in_use_bytes, size_t* cached_bytes) {
     EISEN_CHECK_CTX(ctx);
     if (in_use_bytes) *in_use_bytes = ctx->in_use_bytes;
@@ -227,6 +235,7 @@ int eisen_workspace(eisen_ctx* ctx, size_t bytes, void** out) {
         ws = nullptr;
         ws_bytes = 0;
         size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        ctx->driver_allocs++;
         hipError_t e = hipMallocAsync(&ws, want, ctx->stream);
         if (e != hipSuccess)
             return eisen_set_error(ctx, EISEN_E_NOMEM, "workspace of %zu bytes: %s", want, hipGetErrorString(e));
@@ -255,6 +264,7 @@ int eisen_staging(eisen_ctx* ctx, size_t bytes, eisen_ctx::StageSlot** out) {
         s.ptr = nullptr;
         s.bytes = 0;
         size_t want = (bytes + (size_t(1) << 16) - 1) & ~((size_t(1) << 16) - 1);
+        ctx->driver_allocs++;
         EISEN_HIP_TRY(ctx, hipHostMalloc(&s.ptr, want, hipHostMallocDefault));
         s.bytes = want;
     }

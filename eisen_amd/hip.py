@@ -149,6 +149,11 @@ class Context:
         self._call("eisen_hip_pool_stats", C.byref(a), C.byref(b))
         return a.value, b.value
 
+    def driver_allocs(self):
+        n = _sz()
+        self._call("eisen_hip_driver_allocs", C.byref(n))
+        return n.value
+
     def pool_peak(self, reset=False):
         a = _sz()
         self._call("eisen_hip_pool_peak", C.byref(a), _i(int(reset)))
@@ -184,6 +189,12 @@ class Context:
         for e in arr[:min(n.value, 64)]:
             out[e.name.decode()] = dict(ms=e.ms, launches=int(e.launches), work=e.work, unit="flop" if e.work_is_flops else "byte")
         return out
+
+    def mfma_ceiling(self, lds_reads_per_16_mfma=0, iters=20000):
+        """TFLOP/s of a loop of nothing but bf16 MFMAs on every CU (operands in registers, or re-read from LDS)."""
+        out = C.c_double()
+        self._call("eisen_hip_mfma_ceiling", _i(lds_reads_per_16_mfma), _i(iters), C.byref(out))
+        return out.value
 
     # ---- by-name launch ---------------------------------------------------------------
     def module_load(self, path=HSACO_PATH):

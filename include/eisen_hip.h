@@ -78,6 +78,9 @@ int eisen_hip_pool_trim(eisen_ctx* ctx);
 int eisen_hip_mem_info(eisen_ctx* ctx, size_t* free_bytes, size_t* total_bytes);
 /* Bytes currently handed out / cached by the pool (diagnostics, tests). */
 int eisen_hip_pool_stats(eisen_ctx* ctx, size_t* in_use_bytes, size_t* cached_bytes);
+/* How often this context has asked the driver for memory so far (device-pool misses, workspace growth, rotary tables,
+ * pinned staging): a caller that must not allocate checks that a call leaves it unchanged (diagnostics, tests). */
+int eisen_hip_driver_allocs(eisen_ctx* ctx, size_t* count_out);
 /* Largest value in_use_bytes has had since the last call with reset != 0 (the activation high-water mark of a step). */
 int eisen_hip_pool_peak(eisen_ctx* ctx, size_t* peak_in_use_bytes, int reset);
 
@@ -124,6 +127,13 @@ typedef struct {
 } eisen_prof_entry;
 int eisen_hip_profile_start(eisen_ctx* ctx);
 int eisen_hip_profile_stop(eisen_ctx* ctx, eisen_prof_entry* out, size_t capacity, size_t* count_out);
+/* Measured MFMA ceiling of this GPU, for the roofline figures (no counterpart in the reference, whose kernels use no matrix
+ * instructions): runs a kernel of nothing but v_mfma_f32_32x32x16_bf16 on every CU (two waves per SIMD, four independent
+ * 32x32 accumulators per wave, `iters` x 16 MFMAs per wave), once untimed and once between two events on the context's
+ * stream, and returns the achieved TFLOP/s.  lds_reads_per_16_mfma = 0: operands stay in registers; 16: every contraction
+ * step re-reads two A and two B operands from LDS (the ratio of a 64x64 wave tile); 8: the ratio of a 128x128 wave tile.
+ * Synchronises the stream. */
+int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma, int iters, double* tflops_out);
 
 /* ---- elementwise ---------------------------------------------------------------------- */
 
@@ -334,9 +344,12 @@ int eisen_hip_attention_backward(eisen_ctx* ctx, const void* q, const void* k, c
  * results; the scratch the kernels need beyond the inputs and outputs, D = rowsum(dO o O) and -LSE/scale with one float
  * each per (batch, query head, position), lives in a fixed 8 MiB device array of the library instead of the context's growing
  * workspace, so the call reaches no hipMalloc / hipFree / pool routine.  Limit: B * Hq * S <= 1,048,576, larger
- * shapes return EISEN_E_SHAPE.  Every call on one GPU uses that GPU's one array: calls that overlap on a GPU (two
- * contexts, two streams) race; calls on one context are ordered by its stream.  Nothing in the array has to be
- * cleared between calls: the dQ kernel writes every row that the dK/dV kernel reads. */
+ * shapes return EISEN_E_SHAPE.  Every call on one GPU uses that GPU's one array.  Outside graph capture the library puts
+ * such calls in order itself: each call's stream first waits for an event recorded behind the previous call's kernels
+ * (another context on the GPU, or the context's other stream), so they cannot overlap.  Under graph capture no event
+ * from outside the graph can be waited for: calls captured into graphs that may run at the same time on one GPU race,
+ * and ordering them is the caller's job.  Nothing in the array has to be cleared between calls: the dQ kernel writes
+ * every row that the dK/dV kernel reads. */
 int eisen_hip_attention_backward_noalloc(eisen_ctx* ctx, const void* q, const void* k, const void* v, const void* out,
                                          const void* dout, const float* lse, void* dq, void* dk, void* dv, int dtype, size_t B,
                                          size_t S, size_t Hq, size_t Hkv, size_t hd, const long long* q_strides,

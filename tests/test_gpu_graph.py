@@ -295,6 +295,48 @@ def test_weight_gradient_window_flushes_when_a_gradient_is_read_cleared_or_outgr
         assert_close(b, a, 1e-4, f"weight gradient at read {i}")
 
 
+def test_weight_used_twice_per_pass_outgrows_its_window_entry_alone(ctx):
+    # A weight used twice per pass fills its eight pieces after four passes of a window of eight.  Only that weight's pieces
+    # are contracted then; the other weight's pieces and the pass count stay, so the window still ends with the eighth pass:
+    # three launches in all (the early one, then one per weight: the first weight's second contraction adds to its gradient,
+    # the other's assigns), nothing left allocated, and the sums of the per-pass order.  196 tiles of 256 x 256 per weight: the
+    # size from which a window's contraction runs as one launch.
+    hidden, rows = 3584, 128
+    w1_0, w2_0 = gen.normal(71, (hidden, hidden), 0.03), gen.normal(72, (hidden, hidden), 0.03)
+    xs = [gen.normal(80 + i, (rows, hidden)) for i in range(8)]
+    tg = [gen.uniform_ids(90 + i, (rows,), hidden) for i in range(8)]
+
+    def run(window):
+        g = G.Graph(ctx, G.BF16_MIXED)
+        w1, w2 = g.alloc(w1_0.shape, w1_0), g.alloc(w2_0.shape, w2_0)
+        g.mark_params()
+        g.set_weight_gradient_window(window)
+        opt = G.AdamW(g, [w1, w2], 1e-3)
+        opt.zero_grad()
+        ctx.sync()
+        base = ctx.pool_stats()[0]
+        ctx.profile_start()
+        for i in range(8):
+            loss = g.cross_entropy(g.matmul(g.matmul(g.matmul(g.input(xs[i]), w1), w2), w1), tg[i])
+            g.backward(loss)
+            g.clear_activations()
+        prof = ctx.profile_stop()
+        launches = sum(e["launches"] for k, e in prof.items() if k.endswith("_window"))
+        ctx.sync()
+        left = ctx.pool_stats()[0] - base
+        grads = g.sync_grad_to_cpu(w1), g.sync_grad_to_cpu(w2)
+        g.close()
+        return launches, left, grads
+
+    n_plain, left_plain, plain = run(0)
+    n_win, left_win, windowed = run(8)
+    assert n_plain == 0 and n_win == 3, (n_plain, n_win)
+    assert left_win == left_plain, "operands kept for the window were not given back when it ended"
+    for a, b, name in zip(plain, windowed, ("w1", "w2")):
+        assert a.any()
+        assert_close(b, a, 1e-4, f"weight gradient of {name}")
+
+
 @pytest.mark.parametrize("tie,checkpointing", [(True, False), (False, False), (True, True)], ids=["tied", "untied", "tied-recompute"])
 def test_weight_gradients_beside_the_chain_give_the_same_bits(ctx, tie, checkpointing):
     # Graph::set_weight_gradients_beside (the default): the weight-gradient GEMMs of narrow layers run on the side stream

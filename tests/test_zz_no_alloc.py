@@ -57,6 +57,43 @@ def test_attention_backward_noalloc_matches_the_allocating_entry_point(ctx):
     _run_both(ctx, F32, 2, 37, 4, 2, 16, seed=930)
 
 
+def test_attention_backward_noalloc_first_on_a_fresh_context_asks_the_driver_for_nothing():
+    """The allocation-free call as the first backward of a context of its own, on a shape larger than anything that context
+    has run: no workspace has been grown and no rotary table built that it could lean on.  The context's count of requests
+    to the driver (pool misses, workspace growth, tables, pinned staging) and its workspace must not move; the result must
+    equal the allocating entry point's, run afterwards."""
+    c2 = hip.Context(0)
+    try:
+        B, S, Hq, Hkv, hd = 2, 512, 8, 2, 64
+        sd, scale = 1.0 / np.sqrt(hd), float(1.0 / np.sqrt(hd))
+        q, do = gen.normal(950, (B, S, Hq, hd), sd), gen.normal(951, (B, S, Hq, hd), sd)
+        k, v = gen.normal(952, (B, S, Hkv, hd), sd), gen.normal(953, (B, S, Hkv, hd), sd)
+        dq_, dk_, dv_, ddo = (c2.upload(t, BF16) for t in (q, k, v, do))
+        out, lse = c2.malloc(q.size * 2), c2.malloc(B * Hq * S * 4)
+        got = [c2.malloc(q.size * 2), c2.malloc(k.size * 2), c2.malloc(k.size * 2)]
+        ref = [c2.malloc(q.size * 2), c2.malloc(k.size * 2), c2.malloc(k.size * 2)]
+        c2.attention_forward(dq_, dk_, dv_, out, lse, BF16, B, S, Hq, Hkv, hd, scale, True)
+        c2.sync()
+        before = c2.driver_allocs()
+        c2.attention_backward_noalloc(dq_, dk_, dv_, out, ddo, lse, *got, BF16, B, S, Hq, Hkv, hd, scale, True)
+        c2.sync()
+        assert c2.driver_allocs() == before, "the allocation-free entry point asked the driver for memory"
+        c2.attention_backward(dq_, dk_, dv_, out, ddo, lse, *ref, BF16, B, S, Hq, Hkv, hd, scale, True)
+        assert c2.driver_allocs() == before + 1, "the allocating entry point was expected to grow the workspace once"
+        for name, a, b, shape in zip(("dQ", "dK", "dV"), got, ref, (q.shape, k.shape, k.shape)):
+            assert np.array_equal(c2.download(a, shape, BF16), c2.download(b, shape, BF16)), name
+    finally:
+        c2.close()
+
+
+def test_attention_rejects_a_softmax_scale_that_is_not_positive_and_finite(ctx):
+    dummy = ctx.malloc(1 << 16)
+    for bad in (0.0, -0.125, float("inf"), float("nan"), 1e-40):
+        with pytest.raises(EisenHipError, match="scale"):
+            ctx.attention_backward(dummy, dummy, dummy, dummy, dummy, dummy, dummy, dummy, dummy, BF16, 1, 32, 2, 1, 64, bad, True)
+    dummy.free()
+
+
 def test_attention_backward_noalloc_rejects_shapes_beyond_its_scratch(ctx):
     dummy = ctx.malloc(4096)
     with pytest.raises(EisenHipError, match="exceeds"):
