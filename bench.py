@@ -307,6 +307,39 @@ def bench_c3(steps, warmup, hd=64):
                                   sample="oracle unfused attention chain fwd+bwd on 1 of 32 (batch, KV group) slices, scaled x32"))
 
 
+def bench_c3_ablation(steps, warmup):
+    """Where the time of the two config-3 backward kernels goes: each run leaves one part of their tile loop out
+    (eisen_hip_attention_ablation; results wrong by construction, memory accesses unchanged) and reports the kernels' average
+    durations; what a run gains against the full kernels is that part's share of the critical path."""
+    from eisen_amd import hip
+    B, S, Hq, Hkv, hd = 8, 1024, 16, 4, 64
+    ctx = hip.Context(0)
+    q, do = gen.normal(600, (B, Hq, S, hd), 1.0 / 8), gen.normal(601, (B, Hq, S, hd), 1.0 / 8)
+    k, v = gen.normal(602, (B, Hkv, S, hd), 1.0 / 8), gen.normal(603, (B, Hkv, S, hd), 1.0 / 8)
+    dq_, dk_, dv_, ddo = (ctx.upload(t, hip.BF16) for t in (q, k, v, do))
+    out, lse = ctx.malloc(q.size * 2), ctx.malloc(B * Hq * S * 4)
+    gq, gk, gv = ctx.malloc(q.size * 2), ctx.malloc(k.size * 2), ctx.malloc(k.size * 2)
+    qs, ks = (Hq * S * hd, hd, S * hd), (Hkv * S * hd, hd, S * hd)
+    ctx.attention_forward(dq_, dk_, dv_, out, lse, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+    parts = ["none (the kernels as shipped)", "LDS transpose reads", "16-byte LDS operand reads", "MFMAs after the softmax", "global-to-LDS tile loads",
+             "softmax arithmetic", "S and dP MFMAs", "none (again, after the others)"]
+    rows = []
+    for i, label in enumerate(parts):
+        ctx.attention_ablation(i % 7)
+        for _ in range(warmup):
+            ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+        ctx.sync()
+        ctx.profile_start()
+        for _ in range(steps):
+            ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+        prof = ctx.profile_stop()
+        rows.append(dict(left_out=label, dq_us=round(1e3 * prof["attn_bwd_dq_bf16"]["ms"] / steps, 2), dkv_us=round(1e3 * prof["attn_bwd_dkv_bf16"]["ms"] / steps, 2)))
+    ctx.attention_ablation(0)
+    ctx.close()
+    return dict(metric="config-3 attention backward kernel durations with one part of the tile loop left out", unit="us", steps=steps, warmup=warmup,
+                config=dict(workload="config3 causal GQA flash attention backward, B8 S1024 Hq16 Hkv4 hd64, [B,H,S,hd]"), rows=rows)
+
+
 def bench_c2(steps, warmup):
     """Config 2: fused softmax-cross-entropy forward+backward, bf16 [8192 x 32000]."""
     from eisen_amd import hip
@@ -373,6 +406,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="all", choices=["all", "c5", "c4", "c3", "c2"])
     ap.add_argument("--head-dim", type=int, default=64, choices=[32, 64, 128], help="c3: head size (the token count and Hq * hd = 1024 stay)")
+    ap.add_argument("--ablation", action="store_true", help="c3: time the backward kernels with one part of their tile loop left out at a time")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
     ap.add_argument("--no-window", action="store_true", help="c5: form every micro-batch's weight gradients in its own backward pass, as the reference does, "
                     "instead of once per optimizer step over the whole accumulation window")
@@ -392,6 +426,8 @@ def main():
                 out["other_configs"]["c5_per_pass_weight_gradients"] = {k: ref_order[k] for k in ("value", "unit", "ms_per_step", "steps", "warmup", "config")}
     elif w == "c4":
         out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside)
+    elif w == "c3" and args.ablation:
+        out = bench_c3_ablation(args.steps or 20, args.warmup if args.warmup is not None else 3)
     elif w == "c3":
         out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3, args.head_dim)
     else:

@@ -217,7 +217,8 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
 }
 
 // ---- backward: dQ (query-stationary); also writes D = rowsum(dO o O) for the dK/dV pass ------
-template <int HD, int GW>
+// ABL: a part of the tile loop left out for a measurement (AttnAblation; kAblNone is the kernel)
+template <int HD, int GW, int ABL = kAblNone>
 __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
     constexpr int QS = 4 / GW, BKV = 64, KSTEPS = HD / 16, DT = HD / 32;
     __shared__ __attribute__((aligned(1024))) bf16_t Ksb[2][BKV * HD];  // swizzled tiles, see DirectTile
@@ -275,11 +276,11 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
 
         auto tile = [&](int kt, auto masked_c) {
             constexpr bool MASKED = decltype(masked_c)::value;  // false: no key of the tile is masked for this wave
-            const bf16_t* Ks = Ksb[kt & 1];
-            const bf16_t* Vs = Vsb[kt & 1];
+            const bf16_t* Ks = Ksb[ABL == kAblTileLoads ? 0 : (kt & 1)];
+            const bf16_t* Vs = Vsb[ABL == kAblTileLoads ? 0 : (kt & 1)];
             wait_direct_loads();  // this wave's part of tile kt has landed
             __syncthreads();      // every wave is done with tile kt-1, whose buffer the next loads overwrite
-            if (kt + 1 < n_kt) {
+            if (ABL != kAblTileLoads && kt + 1 < n_kt) {
                 kv_tile.load(Kp, a.k_ss, (kt + 1) * BKV, a.S, Ksb[(kt + 1) & 1], wave, lane);
                 kv_tile.load(Vp, a.k_ss, (kt + 1) * BKV, a.S, Vsb[(kt + 1) & 1], wave, lane);
             }
@@ -292,17 +293,22 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                 for (int v = 0; v < 16; v++) { s[v] = 0.f; dp[v] = -Dq; }  // the MFMA chain delivers dP - D
 #pragma unroll
                 for (int st = 0; st < KSTEPS; st++) {
-                    const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Ks + tile_at<HD>(sub * 32 + c, st * 16 + 8 * g));
-                    const bf16x8 vf = *reinterpret_cast<const bf16x8*>(Vs + tile_at<HD>(sub * 32 + c, st * 16 + 8 * g));
-                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
-                    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[st], dp, 0, 0, 0);
+                    const bf16x8 kf = ABL == kAblOperandReads ? dof[st] : *reinterpret_cast<const bf16x8*>(Ks + tile_at<HD>(sub * 32 + c, st * 16 + 8 * g));
+                    const bf16x8 vf = ABL == kAblOperandReads ? qf[st] : *reinterpret_cast<const bf16x8*>(Vs + tile_at<HD>(sub * 32 + c, st * 16 + 8 * g));
+                    if (ABL == kAblScoreMfmas) {
+                        s[st] += (float)kf[0];
+                        dp[st] += (float)vf[0];
+                    } else {
+                        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[st], s, 0, 0, 0);
+                        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[st], dp, 0, 0, 0);
+                    }
                 }
                 bf16x8 dsf[2];
                 // a query past the end has LSE = +inf; keys past the end (their tile rows repeat the last
                 // key) and keys above the causal diagonal are masked
                 float p[16];
 #pragma unroll
-                for (int v = 0; v < 16; v++) p[v] = fast_exp2(fmaf(s[v], a.scale_log2e, -lse2));
+                for (int v = 0; v < 16; v++) p[v] = ABL == kAblSoftmax ? s[v] : fast_exp2(fmaf(s[v], a.scale_log2e, -lse2));
                 if (MASKED && ((a.causal && k0 + 31 > q0) || k0 + 32 > a.S)) {
                     const int rel = min(a.causal ? q : a.S - 1, a.S - 1) - k0;  // keys k0 + row > rel are masked
 #pragma unroll
@@ -310,13 +316,14 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                         if (acc_row(v, g) > rel) p[v] = 0.f;
                 }
 #pragma unroll
-                for (int v = 0; v < 16; v++) dsf[v >> 3][v & 7] = (bf16_t)(p[v] * dp[v]);
+                for (int v = 0; v < 16; v++) dsf[v >> 3][v & 7] = (bf16_t)(ABL == kAblSoftmax ? dp[v] : p[v] * dp[v]);
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                     for (int t = 0; t < 2; t++) {
-                        const bf16x8 ktr = lds_tr_operand_swz<HD>(Ks, sub * 32, dt * 32, t, lane);
-                        dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsf[t], dq[dt], 0, 0, 0);
+                        const bf16x8 ktr = ABL == kAblTransposedReads ? qf[dt * 2 + t] : lds_tr_operand_swz<HD>(Ks, sub * 32, dt * 32, t, lane);
+                        if (ABL == kAblSecondMfmas) dq[dt][0] += (float)ktr[0] * (float)dsf[t][0];
+                        else dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsf[t], dq[dt], 0, 0, 0);
                     }
             }
         };
@@ -712,7 +719,16 @@ void launch_bwd(eisen_ctx* ctx, AttnArgs a) {
     dim3 grid((unsigned)((a.paired ? (n_qblk + 1) / 2 : n_qblk) * per_q));
     {   // dQ = scale dS K: one of the four backward GEMMs (S and dP are recomputed here as well)
         EisenProfScope prof(ctx, "attn_bwd_dq_bf16", 1.0 * attn_pair_flops(a), true);
-        if (gw == 4) fa_bwd_dq_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
+        if (HD == 64 && gw == 4 && a.ablation != kAblNone) {  // measurement runs, at the shape the measurements are quoted for
+            switch (a.ablation) {
+                case kAblTransposedReads: fa_bwd_dq_kernel<64, 4, kAblTransposedReads><<<grid, 256, 0, ctx->stream>>>(a); break;
+                case kAblOperandReads: fa_bwd_dq_kernel<64, 4, kAblOperandReads><<<grid, 256, 0, ctx->stream>>>(a); break;
+                case kAblSecondMfmas: fa_bwd_dq_kernel<64, 4, kAblSecondMfmas><<<grid, 256, 0, ctx->stream>>>(a); break;
+                case kAblTileLoads: fa_bwd_dq_kernel<64, 4, kAblTileLoads><<<grid, 256, 0, ctx->stream>>>(a); break;
+                case kAblSoftmax: fa_bwd_dq_kernel<64, 4, kAblSoftmax><<<grid, 256, 0, ctx->stream>>>(a); break;
+                default: fa_bwd_dq_kernel<64, 4, kAblScoreMfmas><<<grid, 256, 0, ctx->stream>>>(a); break;
+            }
+        } else if (gw == 4) fa_bwd_dq_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
         else if (gw == 2) fa_bwd_dq_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
         else fa_bwd_dq_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
     }
@@ -752,6 +768,13 @@ extern "C" int eisen_hip_attention_forward(eisen_ctx* ctx, const void* q, const 
     return 0;
 }
 
+extern "C" int eisen_hip_attention_ablation(eisen_ctx* ctx, int part) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, part >= 0 && part < kAblCount, EISEN_E_ARG, "attention_ablation: part %d outside [0, %d)", part, (int)kAblCount);
+    ctx->attn_ablation = part;
+    return 0;
+}
+
 int eisen_attention_scratch_init(eisen_ctx* ctx) {
     EISEN_REQUIRE(ctx, ctx->device >= 0 && ctx->device < kMaxDevices, EISEN_E_ARG, "device index %d beyond the %d this library keeps scratch for", ctx->device, kMaxDevices);
     std::lock_guard<std::mutex> lock(g_attn_bwd_scratch_mu);
@@ -783,6 +806,7 @@ static int attention_backward_common(eisen_ctx* ctx, const void* q, const void* 
     if (rc) return rc;
     a.Q = q; a.K = k; a.V = v; a.O = out; a.dO = dout; a.LSE = const_cast<float*>(lse);
     a.dQ = dq; a.dK = dk; a.dV = dv;
+    a.ablation = ctx->attn_ablation;
     if (scratch) {
         a.D = scratch;
     } else {

@@ -10,9 +10,9 @@
 //   * A workgroup owns the keys of two 32-key blocks of one KV head, a heavy one and its light mirror image under the
 //     causal mask (equal work everywhere).  Its four waves each take every fourth (query head of the group, 32-query
 //     tile) item; their partial dK / dV meet in LDS once per key block, in wave order (no atomics).
-//   * A wave issues in order and its MFMAs and vector ALU work do not overlap each other; they overlap with those of
-//     the other wave on the SIMD.  So a wave must fit 256 registers (two per SIMD) and should spend as few cycles as
-//     possible on anything but MFMAs and the softmax:
+//   * A tile is a chain of latencies per wave (loads issued, operand reads, two dependent MFMA groups with the softmax
+//     between them) that the second wave of the SIMD covers in part.  So a wave must fit 256 registers (two per SIMD) and
+//     should spend as few cycles as possible on anything but MFMAs and the softmax:
 //       - every MFMA takes its accumulator in ordinary VGPRs (the file is compiled that way): with the AGPR form the
 //         compiler copies the score accumulators between the register files around the softmax of every tile;
 //       - Q / dO tiles and the two per-query statistics go from global memory straight into a private two-stage LDS
@@ -46,7 +46,8 @@ __device__ __forceinline__ void mfma(f32x16& acc, const bf16x8& a, const bf16x8&
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
 }
 
-template <int HD>
+// ABL: a part of the tile loop left out for a measurement (AttnAblation; kAblNone is the kernel)
+template <int HD, int ABL>
 __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
     constexpr int KSTEPS = HD / 16, DT = HD / 32, NST = 2;
     constexpr int TILE = 32 * HD;                        // elements of a Q or dO tile
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
         const int n_items = a.G * per_head;       // (query head of the group, query tile), head-major
         const int n_mine = n_items > wave ? (n_items - wave + 3) / 4 : 0;
 
-        auto stage_of = [&](int i) { return ring + (i % NST) * STAGE_BYTES; };
+        auto stage_of = [&](int i) { return ring + (ABL == kAblTileLoads ? 0 : (i % NST)) * STAGE_BYTES; };
         auto issue = [&](int i) {  // the loads of this wave's i-th tile into ring stage i % NST
             const int item = wave + 4 * i;
             const int hq = kvh * a.G + item / per_head, q0 = (qt_start + item % per_head) * 32;
@@ -166,10 +167,13 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
             }
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ks++) {
-                const bf16x8 qa = *reinterpret_cast<const bf16x8*>(Qs + tile_at<HD>(c, ks * 16 + 8 * g));
-                const bf16x8 da = *reinterpret_cast<const bf16x8*>(dOs + tile_at<HD>(c, ks * 16 + 8 * g));
+                const bf16x8 qa = ABL == kAblOperandReads ? vn[ks] : *reinterpret_cast<const bf16x8*>(Qs + tile_at<HD>(c, ks * 16 + 8 * g));
+                const bf16x8 da = ABL == kAblOperandReads ? kf[ks] : *reinterpret_cast<const bf16x8*>(dOs + tile_at<HD>(c, ks * 16 + 8 * g));
+                if (ABL == kAblScoreMfmas) { s[ks] += (float)qa[0]; dp[ks] += (float)da[0]; }
+                else {
                 mfma(s, qa, kf[ks]);
                 mfma(dp, da, vn[ks]);
+                }
             }
             // the transposed operands of the accumulation, requested before the softmax so that they arrive under it
             bf16x8 dotr[DT][2], qtr[DT][2];
@@ -177,15 +181,18 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
+                    if (ABL == kAblTransposedReads) { dotr[dt][t] = kf[dt * 2 + t]; qtr[dt][t] = vn[dt * 2 + t]; }
+                    else {
                     dotr[dt][t] = lds_tr_operand_swz<HD>(dOs, 0, dt * 32, t, lane);
                     qtr[dt][t] = lds_tr_operand_swz<HD>(Qs, 0, dt * 32, t, lane);
+                    }
                 }
             // the next tile's loads go out while the score MFMAs run (the other stage was read by tile i - 1, whose operand reads
             // have all returned)
-            if (i + 1 < n_mine) issue(i + 1);
+            if (ABL != kAblTileLoads && i + 1 < n_mine) issue(i + 1);
             float p[16];
 #pragma unroll
-            for (int v = 0; v < 16; v++) p[v] = fast_exp2(s[v] * a.scale_log2e);
+            for (int v = 0; v < 16; v++) p[v] = ABL == kAblSoftmax ? s[v] : fast_exp2(s[v] * a.scale_log2e);
             // only the diagonal tile is cut by the causal mask
             if (a.causal && q0 == k0) {
                 asm volatile("" ::: "memory");  // keeps this a branch taken once per head, not 16 selects per tile
@@ -197,14 +204,17 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 pf[v >> 3][v & 7] = (bf16_t)p[v];
-                dsf[v >> 3][v & 7] = (bf16_t)(p[v] * dp[v]);  // = -dS: dp holds D - dP
+                dsf[v >> 3][v & 7] = (bf16_t)(ABL == kAblSoftmax ? dp[v] : p[v] * dp[v]);  // = -dS: dp holds D - dP
             }
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
+                    if (ABL == kAblSecondMfmas) { dv[dt][0] += (float)pf[t][0] * (float)dotr[dt][t][0]; dk[dt][0] += (float)dsf[t][0] * (float)qtr[dt][t][0]; }
+                    else {
                     mfma(dv[dt], pf[t], dotr[dt][t]);
                     mfma(dk[dt], dsf[t], qtr[dt][t]);
+                    }
                 }
         }
 
@@ -258,6 +268,16 @@ bool eisen_attention_dkv32_supports(const AttnArgs& a) {
 void eisen_attention_launch_dkv32(eisen_ctx* ctx, const AttnArgs& a) {
     const int n_kb = (a.S + 31) / 32;  // 32-key blocks, handled in heavy / light pairs
     dim3 grid((unsigned)((n_kb + 1) / 2 * a.Hkv * a.B));
-    if (a.hd == 64) fa_bwd_dkv32_kernel<64><<<grid, 256, 0, ctx->stream>>>(a);
-    else fa_bwd_dkv32_kernel<32><<<grid, 256, 0, ctx->stream>>>(a);
+    if (a.hd == 64) {
+        switch (a.ablation) {  // hd 64 only: the head size the measurements are quoted for
+            case kAblTransposedReads: fa_bwd_dkv32_kernel<64, kAblTransposedReads><<<grid, 256, 0, ctx->stream>>>(a); break;
+            case kAblOperandReads: fa_bwd_dkv32_kernel<64, kAblOperandReads><<<grid, 256, 0, ctx->stream>>>(a); break;
+            case kAblSecondMfmas: fa_bwd_dkv32_kernel<64, kAblSecondMfmas><<<grid, 256, 0, ctx->stream>>>(a); break;
+            case kAblTileLoads: fa_bwd_dkv32_kernel<64, kAblTileLoads><<<grid, 256, 0, ctx->stream>>>(a); break;
+            case kAblSoftmax: fa_bwd_dkv32_kernel<64, kAblSoftmax><<<grid, 256, 0, ctx->stream>>>(a); break;
+            case kAblScoreMfmas: fa_bwd_dkv32_kernel<64, kAblScoreMfmas><<<grid, 256, 0, ctx->stream>>>(a); break;
+            default: fa_bwd_dkv32_kernel<64, kAblNone><<<grid, 256, 0, ctx->stream>>>(a); break;
+        }
+    }
+    else fa_bwd_dkv32_kernel<32, kAblNone><<<grid, 256, 0, ctx->stream>>>(a);
 }

@@ -20,6 +20,22 @@ struct AttnArgs {
     // backward only: when set ([S][hd/2] cos/sin), Q and K are rotary-embedded projections and dQ, dK are the
     // gradients of the projections before the rotation (the inverse rotation is applied as the gradients are stored)
     const float2* rope;
+    // measurement only (eisen_hip_attention_ablation): which part of the backward kernels' tile loop is left out, 0 = none
+    int ablation;
+};
+
+// Parts of a backward kernel's tile loop that an ablation run leaves out (the results are then wrong by construction; every
+// memory access that remains is one the full kernel makes as well).  What a run without one part gains is that part's
+// share of the kernel's critical path.
+enum AttnAblation {
+    kAblNone = 0,
+    kAblTransposedReads = 1,  // the LDS transpose reads (operands of the second MFMA group) -> registers already held
+    kAblOperandReads = 2,     // the 16-byte LDS operand reads of the score MFMAs -> registers already held
+    kAblSecondMfmas = 3,      // the MFMAs after the softmax (dK/dV kernel: dV and dK; dQ kernel: dQ)
+    kAblTileLoads = 4,        // the direct-to-LDS loads of every tile after the first
+    kAblSoftmax = 5,          // scale, exp2 and the dS product (the bf16 conversions stay)
+    kAblScoreMfmas = 6,       // the S and dP MFMAs
+    kAblCount = 7
 };
 
 // the key-stationary dK / dV kernel for head_dim 32 and 64 (attention_bwd.hip); a.D and a.L2 must have been written

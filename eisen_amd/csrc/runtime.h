@@ -66,6 +66,7 @@ struct eisen_ctx {
     size_t ws_side_bytes = 0;
     std::vector<eisen_rope_table> rope_tables;
     float* attn_scratch = nullptr;  // this device's copy of the file-scope scratch array in attention.hip (never freed)
+    int attn_ablation = 0;  // measurement only: the part of the attention backward kernels' tile loop to leave out (0 = none)
     eisen_prof prof;
     char last_error[512] = {0};
 };

@@ -389,6 +389,10 @@ class Context:
                    _ptr(dv), _i(dtype), _sz(B), _sz(S), _sz(Hq), _sz(Hkv), _sz(hd), self._strides(q_strides), self._strides(kv_strides),
                    _f(scale), _i(int(causal)))
 
+    def attention_ablation(self, part):
+        """Measurement only: leave one part of the backward kernels' tile loop out (0 = the real kernels)."""
+        self._call("eisen_hip_attention_ablation", _i(part))
+
     def attention_rope_backward(self, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, scale, causal=True):
         """Backward for rotary-embedded q, k: dq, dk come out as gradients of the un-rotated projections."""
         self._call("eisen_hip_attention_rope_backward", _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk),

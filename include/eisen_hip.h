@@ -355,6 +355,14 @@ int eisen_hip_attention_backward_noalloc(eisen_ctx* ctx, const void* q, const vo
                                          size_t S, size_t Hq, size_t Hkv, size_t hd, const long long* q_strides,
                                          const long long* kv_strides, float scale, int causal);
 
+/* Measurement aid for the two bf16 backward kernels at head_dim 64 with four query heads per KV head (no counterpart in
+ * the reference): until called again with 0, every eisen_hip_attention_backward* call on this context runs kernels that
+ * leave one part of their tile loop out, so that the part's share of the kernel's duration can be read from the
+ * difference.  THE RESULTS OF SUCH A CALL ARE WRONG BY CONSTRUCTION; the memory accesses that remain are those of the
+ * full kernels.  part: 1 the LDS transpose reads, 2 the 16-byte LDS operand reads, 3 the MFMAs after the softmax,
+ * 4 the global-to-LDS loads of every tile after the first, 5 the softmax arithmetic, 6 the S and dP MFMAs; 0 none. */
+int eisen_hip_attention_ablation(eisen_ctx* ctx, int part);
+
 /* eisen_hip_attention_backward for q and k that are rotary-embedded projections, q = rope(q0), k = rope(k0)
  * (src/nn/attention.rs:316-317 applies `g.rope` to both before the attention chain): dq and dk receive the
  * gradients of q0 and k0, i.e. the rotary backward (src/graph/ops/transform.rs:592-595) is applied to the f32
