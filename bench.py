@@ -41,10 +41,10 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs, per workload and per kernel symbol as
 # `symbol_of` names it; the summaries (command, calibration factors, per-kernel rows) are the files named here.
-TRAFFIC_SOURCE = {"c5": "profiles/c5_step_hbm_traffic_pmc.md", "c3": "profiles/c2_c3_hbm_traffic_pmc.md", "c2": "profiles/c2_c3_hbm_traffic_pmc.md"}
+TRAFFIC_SOURCE = {"c5": "profiles/c5_step_hbm_traffic_pmc.md", "c4": "profiles/c4_step_hbm_traffic_pmc.md", "c3": "profiles/c2_c3_hbm_traffic_pmc.md", "c2": "profiles/c2_c3_hbm_traffic_pmc.md"}
 MEASURED_TRAFFIC = {
     "c5": {"gemm_tn_bf16_f32out_256x256x32_window": 24423.6e6, "gemm_tn_bf16_f32out_256x256x32": 902.8e6, "gemm_nt_bf16_bf16out_256x128x64": 213.4e6},
-    "c4": {},
+    "c4": {"gemm_tn_bf16_f32out_128x128x64_splitk": 57.7e6},
     "c3": {"attn_bwd": 78.7e6 + 52.4e6},
     "c2": {"ce_fused_bf16": 1048.9e6},
 }

@@ -211,8 +211,17 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
     // Tile order: the workgroups resident at one time (about one per CU, in dispatch order) should cover a
     // compact block of C, so that the A and B panels they stream fit the caches together: C is walked in groups
     // of g.tile_group N tiles, all M tiles of a group before the next group, N index fastest inside a group.
-    int mt = blockIdx.y, nt = blockIdx.x;
-    if (g.tile_group < 0) {
+    int mt = blockIdx.y, nt = blockIdx.x, zz = blockIdx.z, gt = blockIdx.x;
+    if (g.split > 1) {
+        // Parts of a split contraction: the tiles of one part read the same K range of A and B, and nothing else does.  In
+        // dispatch order (x fastest, z = part slowest, handed to the XCDs round-robin) every XCD would hold tiles of every
+        // part and fetch every K range into its own L2; renumbered, an XCD holds whole parts.
+        const int gx = gridDim.x, gy = gridDim.y;
+        const int lin = xcd_contiguous_id(blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z), gx * gy * gridDim.z);
+        nt = gt = lin % gx;
+        mt = (lin / gx) % gy;
+        zz = lin / (gx * gy);
+    } else if (g.tile_group < 0) {
         xcd_block_tile<4, 8>(blockIdx.y * gridDim.x + blockIdx.x, gridDim.y, gridDim.x, mt, nt);
     } else if (g.tile_group > 0) {
         const int m_tiles = gridDim.y, n_tiles = gridDim.x;
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
         nt = grp * g.tile_group + within % width;
     }
     if (g.ngroup > 0) {  // which product this tile belongs to (uniform); static indices keep the tables in scalar registers
-        const int t = blockIdx.x;
+        const int t = gt;
         int first = 0;
         long long partial_off = g.grp_partial_off[0];
         g.A = g.grp_A[0]; g.B = g.grp_B[0]; g.C = g.grp_C[0]; g.N = g.grp_N[0];
@@ -243,7 +252,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
     }
     const int m0 = mt * BM, n0 = nt * BN;
     const int split = g.split > 1 ? g.split : 1;
-    const int bz = blockIdx.z / split, part = blockIdx.z % split;
+    const int bz = zz / split, part = zz % split;
     const int k_lo = part * g.k_part, k_hi = split > 1 ? min(g.K, k_lo + g.k_part) : g.K;
     const bf16_t* A = static_cast<const bf16_t*>(g.A) + (long long)bz * g.sA;
     const bf16_t* B = static_cast<const bf16_t*>(g.B) + (long long)bz * g.sB;
