@@ -44,7 +44,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 TRAFFIC_SOURCE = {"c5": "profiles/c5_step_hbm_traffic_pmc.md", "c4": "profiles/c4_step_hbm_traffic_pmc.md", "c3": "profiles/c2_c3_hbm_traffic_pmc.md", "c2": "profiles/c2_c3_hbm_traffic_pmc.md"}
 MEASURED_TRAFFIC = {
     "c5": {"gemm_tn_bf16_f32out_256x256x32_window": 24423.6e6, "gemm_tn_bf16_f32out_256x256x32": 902.8e6, "gemm_nt_bf16_bf16out_256x128x64": 213.4e6},
-    "c4": {"gemm_tn_bf16_f32out_128x128x64_splitk": 57.7e6},
+    "c4": {"gemm_tn_bf16_f32out_128x128x64_splitk": 57.7e6, "gemm_nt_bf16_bf16out_128x128x64": 35.7e6, "gemm_nt_bf16_bf16out_256x128x64_swiglu_bwd": 101.4e6,
+           "gemm_tn_bf16_f32out_64x64x32_grouped_splitk": 40.1e6, "gemm_nn_bf16_bf16out_128x128x64_splitk": 54.2e6, "gemm_nn_bf16_swiglu_256x128x32": 85.1e6},
     "c3": {"attn_bwd": 78.7e6 + 52.4e6},
     "c2": {"ce_fused_bf16": 1048.9e6},
 }
@@ -92,8 +93,10 @@ def roofline_of(name, e, workload, strict=False):
     table = MEASURED_TRAFFIC.get(workload, {})
     traffic = table.get(name)
     if strict and table and traffic is None:
-        raise KeyError(f"{workload}: the dominant kernel symbol {name!r} has no row in MEASURED_TRAFFIC (table of {TRAFFIC_SOURCE.get(workload)}); "
-                       f"a kernel was renamed or the counter runs are stale")
+        # not fatal (the line must still come out), but loud: a kernel was renamed or the counter runs are stale.  That every key of
+        # the table still names a profile entry of the library is checked by tests/test_bench_tables.py.
+        print(f"bench.py: {workload}: the dominant kernel symbol {name!r} has no row in MEASURED_TRAFFIC (table of {TRAFFIC_SOURCE.get(workload)})",
+              file=sys.stderr)
     src = TRAFFIC_SOURCE.get(workload) if traffic is not None else None
     if e["unit"] == "flop":
         achieved = e["work"] / (e["ms"] * 1e-3) / 1e12
