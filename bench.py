@@ -287,6 +287,7 @@ def bench_c3(steps, warmup, hd=64):
     bwd_flops = 4 * 2 * hd * (S * (S + 1) / 2) * B * Hq          # 34.39 GFLOP: four GEMMs, causal pairs, no recompute
     achieved = bwd_flops / (bwd_ms * 1e-3) / 1e12
     tokens = B * S
+    ceiling = mfma_ceiling(ctx)
     ctx.close()
     # CPU: the unfused chain on one batch element and one KV group (4 query heads), scaled by B*Hkv
     R.set_threads(1)
@@ -304,7 +305,7 @@ def bench_c3(steps, warmup, hd=64):
                               frac=round(achieved / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC["c3"]["attn_bwd"] if hd == 64 else None,
                               traffic_source=TRAFFIC_SOURCE["c3"] if hd == 64 else None,
                               kernel="attn_bwd (" + " + ".join(sorted(bwd_keys)) + ")", bwd_us=round(1e3 * bwd_ms, 2),
-                              algorithmic_gflop=round(bwd_flops / 1e9, 2)),
+                              algorithmic_gflop=round(bwd_flops / 1e9, 2), mfma_ceiling=ceiling),
                 kernels=kernel_table(prof),
                 cpu_baseline=dict(value=round(tokens / cpu_s, 2), unit="tokens/s", cores=1, kind="port",
                                   sample="oracle unfused attention chain fwd+bwd on 1 of 32 (batch, KV group) slices, scaled x32"))

@@ -108,7 +108,9 @@ __device__ __forceinline__ void xcd_block_tile(int lin, int m_tiles, int n_tiles
 
 // d(silu(gate) * up) for one element, given dh (src/graph/ops/elementwise.rs:442-455 for silu, :294-331 for mul)
 __device__ __forceinline__ void swiglu_backward_elem(float gate, float up, float dh, float& dgate, float& dup) {
-    const float sig = 1.0f / (1.0f + __expf(-gate));
+    // v_rcp_f32 (1 ulp) instead of the correctly rounded division's ten instructions: in a GEMM epilogue every vector
+    // instruction is exposed, and the result is rounded to bf16 or compared at 1e-4
+    const float sig = __builtin_amdgcn_rcpf(1.0f + __expf(-gate));
     const float silu = gate * sig;
     dgate = (dh * up) * (silu + sig * (1.0f - silu));
     dup = dh * silu;
