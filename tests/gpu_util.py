@@ -15,6 +15,8 @@ Tolerances (stated once, used by every GPU test), e = oracle value, a = GPU valu
                   relative L2 error of every gradient tensor <= 2e-2 and, per element,
                   |a - e| <= 2e-2 * |e| + 2e-2 * max|e|   (assert_close(..., step=True))
   integer/index : bit-exact
+A test that widens one of these bounds passes the widened figure to assert_close (outliers, worst_cap, row_scale,
+row_floor, step_outliers) and says why at the call; what every comparison of a run observed is printed at its end.
 """
 import numpy as np
 import pytest
