@@ -455,7 +455,9 @@ extern "C" int eisen_hip_profile_stop(eisen_ctx* ctx, eisen_prof_entry* out, siz
     EISEN_REQUIRE(ctx, count_out != nullptr, EISEN_E_ARG, "eisen_hip_profile_stop: null count_out");
     eisen_prof& p = ctx->prof;
     p.enabled = false;
-    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    // instrumented launches may sit on either stream: both have to be done before their events are read
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->side_stream));
+    EISEN_HIP_TRY(ctx, hipStreamSynchronize(ctx->main_stream));
     std::vector<eisen_prof_entry> acc(p.names.size());
     for (size_t i = 0; i < p.names.size(); i++) {
         std::memset(&acc[i], 0, sizeof(eisen_prof_entry));
