@@ -218,11 +218,19 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
 
 // ---- backward: dQ (query-stationary); also writes D = rowsum(dO o O) for the dK/dV pass ------
 // ABL: a part of the tile loop left out for a measurement (AttnAblation; kAblNone is the kernel)
+//
+// A block runs a long query block and then its short mirror image.  For head sizes up to 64 the two are one stream of
+// K / V tiles through the two LDS buffers (the short block's first tile is requested under the long block's last one), and
+// the rows of Q, dO and O of a wave's 32 queries arrive through three private LDS tiles of the wave, in whole rows; those of
+// the short block are requested while the long block's tile loop runs, so that its start-up costs no trip to memory.
 template <int HD, int GW, int ABL = kAblNone>
 __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
     constexpr int QS = 4 / GW, BKV = 64, KSTEPS = HD / 16, DT = HD / 32;
+    constexpr bool STREAM = HD <= 64 && ABL != kAblTileLoads;
+    constexpr int ROWS = 32 * HD;  // elements of a wave's Q, dO or O rows
     __shared__ __attribute__((aligned(1024))) bf16_t Ksb[2][BKV * HD];  // swizzled tiles, see DirectTile
     __shared__ __attribute__((aligned(1024))) bf16_t Vsb[2][BKV * HD];
+    __shared__ __attribute__((aligned(1024))) bf16_t Rows[STREAM ? 4 * 3 * ROWS : 8];  // [wave][Q | dO | O], swizzled like the tiles
     const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hsub = wave % GW, qsub = wave / GW;
@@ -230,38 +238,77 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
     const int kvh = blk.kvh, hq = kvh * a.G + blk.hgrp * GW + hsub, b = blk.b;
     const bf16_t* Kp = static_cast<const bf16_t*>(a.K) + b * a.k_sb + kvh * a.k_sh;
     const bf16_t* Vp = static_cast<const bf16_t*>(a.V) + b * a.k_sb + kvh * a.k_sh;
+    const long long head_off = b * a.q_sb + hq * a.q_sh;
+    const long long head_stat = ((long long)b * a.Hq + hq) * a.S;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
     DirectTile<HD, BKV, 4> kv_tile;
     kv_tile.init(a.k_ss, wave, lane);
+    DirectTile<HD, 32, 1> row_tile;
+    if (STREAM) row_tile.init(a.q_ss, 0, lane);
+    bf16_t* my_rows = Rows + (STREAM ? wave * 3 * ROWS : 0);
+    // the rows of Q, dO and O of this wave's queries of query block qb, straight into the wave's LDS tiles (rows past the
+    // end repeat the last row; their queries get LSE = +inf below)
+    auto request_rows = [&](int qb) {
+        const int first = (qb * QS + qsub) * 32;
+        row_tile.load_untracked(static_cast<const bf16_t*>(a.Q) + head_off, a.q_ss, first, a.S, my_rows, 0, lane);
+        row_tile.load_untracked(static_cast<const bf16_t*>(a.dO) + head_off, a.q_ss, first, a.S, my_rows + ROWS, 0, lane);
+        row_tile.load_untracked(static_cast<const bf16_t*>(a.O) + head_off, a.q_ss, first, a.S, my_rows + 2 * ROWS, 0, lane);
+    };
+    const int qblk_long = blk.n_qblk - 1 - blk.pair, qblk_short = blk.pair;
+    const bool two = a.paired && qblk_short < qblk_long;  // the middle block has no mirror
+    float lse_short = 0.f;  // STREAM: the short block's LSE, requested with the long block's
+    if (STREAM) {
+        kv_tile.load_untracked(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
+        kv_tile.load_untracked(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
+        request_rows(qblk_long);
+        const int qs = (qblk_short * QS + qsub) * 32 + c;
+        if (two && qs < a.S) lse_short = a.LSE[head_stat + qs];
+    }
+    int par = 0;  // STREAM: LDS buffer of the pass's first K / V tile
 
     for (int pass = 0; pass < 2; pass++) {
-        const int qblk = pass == 0 ? blk.n_qblk - 1 - blk.pair : blk.pair;
-        if (pass == 1 && (!a.paired || qblk >= blk.n_qblk - 1 - blk.pair)) break;
-        if (pass == 1) __syncthreads();
+        const int qblk = pass == 0 ? qblk_long : qblk_short;
+        if (pass == 1 && !two) break;
         const int q0 = (qblk * QS + qsub) * 32, q = q0 + c;
         const bool valid_q = q < a.S;
-        const long long qoff = b * a.q_sb + hq * a.q_sh + (long long)q * a.q_ss;
-        // the first K / V tile travels with the rows of Q, dO and O, not behind the reduction that waits for them
-        kv_tile.load(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
-        kv_tile.load(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
-
+        const long long qoff = head_off + (long long)q * a.q_ss;
+        const long long stat = head_stat + q;
         bf16x8 qf[KSTEPS], dof[KSTEPS];
-        float dpart = 0.f;
+        float dpart = 0.f, lse = 0.f;
+        if (STREAM) {
+            if (pass == 0) lse = valid_q ? a.LSE[stat] : 0.f;
+            else lse = lse_short;
+            wait_direct_loads();  // this wave's rows have landed (they are private to the wave: no barrier)
 #pragma unroll
-        for (int st = 0; st < KSTEPS; st++) {
-            const int d = st * 16 + 8 * g;
-            qf[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.Q) + qoff + d) : zero8;
-            dof[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.dO) + qoff + d) : zero8;
-            const bf16x8 of = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.O) + qoff + d) : zero8;
+            for (int st = 0; st < KSTEPS; st++) {
+                const int at = tile_at<HD>(c, st * 16 + 8 * g);
+                qf[st] = *reinterpret_cast<const bf16x8*>(my_rows + at);
+                dof[st] = *reinterpret_cast<const bf16x8*>(my_rows + ROWS + at);
+                const bf16x8 of = *reinterpret_cast<const bf16x8*>(my_rows + 2 * ROWS + at);
 #pragma unroll
-            for (int e = 0; e < 8; e++) dpart += (float)dof[st][e] * (float)of[e];
+                for (int e = 0; e < 8; e++) dpart += (float)dof[st][e] * (float)of[e];
+            }
+        } else {
+            if (pass == 1) __syncthreads();
+            // the first K / V tile travels with the rows of Q, dO and O, not behind the reduction that waits for them
+            kv_tile.load_untracked(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
+            kv_tile.load_untracked(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
+#pragma unroll
+            for (int st = 0; st < KSTEPS; st++) {
+                const int d = st * 16 + 8 * g;
+                qf[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.Q) + qoff + d) : zero8;
+                dof[st] = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.dO) + qoff + d) : zero8;
+                const bf16x8 of = valid_q ? *reinterpret_cast<const bf16x8*>(static_cast<const bf16_t*>(a.O) + qoff + d) : zero8;
+#pragma unroll
+                for (int e = 0; e < 8; e++) dpart += (float)dof[st][e] * (float)of[e];
+            }
+            lse = valid_q ? a.LSE[stat] : 0.f;
         }
         const float Dq = dpart + __shfl_xor(dpart, 32, 64);
-        const long long stat = ((long long)b * a.Hq + hq) * a.S + q;
-        const float lse2 = valid_q ? a.LSE[stat] * kLog2e : INFINITY;
+        const float lse2 = valid_q ? lse * kLog2e : INFINITY;
         if (valid_q && g == 0) {
             a.D[stat] = Dq;
-            a.L2[stat] = -a.LSE[stat] / a.scale;  // start value of the dK / dV kernel's score accumulators
+            a.L2[stat] = -lse / a.scale;  // start value of the dK / dV kernel's score accumulators
         }
 
         f32x16 dq[DT];
@@ -273,16 +320,32 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
         const int block_qmax = min(a.S - 1, (qblk * QS + QS - 1) * 32 + 31);
         const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
         const int my_qmax = q0 < a.S ? q0 + 31 : -1;
+        // STREAM, first pass: the short block's rows are requested under the second tile (the first one still shares the
+        // memory system with every block's start-up), or under the only tile
+        const int rows_at = pass == 0 && two ? min(1, n_kt - 1) : -1;
 
         auto tile = [&](int kt, auto masked_c) {
             constexpr bool MASKED = decltype(masked_c)::value;  // false: no key of the tile is masked for this wave
-            const bf16_t* Ks = Ksb[ABL == kAblTileLoads ? 0 : (kt & 1)];
-            const bf16_t* Vs = Vsb[ABL == kAblTileLoads ? 0 : (kt & 1)];
+            const int buf = STREAM ? ((kt + par) & 1) : 0;
+            const bf16_t* Ks = Ksb[ABL == kAblTileLoads ? 0 : (STREAM ? buf : (kt & 1))];
+            const bf16_t* Vs = Vsb[ABL == kAblTileLoads ? 0 : (STREAM ? buf : (kt & 1))];
             wait_direct_loads();  // this wave's part of tile kt has landed
-            __syncthreads();      // every wave is done with tile kt-1, whose buffer the next loads overwrite
-            if (ABL != kAblTileLoads && kt + 1 < n_kt) {
-                kv_tile.load(Kp, a.k_ss, (kt + 1) * BKV, a.S, Ksb[(kt + 1) & 1], wave, lane);
-                kv_tile.load(Vp, a.k_ss, (kt + 1) * BKV, a.S, Vsb[(kt + 1) & 1], wave, lane);
+            __syncthreads();      // every wave is done with the tile before, whose buffer the next loads overwrite
+            if (STREAM) {
+                // the next tile of the stream: this pass's, or the first one of the short block
+                const bool more = kt + 1 < n_kt;
+                if (more || (pass == 0 && two)) {
+                    const int first = more ? (kt + 1) * BKV : 0;
+                    kv_tile.load_untracked(Kp, a.k_ss, first, a.S, Ksb[buf ^ 1], wave, lane);
+                    kv_tile.load_untracked(Vp, a.k_ss, first, a.S, Vsb[buf ^ 1], wave, lane);
+                }
+                if (kt == rows_at) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the long block's rows have been read
+                    request_rows(qblk_short);
+                }
+            } else if (ABL != kAblTileLoads && kt + 1 < n_kt) {
+                kv_tile.load_untracked(Kp, a.k_ss, (kt + 1) * BKV, a.S, Ksb[(kt + 1) & 1], wave, lane);
+                kv_tile.load_untracked(Vp, a.k_ss, (kt + 1) * BKV, a.S, Vsb[(kt + 1) & 1], wave, lane);
             }
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
@@ -331,6 +394,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
         int kt = 0;
         for (; kt < n_plain; kt++) tile(kt, std::false_type{});
         for (; kt < n_kt; kt++) tile(kt, std::true_type{});
+        par = (par + n_kt) & 1;
         if (valid_q) {
             bf16_t* dQp = static_cast<bf16_t*>(a.dQ) + qoff;
 #pragma unroll

@@ -31,17 +31,6 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// One wave instruction of a direct-to-LDS load with a wave-uniform 64-bit base and a 32-bit byte offset per lane: lane l's
-// SIZE bytes land at lds_dst + SIZE * l.  Two scalar instructions and the load; no address arithmetic in vector registers.
-__device__ __forceinline__ void load_lds_16(const void* base, unsigned lane_offset, const void* lds_dst) {
-    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
-}
-__device__ __forceinline__ void load_lds_4(const void* base, unsigned lane_offset, const void* lds_dst) {
-    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
-}
-
 __device__ __forceinline__ void mfma(f32x16& acc, const bf16x8& a, const bf16x8& b) {
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
 }
@@ -103,14 +92,26 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
         const int n_mine = n_items > wave ? (n_items - wave + 3) / 4 : 0;
 
         auto stage_of = [&](int i) { return ring + (ABL == kAblTileLoads ? 0 : (i % NST)) * STAGE_BYTES; };
-        auto issue = [&](int i) {  // the loads of this wave's i-th tile into ring stage i % NST
-            const int item = wave + 4 * i;
-            const int hq = kvh * a.G + item / per_head, q0 = (qt_start + item % per_head) * 32;
+        // The tile that the next issue() requests, kept as running sums (all wave-uniform, so scalar registers): this wave's
+        // items are wave, wave + 4, ... in head-major order; a step of four tiles that runs past the head's last tile
+        // wraps into the next head.
+        int nrel = wave % per_head;                    // tile index within the head, from the diagonal tile
+        int nq0 = (qt_start + nrel) * 32;              // its first query
+        long long ntile, nstat;                        // element offsets of its Q / dO rows and of its statistics
+        {
+            const int hq = kvh * a.G + wave / per_head;
+            ntile = b * a.q_sb + hq * a.q_sh + (long long)nq0 * a.q_ss;
+            nstat = ((long long)b * a.Hq + hq) * a.S + nq0;
+        }
+        const long long tile_wrap = a.q_sh - (long long)per_head * 32 * a.q_ss, stat_wrap = (long long)a.S - per_head * 32;
+        auto issue = [&](int i) -> int {  // the loads of this wave's i-th tile into ring stage i % NST; returns the tile's first query
+            const int q0 = nq0;
             char* stage = stage_of(i);
-            const long long tile0 = b * a.q_sb + hq * a.q_sh + (long long)q0 * a.q_ss;  // wave-uniform
-            const char* qbase = reinterpret_cast<const char*>(static_cast<const bf16_t*>(a.Q) + tile0);
-            const char* dobase = reinterpret_cast<const char*>(static_cast<const bf16_t*>(a.dO) + tile0);
-            const char* sbase = reinterpret_cast<const char*>(a.D + ((long long)b * a.Hq + hq) * a.S + q0);
+            const char* qbase = reinterpret_cast<const char*>(static_cast<const bf16_t*>(a.Q) + ntile);
+            const char* dobase = reinterpret_cast<const char*>(static_cast<const bf16_t*>(a.dO) + ntile);
+            const char* sbase = reinterpret_cast<const char*>(a.D + nstat);
+            nrel += 4; nq0 += 128; ntile += 128 * a.q_ss; nstat += 128;
+            while (nrel >= per_head) { nrel -= per_head; nq0 -= per_head * 32; ntile += tile_wrap; nstat += stat_wrap; }
             if (q0 + 32 <= a.S) {
 #pragma unroll
                 for (int r = 0; r < Loader::PER_WAVE; r++) {
@@ -128,9 +129,10 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
                 }
                 load_lds_4(sbase, stat_off - 4 * (unsigned)(c - min(c, a.S - 1 - q0)), stage + 2 * TILE * 2);
             }
+            return q0;
         };
 
-        if (n_mine > 0) issue(0);
+        int q0_next = n_mine > 0 ? issue(0) : 0;
         bf16x8 kf[KSTEPS], vn[KSTEPS];  // K and -V of the 32 keys, MFMA B operands (requested before the first tile, used after it is)
 #pragma unroll
         for (int st = 0; st < KSTEPS; st++) {
@@ -145,8 +147,7 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
         }
         for (int i = 0; i < n_mine; i++) {
             wait_vmcnt<0>();  // tile i was requested in the middle of tile i - 1
-            const int item = wave + 4 * i;
-            const int q0 = (qt_start + item % per_head) * 32;
+            const int q0 = q0_next;
             const bf16_t* Qs = reinterpret_cast<const bf16_t*>(stage_of(i));
             const bf16_t* dOs = Qs + TILE;
             float* st = reinterpret_cast<float*>(stage_of(i) + 2 * TILE * 2);
@@ -189,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
                 }
             // the next tile's loads go out while the score MFMAs run (the other stage was read by tile i - 1, whose operand reads
             // have all returned)
-            if (ABL != kAblTileLoads && i + 1 < n_mine) issue(i + 1);
+            if (ABL != kAblTileLoads && i + 1 < n_mine) q0_next = issue(i + 1);
             float p[16];
 #pragma unroll
             for (int v = 0; v < 16; v++) p[v] = ABL == kAblSoftmax ? s[v] : fast_exp2(s[v] * a.scale_log2e);
@@ -217,7 +218,6 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
                     }
                 }
         }
-
         // the mirror block's K and V rows travel while this block's partial results are summed
         if (pass == 0 && n_qt - 1 - pair > pair) load_kv(n_qt - 1 - pair);
         // Sum the four waves' partial results through the (now idle) rings, dK then dV, and store.

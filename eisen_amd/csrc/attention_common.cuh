@@ -177,7 +177,46 @@ struct DirectTile {
                                              (lds_void_ptr)(lds_tile + (wave * PER_WAVE + i) * 512), 16, 0, 0);
         }
     }
+    // the same tile through load_lds_16 (see there); src + first_row * row_stride must be wave-uniform
+    __device__ __forceinline__ void load_untracked(const bf16_t* src, long long row_stride, int first_row, int limit_rows, bf16_t* lds_tile,
+                                                   int wave, int lane) const;
 };
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// One wave instruction of a direct-to-LDS load, written out: lane l's 16 (4) bytes land at lds_dst + 16 (4) * l.  The
+// compiler does not know that these write LDS, so it orders nothing around them: the kernel waits (s_waitcnt vmcnt)
+// before it reads what they bring and does not overwrite what is still being read.  With the builtin, the compiler may
+// place a wait for every load in flight in front of the next LDS read, the prefetched tile's included.
+//   *_saddr: wave-uniform 64-bit base and a 32-bit byte offset per lane (two scalar instructions and the load; no address
+//   arithmetic in vector registers); *_vaddr: a 64-bit address per lane.
+__device__ __forceinline__ void load_lds_16(const void* base, unsigned lane_offset, const void* lds_dst) {
+    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void load_lds_4(const void* base, unsigned lane_offset, const void* lds_dst) {
+    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void load_lds_16_vaddr(const void* lane_ptr, const void* lds_dst) {
+    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(lane_ptr) : "memory", "m0");
+}
+
+template <int HD, int ROWS, int WAVES>
+__device__ __forceinline__ void DirectTile<HD, ROWS, WAVES>::load_untracked(const bf16_t* src, long long row_stride, int first_row, int limit_rows,
+                                                                            bf16_t* lds_tile, int wave, int lane) const {
+    if (first_row + ROWS <= limit_rows) {  // whole tile in range (uniform)
+        const char* base = reinterpret_cast<const char*>(src + (long long)first_row * row_stride);
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) load_lds_16(base, off[i], lds_tile + (wave * PER_WAVE + i) * 512);
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) {
+        const int row = lane_row(wave, i, lane);
+        const int gr = min(first_row + row, limit_rows - 1);
+        load_lds_16_vaddr(src + (long long)gr * row_stride + lane_chunk(row, lane) * 8, lds_tile + (wave * PER_WAVE + i) * 512);
+    }
+}
 
 }  // namespace
