@@ -57,7 +57,16 @@ __device__ __forceinline__ QBlock decode_qblock(const AttnArgs& a) {
     QBlock r;
     r.n_qblk = (a.S + 32 * QS - 1) / (32 * QS);
     const int n_pairs = a.paired ? (r.n_qblk + 1) / 2 : r.n_qblk, groups = a.G / GW;
-    const int bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    // Blocks of one (batch, KV head) on one XCD.  Unpaired blocks differ in length under the causal mask: each XCD then
+    // starts its longest ones first (pair index slowest in launch order), so that the short ones fill the end.
+    int bid;
+    const int per = gridDim.x / 8;
+    if (!a.paired && gridDim.x % 8 == 0 && per % n_pairs == 0) {
+        const int gx = per / n_pairs, xcd = blockIdx.x % 8, local = blockIdx.x / 8;  // gx groups of n_pairs blocks per XCD
+        bid = (xcd * gx + local % gx) * n_pairs + local / gx;
+    } else {
+        bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    }
     r.pair = bid % n_pairs;
     const int y = (bid / n_pairs) % (a.Hkv * groups);
     r.kvh = y / groups;
@@ -107,8 +116,12 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
         const int n_kt = a.causal ? block_qmax / BKV + 1 : (a.S + BKV - 1) / BKV;
         const int my_qmax = q0 < a.S ? q0 + 31 : -1;
 
-        kv_tile.load(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
-        kv_tile.load(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
+        kv_tile.load_untracked(Kp, a.k_ss, 0, a.S, Ksb[0], wave, lane);
+        kv_tile.load_untracked(Vp, a.k_ss, 0, a.S, Vsb[0], wave, lane);
+        // The rows of Q have arrived before the tile loop: left pending, the compiler would wait for them at their first use
+        // inside it, in every tile and for every load in flight, the prefetched tile's included.
+#pragma unroll
+        for (int st = 0; st < KSTEPS; st++) asm volatile("" : "+v"(qf[st]));
         // One 64-key tile.  MASKED is a compile-time flag: the tiles entirely below the diagonal and inside
         // the sequence run a loop body with no mask code and no branches at all.
         auto tile = [&](int kt, auto masked_c) {
@@ -118,8 +131,8 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
             wait_direct_loads();  // this wave's part of tile kt has landed
             __syncthreads();      // one barrier per tile: every wave is done with tile kt-1, whose buffer the next loads overwrite
             if (kt + 1 < n_kt) {
-                kv_tile.load(Kp, a.k_ss, (kt + 1) * BKV, a.S, Ksb[(kt + 1) & 1], wave, lane);
-                kv_tile.load(Vp, a.k_ss, (kt + 1) * BKV, a.S, Vsb[(kt + 1) & 1], wave, lane);
+                kv_tile.load_untracked(Kp, a.k_ss, (kt + 1) * BKV, a.S, Ksb[(kt + 1) & 1], wave, lane);
+                kv_tile.load_untracked(Vp, a.k_ss, (kt + 1) * BKV, a.S, Vsb[(kt + 1) & 1], wave, lane);
             }
             const int k0 = kt * BKV;
             if (my_qmax < 0 || (a.causal && k0 > my_qmax)) return;                // wave-uniform
@@ -764,9 +777,10 @@ void launch_fwd(eisen_ctx* ctx, AttnArgs a) {
     const int gw = a.G % 4 == 0 ? 4 : (a.G % 2 == 0 ? 2 : 1);
     const int qs = 4 / gw;
     const int n_qblk = eisen_ceil_div(a.S, 32 * qs), per_q = a.Hkv * (a.G / gw) * a.B;
-    // pairing long and short query blocks balances the causal mask; it is only worth halving the
-    // number of blocks when at least two per CU remain
-    a.paired = a.causal && (long long)n_qblk * per_q >= 1024;
+    // One block per query block, the long ones launched first (decode_qblock): blocks that finish early take the next one,
+    // which evens out more than pairing long with short blocks does.  Pairing remains for grids that cannot be ordered so.
+    const long long blocks = (long long)n_qblk * per_q;
+    a.paired = a.causal && blocks >= 1024 && !(blocks % 8 == 0 && (blocks / 8) % n_qblk == 0);
     dim3 grid((unsigned)((a.paired ? (n_qblk + 1) / 2 : n_qblk) * per_q));
     if (gw == 4) fa_fwd_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
     else if (gw == 2) fa_fwd_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
