@@ -403,6 +403,65 @@ def brief(r):
     return {k: r[k] for k in keep if k in r}
 
 
+def bench_c3_timeline(steps, warmup):
+    """Where a wave of the three config-3 attention kernels spends its life: the kernels drop time stamps of every wave's progress
+    (eisen_hip_attention_timeline, the GPU's 100 MHz counter and its shader clock; the results are the usual ones) and this
+    reports, per kernel and in microseconds, the phases between the stamps averaged over the waves, the span from the first wave's
+    entry to the last wave's end and how far apart the waves finish."""
+    from eisen_amd import hip
+    B, S, Hq, Hkv, hd = 8, 1024, 16, 4, 64
+    ctx = hip.Context(0)
+    q, do = gen.normal(600, (B, Hq, S, hd), 1.0 / 8), gen.normal(601, (B, Hq, S, hd), 1.0 / 8)
+    k, v = gen.normal(602, (B, Hkv, S, hd), 1.0 / 8), gen.normal(603, (B, Hkv, S, hd), 1.0 / 8)
+    dq_, dk_, dv_, ddo = (ctx.upload(t, hip.BF16) for t in (q, k, v, do))
+    out, lse = ctx.malloc(q.size * 2), ctx.malloc(B * Hq * S * 4)
+    gq, gk, gv = ctx.malloc(q.size * 2), ctx.malloc(k.size * 2), ctx.malloc(k.size * 2)
+    qs, ks = (Hq * S * hd, hd, S * hd), (Hkv * S * hd, hd, S * hd)
+    waves = 4096                      # the forward runs 1024 blocks of four waves, the backward kernels 512
+    stamps = ctx.malloc(3 * waves * 16 * 8, zero=True)
+    ctx.attention_timeline(stamps, waves)
+    acc = None
+    for i in range(warmup + steps):
+        ctx.memset_zero(stamps, 3 * waves * 16 * 8)
+        ctx.attention_forward(dq_, dk_, dv_, out, lse, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+        ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, hip.BF16, B, S, Hq, Hkv, hd, 0.125, True, qs, ks)
+        ctx.sync()
+        if i < warmup:
+            continue
+        t = ctx.download(stamps, (3, waves, 8, 2), np.int64).astype(np.float64)
+        rows = []
+        for kern in range(3):
+            w = t[kern, :, :, 0] * 1e-2          # microseconds (100 MHz)
+            cyc = t[kern, :, :, 1]
+            live = w[:, 0] > 0
+            w, cyc = w[live], cyc[live]
+            t0 = w[:, 0].min()
+            second = w[:, 6] > 0                 # waves with a second block
+            end = np.where(second, w[:, 6], w[:, 3])
+            loop = (w[:, 2] - w[:, 1]) + np.where(second, w[:, 5] - w[:, 4], 0.0)
+            loop_cyc = (cyc[:, 2] - cyc[:, 1]) + np.where(second, cyc[:, 5] - cyc[:, 4], 0.0)
+            rows.append([float(live.sum()), float((w[:, 1] - w[:, 0]).mean()), float(loop.mean()), float((w[:, 3] - w[:, 2]).mean()),
+                         float(np.where(second, w[:, 4] - w[:, 3], 0.0).sum() / max(1, second.sum())),
+                         float(np.where(second, w[:, 6] - w[:, 5], 0.0).sum() / max(1, second.sum())),
+                         float(end.max() - t0), float(np.median(end) - t0), float(end.min() - t0), float(loop_cyc.sum() / (loop.sum() * 1e3))])
+        acc = np.array(rows) if acc is None else acc + np.array(rows)
+    acc /= steps
+    ctx.attention_timeline(None, 0)
+    # the dK/dV kernel's tile loop rebuilt from the same instructions on made-up data: what each part costs alone and together
+    model = {}
+    for label, parts in (("mfma", 1), ("mfma_valu", 3), ("mfma_valu_lds", 7), ("tile_loads", 8), ("all", 15)):
+        for wps in (1, 2):
+            model[f"{label}_{wps}_per_simd"] = round(ctx.attention_tile_model(parts, wps, 4000), 1)
+    ctx.close()
+    names = ["attn_fwd_bf16", "attn_bwd_dq_bf16", "attn_bwd_dkv_bf16"]
+    keys = ["waves", "entry_to_first_loop_us", "tile_loops_us", "first_block_stored_us", "to_second_loop_us", "second_block_stored_us",
+            "first_entry_to_last_end_us", "first_entry_to_median_end_us", "first_entry_to_first_end_us", "loop_clock_ghz"]
+    return dict(metric="config-3 attention kernels: a wave's life by phase (in-kernel time stamps, mean over waves)", unit="us", steps=steps, warmup=warmup,
+                config=dict(workload="config3 causal GQA flash attention fwd+bwd, B8 S1024 Hq16 Hkv4 hd64, [B,H,S,hd]"),
+                rows=[dict(kernel=n, **{k_: round(float(x), 2) for k_, x in zip(keys, r)}) for n, r in zip(names, acc)],
+                dkv_tile_loop_model_ns_per_tile_and_simd=model)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -411,6 +470,7 @@ def main():
     ap.add_argument("--workload", default="all", choices=["all", "c5", "c4", "c3", "c2"])
     ap.add_argument("--head-dim", type=int, default=64, choices=[32, 64, 128], help="c3: head size (the token count and Hq * hd = 1024 stay)")
     ap.add_argument("--ablation", action="store_true", help="c3: time the backward kernels with one part of their tile loop left out at a time")
+    ap.add_argument("--timeline", action="store_true", help="c3: where a wave of the three kernels spends its life (time stamps dropped inside the kernels)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
     ap.add_argument("--no-window", action="store_true", help="c5: form every micro-batch's weight gradients in its own backward pass, as the reference does, "
                     "instead of once per optimizer step over the whole accumulation window")
@@ -432,6 +492,8 @@ def main():
         out = bench_lm("c4", args.steps if args.steps is not None else 20, args.warmup if args.warmup is not None else 3, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside)
     elif w == "c3" and args.ablation:
         out = bench_c3_ablation(args.steps or 20, args.warmup if args.warmup is not None else 3)
+    elif w == "c3" and args.timeline:
+        out = bench_c3_timeline(args.steps or 10, args.warmup if args.warmup is not None else 3)
     elif w == "c3":
         out = bench_c3(args.steps or 20, args.warmup if args.warmup is not None else 3, args.head_dim)
     else:

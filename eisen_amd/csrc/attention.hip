@@ -75,7 +75,8 @@ __device__ __forceinline__ QBlock decode_qblock(const AttnArgs& a) {
     return r;
 }
 
-template <int HD, int GW>
+// TL: the kernel as it is plus time stamps (eisen_hip_attention_timeline)
+template <int HD, int GW, bool TL = false>
 __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
     constexpr int QS = 4 / GW, BKV = 64, KSTEPS = HD / 16, DT = HD / 32;
     __shared__ __attribute__((aligned(1024))) bf16_t Ksb[2][BKV * HD];  // swizzled tiles, see DirectTile
@@ -91,6 +92,7 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
     DirectTile<HD, BKV, 4> kv_tile;
     kv_tile.init(a.k_ss, wave, lane);
+    attn_stamp<TL>(a, 0, kStampStart, lane, wave);
 
     for (int pass = 0; pass < 2; pass++) {
         const int qblk = pass == 0 ? blk.n_qblk - 1 - blk.pair : blk.pair;  // the long one first
@@ -209,8 +211,10 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
         // tiles [0, n_plain) need no mask for any query of this wave: all their keys are <= q0 and < S
         const int n_plain = min(n_kt, min(a.causal ? (q0 + 1) / BKV : n_kt, a.S / BKV));
         int kt = 0;
+        attn_stamp<TL>(a, 0, kStampLoop + kStampsPerPass * pass, lane, wave);
         for (; kt < n_plain; kt++) tile(kt, std::false_type{});
         for (; kt < n_kt; kt++) tile(kt, std::true_type{});
+        attn_stamp<TL>(a, 0, kStampLoopEnd + kStampsPerPass * pass, lane, wave);
         l += __shfl_xor(l, 32, 64);
         if (valid_q) {
             const float inv = l > 0.f ? 1.0f / l : 0.f;
@@ -226,6 +230,7 @@ __global__ __launch_bounds__(256) void fa_fwd_kernel(AttnArgs a) {
                 }
             if (g == 0) a.LSE[((long long)b * a.Hq + hq) * a.S + q] = (m + log2f(l)) * kLn2;
         }
+        attn_stamp<TL>(a, 0, kStampStored + kStampsPerPass * pass, lane, wave);
     }
 }
 
@@ -258,6 +263,8 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
     kv_tile.init(a.k_ss, wave, lane);
     DirectTile<HD, 32, 1> row_tile;
     if (STREAM) row_tile.init(a.q_ss, 0, lane);
+    constexpr bool TL = ABL == kAblTimeline;
+    attn_stamp<TL>(a, 1, kStampStart, lane, wave);
     bf16_t* my_rows = Rows + (STREAM ? wave * 3 * ROWS : 0);
     // the rows of Q, dO and O of this wave's queries of query block qb, straight into the wave's LDS tiles (rows past the
     // end repeat the last row; their queries get LSE = +inf below)
@@ -405,8 +412,10 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
         };
         const int n_plain = my_qmax < 0 ? 0 : min(n_kt, min(a.causal ? (q0 + 1) / BKV : n_kt, a.S / BKV));
         int kt = 0;
+        attn_stamp<TL>(a, 1, kStampLoop + kStampsPerPass * pass, lane, wave);
         for (; kt < n_plain; kt++) tile(kt, std::false_type{});
         for (; kt < n_kt; kt++) tile(kt, std::true_type{});
+        attn_stamp<TL>(a, 1, kStampLoopEnd + kStampsPerPass * pass, lane, wave);
         par = (par + n_kt) & 1;
         if (valid_q) {
             bf16_t* dQp = static_cast<bf16_t*>(a.dQ) + qoff;
@@ -424,6 +433,7 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(AttnArgs a) {
                     *reinterpret_cast<bf16x4*>(dQp + dt * 32 + 8 * vg + 4 * g) = w;
                 }
         }
+        attn_stamp<TL>(a, 1, kStampStored + kStampsPerPass * pass, lane, wave);
     }
 }
 
@@ -782,7 +792,8 @@ void launch_fwd(eisen_ctx* ctx, AttnArgs a) {
     const long long blocks = (long long)n_qblk * per_q;
     a.paired = a.causal && blocks >= 1024 && !(blocks % 8 == 0 && (blocks / 8) % n_qblk == 0);
     dim3 grid((unsigned)((a.paired ? (n_qblk + 1) / 2 : n_qblk) * per_q));
-    if (gw == 4) fa_fwd_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
+    if (HD == 64 && gw == 4 && a.stamps) fa_fwd_kernel<64, 4, true><<<grid, 256, 0, ctx->stream>>>(a);
+    else if (gw == 4) fa_fwd_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
     else if (gw == 2) fa_fwd_kernel<HD, 2><<<grid, 256, 0, ctx->stream>>>(a);
     else fa_fwd_kernel<HD, 1><<<grid, 256, 0, ctx->stream>>>(a);
 }
@@ -804,6 +815,7 @@ void launch_bwd(eisen_ctx* ctx, AttnArgs a) {
                 case kAblSecondMfmas: fa_bwd_dq_kernel<64, 4, kAblSecondMfmas><<<grid, 256, 0, ctx->stream>>>(a); break;
                 case kAblTileLoads: fa_bwd_dq_kernel<64, 4, kAblTileLoads><<<grid, 256, 0, ctx->stream>>>(a); break;
                 case kAblSoftmax: fa_bwd_dq_kernel<64, 4, kAblSoftmax><<<grid, 256, 0, ctx->stream>>>(a); break;
+                case kAblTimeline: fa_bwd_dq_kernel<64, 4, kAblTimeline><<<grid, 256, 0, ctx->stream>>>(a); break;
                 default: fa_bwd_dq_kernel<64, 4, kAblScoreMfmas><<<grid, 256, 0, ctx->stream>>>(a); break;
             }
         } else if (gw == 4) fa_bwd_dq_kernel<HD, 4><<<grid, 256, 0, ctx->stream>>>(a);
@@ -831,6 +843,8 @@ extern "C" int eisen_hip_attention_forward(eisen_ctx* ctx, const void* q, const 
     int rc = fill_args(ctx, a, dtype, B, S, Hq, Hkv, hd, q_strides, kv_strides, scale, causal, "attention_forward");
     if (rc) return rc;
     a.Q = q; a.K = k; a.V = v; a.Out = out; a.LSE = lse;
+    a.stamps = ctx->attn_stamps;
+    a.stamp_waves = ctx->attn_stamp_waves;
     if (dtype == EISEN_BF16) {
         EISEN_REQUIRE(ctx, eisen_aligned(q, 16) && eisen_aligned(k, 16) && eisen_aligned(v, 16) && eisen_aligned(out, 16),
                       EISEN_E_ALIGN, "attention_forward: bf16 buffers must be 16-byte aligned");
@@ -850,6 +864,16 @@ extern "C" int eisen_hip_attention_ablation(eisen_ctx* ctx, int part) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, part >= 0 && part < kAblCount, EISEN_E_ARG, "attention_ablation: part %d outside [0, %d)", part, (int)kAblCount);
     ctx->attn_ablation = part;
+    return 0;
+}
+
+extern "C" int eisen_hip_attention_timeline(eisen_ctx* ctx, long long* stamps, size_t waves) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, (stamps == nullptr) == (waves == 0), EISEN_E_ARG, "attention_timeline: a buffer and a wave count come together (or neither)");
+    EISEN_REQUIRE(ctx, waves <= (size_t(1) << 24), EISEN_E_ARG, "attention_timeline: %zu waves is beyond 2^24", waves);
+    EISEN_REQUIRE(ctx, eisen_aligned(stamps, 8), EISEN_E_ALIGN, "attention_timeline: the buffer must be 8-byte aligned");
+    ctx->attn_stamps = stamps;
+    ctx->attn_stamp_waves = (int)waves;
     return 0;
 }
 
@@ -885,6 +909,9 @@ static int attention_backward_common(eisen_ctx* ctx, const void* q, const void* 
     a.Q = q; a.K = k; a.V = v; a.O = out; a.dO = dout; a.LSE = const_cast<float*>(lse);
     a.dQ = dq; a.dK = dk; a.dV = dv;
     a.ablation = ctx->attn_ablation;
+    a.stamps = ctx->attn_stamps;
+    a.stamp_waves = ctx->attn_stamp_waves;
+    if (a.stamps && a.ablation == kAblNone) a.ablation = kAblTimeline;
     if (scratch) {
         a.D = scratch;
     } else {

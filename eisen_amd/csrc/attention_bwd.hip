@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
     using Loader = DirectTile<HD, 32, 1>;
     constexpr int LOADS = 2 * Loader::PER_WAVE + 1;      // load instructions per tile
     static_assert(LOADS <= 63, "the tile in flight must fit the vmcnt counter");
-    static_assert(4 * 32 * HD * sizeof(float) <= 4 * NST * STAGE_BYTES, "the reduction reuses the rings");
+    static_assert(2 * 4 * 32 * HD * sizeof(float) <= 4 * NST * STAGE_BYTES, "the reduction of dK and dV reuses the rings");
     __shared__ __attribute__((aligned(1024))) char lds[4 * NST * STAGE_BYTES];
 
     const int lane = threadIdx.x & 63, g = lane >> 5, c = lane & 31;
@@ -61,6 +61,8 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
     const unsigned stat_off = (unsigned)(g == 0 ? (a.L2 - a.D) * 4 : 0) + 4 * (unsigned)c;
     Loader loader;
     loader.init(a.q_ss, 0, lane);
+    constexpr bool TL = ABL == kAblTimeline;
+    attn_stamp<TL>(a, 2, kStampStart, lane, wave);
 
     // K and V rows of this lane's key of key block kb_, as they are stored
     bf16x8 kraw[KSTEPS], vraw[KSTEPS];
@@ -145,6 +147,7 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
             // the prefetched tile's included)
             asm volatile("" : "+v"(vn[st]), "+v"(kf[st]));
         }
+        attn_stamp<TL>(a, 2, kStampLoop + kStampsPerPass * pass, lane, wave);
         for (int i = 0; i < n_mine; i++) {
             wait_vmcnt<0>();  // tile i was requested in the middle of tile i - 1
             const int q0 = q0_next;
@@ -218,25 +221,29 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
                     }
                 }
         }
+        attn_stamp<TL>(a, 2, kStampLoopEnd + kStampsPerPass * pass, lane, wave);
         // the mirror block's K and V rows travel while this block's partial results are summed
         if (pass == 0 && n_qt - 1 - pair > pair) load_kv(n_qt - 1 - pair);
-        // Sum the four waves' partial results through the (now idle) rings, dK then dV, and store.
-        float* red = reinterpret_cast<float*>(lds);  // [wave][32 keys][HD]
+        // Sum the four waves' partial results through the (now idle) rings and store: dK and dV in one round.
+        float* red = reinterpret_cast<float*>(lds);  // [dK | dV][wave][32 keys][HD]
         bf16_t* outs[2] = {static_cast<bf16_t*>(a.dK) + b * a.k_sb + kvh * a.k_sh, static_cast<bf16_t*>(a.dV) + b * a.k_sb + kvh * a.k_sh};
+        __syncthreads();  // every wave is done with its ring
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int at = (wave * 32 + acc_row(v, g)) * HD + dt * 32 + c;
+                red[at] = dk[dt][v] * -a.scale;
+                red[4 * 32 * HD + at] = dv[dt][v];
+            }
+        __syncthreads();
 #pragma unroll
         for (int which = 0; which < 2; which++) {
-            __syncthreads();  // every wave is done with its ring / with the previous reduction
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                for (int v = 0; v < 16; v++)
-                    red[(wave * 32 + acc_row(v, g)) * HD + dt * 32 + c] = which == 0 ? dk[dt][v] * -a.scale : dv[dt][v];
-            __syncthreads();
             for (int e0 = threadIdx.x * 8; e0 < 32 * HD; e0 += 256 * 8) {
                 float acc8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int w = 0; w < 4; w++) {
-                    const float* src = red + w * 32 * HD + e0;
+                    const float* src = red + (which * 4 + w) * 32 * HD + e0;
                     const float4 x0 = *reinterpret_cast<const float4*>(src);
                     const float4 x1 = *reinterpret_cast<const float4*>(src + 4);
                     acc8[0] += x0.x; acc8[1] += x0.y; acc8[2] += x0.z; acc8[3] += x0.w;
@@ -253,6 +260,7 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
             }
         }
         __syncthreads();  // the reduction's reads are over before the next pass refills the rings
+        attn_stamp<TL>(a, 2, kStampStored + kStampsPerPass * pass, lane, wave);
     }
 }
 
@@ -276,6 +284,7 @@ void eisen_attention_launch_dkv32(eisen_ctx* ctx, const AttnArgs& a) {
             case kAblTileLoads: fa_bwd_dkv32_kernel<64, kAblTileLoads><<<grid, 256, 0, ctx->stream>>>(a); break;
             case kAblSoftmax: fa_bwd_dkv32_kernel<64, kAblSoftmax><<<grid, 256, 0, ctx->stream>>>(a); break;
             case kAblScoreMfmas: fa_bwd_dkv32_kernel<64, kAblScoreMfmas><<<grid, 256, 0, ctx->stream>>>(a); break;
+            case kAblTimeline: fa_bwd_dkv32_kernel<64, kAblTimeline><<<grid, 256, 0, ctx->stream>>>(a); break;
             default: fa_bwd_dkv32_kernel<64, kAblNone><<<grid, 256, 0, ctx->stream>>>(a); break;
         }
     }

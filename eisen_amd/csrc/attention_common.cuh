@@ -22,6 +22,10 @@ struct AttnArgs {
     const float2* rope;
     // measurement only (eisen_hip_attention_ablation): which part of the backward kernels' tile loop is left out, 0 = none
     int ablation;
+    // measurement only (eisen_hip_attention_timeline): where the kernels drop time stamps of their waves' progress,
+    // [kernel][wave][8 stamps][100 MHz counter | shader clock]; waves from stamp_waves on drop none
+    long long* stamps;
+    int stamp_waves;
 };
 
 // Parts of a backward kernel's tile loop that an ablation run leaves out (the results are then wrong by construction; every
@@ -35,8 +39,12 @@ enum AttnAblation {
     kAblTileLoads = 4,        // the direct-to-LDS loads of every tile after the first
     kAblSoftmax = 5,          // scale, exp2 and the dS product (the bf16 conversions stay)
     kAblScoreMfmas = 6,       // the S and dP MFMAs
-    kAblCount = 7
+    kAblCount = 7,
+    kAblTimeline = 7          // nothing left out: the kernels as they are, plus the time stamps of AttnArgs::stamps
 };
+// Stamps of a wave: 0 kernel entered, 1 / 2 first tile loop begins / ends, 3 its results stored, 4 / 5 second tile loop
+// (the mirror block of a pair) begins / ends, 6 its results stored.  Kernel index: 0 forward, 1 dQ, 2 dK/dV.
+enum AttnStamp { kStampStart = 0, kStampLoop = 1, kStampLoopEnd = 2, kStampStored = 3, kStampsPerPass = 3 };
 
 // the key-stationary dK / dV kernel for head_dim 32 and 64 (attention_bwd.hip); a.D and a.L2 must have been written
 bool eisen_attention_dkv32_supports(const AttnArgs& a);
@@ -44,6 +52,18 @@ void eisen_attention_launch_dkv32(eisen_ctx* ctx, const AttnArgs& a);
 
 namespace {
 
+
+template <bool ON>
+__device__ __forceinline__ void attn_stamp(const AttnArgs& a, int kernel, int k, int lane, int wave) {
+    if (!ON) return;
+    const long long w = wall_clock64(), c = clock64();
+    const int id = (int)blockIdx.x * 4 + wave;
+    if (lane == 0 && id < a.stamp_waves) {
+        long long* p = a.stamps + ((size_t)kernel * a.stamp_waves + id) * 16 + 2 * k;
+        p[0] = w;
+        p[1] = c;
+    }
+}
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;

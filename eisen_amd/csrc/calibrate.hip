@@ -3,6 +3,7 @@
 // dense bf16) assumes the boost clock; under sustained matrix load the part holds a lower clock, so a kernel's distance
 // from what is reachable is better read against these numbers, measured in the same process as the kernel.
 // No counterpart in the reference (its kernels use no matrix instructions); a measurement aid, not an operator.
+#include "attention_common.cuh"
 #include "device_utils.cuh"
 #include "runtime.h"
 
@@ -58,6 +59,134 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(int iters, float* sin
     if (t == 12345.678f) sink[blockIdx.x * 512 + threadIdx.x] = t;  // keeps the loop alive; never true for these operands
 }
 
+// A model of the tile loop of the key-stationary attention-backward kernel (attention_bwd.hip), built from the same
+// instructions on made-up data, so that each of its parts can be timed alone and together at one or two waves per SIMD:
+//   1  the 16 MFMAs of a 32 x 32 x (head_dim 64) tile: two chains of four (S, dP), then four pairs (dV, dK)
+//   2  the vector work between them: scale, exp2, product and four packed bf16 conversions per element owned
+//   4  the LDS reads: eight 16-byte operand reads, eight broadcast reads of start values, sixteen 8-byte transposing reads
+//   8  the eight direct-to-LDS loads of 1 KB that bring a wave's next Q and dO tile (from a 4 MB region that stays in L2)
+// Four waves per block with a private two-stage ring each, as in the kernel.
+template <int PARTS>
+__global__ __launch_bounds__(256, 2) void tile_model_kernel(int iters, const char* gsrc, float* sink) {
+    constexpr int STAGE = 8448;
+    __shared__ __attribute__((aligned(1024))) char lds[4 * 2 * STAGE];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    char* ring = lds + wave * 2 * STAGE;
+    for (int i = lane; i < 2 * STAGE / 4; i += 64) reinterpret_cast<float*>(ring)[i] = 0.001f * (float)((i * 37) % 113) - 0.05f;
+    __syncthreads();
+    bf16x8 kf[4], vn[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            kf[j][e] = (bf16_t)(0.003f * (float)((lane * 7 + j * 13 + e * 5) % 61) - 0.09f);
+            vn[j][e] = (bf16_t)(0.004f * (float)((lane * 11 + j * 3 + e * 17) % 53) - 0.10f);
+        }
+    f32x16 dk[2], dv[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) { dk[t][v] = 0.f; dv[t][v] = 0.f; }
+    // 16 tiles of 8 KB per wave; the blocks of an XCD share one 512 KB set
+    const char* gbase = gsrc + (size_t)((blockIdx.x % 8) * 4 + wave) * 16 * 8192;
+    const unsigned loff = lane * 16;
+    if (PARTS & 8) {
+#pragma unroll
+        for (int r = 0; r < 8; r++) load_lds_16(gbase, loff + r * 1024, ring + r * 1024);
+    }
+    for (int it = 0; it < iters; it++) {
+        char* stage = ring + (it & 1) * STAGE;
+        if (PARTS & 8) wait_direct_loads();
+#pragma unroll
+        for (int j = 0; j < 4; j++) asm volatile("" : "+v"(kf[j]), "+v"(vn[j]));  // nothing is hoisted out of the loop
+        f32x16 s, dp;
+        if (PARTS & 4) {
+            const float* st = reinterpret_cast<const float*>(stage + 8192);
+#pragma unroll
+            for (int vg = 0; vg < 4; vg++) {
+                const float4 l4 = *reinterpret_cast<const float4*>(st + 8 * vg + 4 * (lane >> 5));
+                const float4 d4 = *reinterpret_cast<const float4*>(st + 32 + 8 * vg + 4 * (lane >> 5));
+                s[4 * vg] = l4.x; s[4 * vg + 1] = l4.y; s[4 * vg + 2] = l4.z; s[4 * vg + 3] = l4.w;
+                dp[4 * vg] = d4.x; dp[4 * vg + 1] = d4.y; dp[4 * vg + 2] = d4.z; dp[4 * vg + 3] = d4.w;
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; v++) { s[v] = -3.f - 0.01f * v; dp[v] = 0.5f; }
+            asm volatile("" : "+v"(s), "+v"(dp));
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            bf16x8 qa = kf[(ks + 1) & 3], da = vn[(ks + 1) & 3];
+            if (PARTS & 4) {
+                const int at = (lane & 31) * 128 + ((ks * 2 + (lane >> 5)) ^ (lane & 7)) * 16;  // byte offset, chunks permuted by row
+                qa = *reinterpret_cast<const bf16x8*>(stage + at);
+                da = *reinterpret_cast<const bf16x8*>(stage + 4096 + at);
+            }
+            if (PARTS & 1) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vn[ks], dp, 0, 0, 0);
+            } else { s[ks] += (float)qa[0]; dp[ks] += (float)da[0]; }
+        }
+        bf16x8 dotr[2][2], qtr[2][2];
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                if (PARTS & 4) {
+                    const int at = (t * 16 + (lane >> 4) * 2) * 64 + ((dt * 4 + ((lane >> 2) & 3)) ^ (lane & 7)) * 8;  // element offset, rows 0..30
+                    const bf16_t* p0 = reinterpret_cast<const bf16_t*>(stage + 4096) + at;
+                    const bf16_t* p1 = reinterpret_cast<const bf16_t*>(stage) + at;
+                    dotr[dt][t] = concat4(lds_read_tr(p0), lds_read_tr(p0 + 64));
+                    qtr[dt][t] = concat4(lds_read_tr(p1), lds_read_tr(p1 + 64));
+                } else { dotr[dt][t] = kf[dt * 2 + t]; qtr[dt][t] = vn[dt * 2 + t]; }
+            }
+        if ((PARTS & 8) && it + 1 < iters) {
+            char* nxt = ring + ((it + 1) & 1) * STAGE;
+            const char* g = gbase + ((it + 1) & 15) * 8192;
+#pragma unroll
+            for (int r = 0; r < 8; r++) load_lds_16(g, loff + r * 1024, nxt + r * 1024);
+        }
+        bf16x8 pf[2], dsf[2];
+        if (PARTS & 2) {
+            float p[16];
+#pragma unroll
+            for (int v = 0; v < 16; v++) p[v] = fast_exp2(s[v] * 0.18f);
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                pf[v >> 3][v & 7] = (bf16_t)p[v];
+                dsf[v >> 3][v & 7] = (bf16_t)(p[v] * dp[v]);
+            }
+        } else {
+            typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                u32x4 x, y;
+#pragma unroll
+                for (int e = 0; e < 4; e++) { x[e] = __builtin_bit_cast(unsigned, s[t * 4 + e]); y[e] = __builtin_bit_cast(unsigned, dp[t * 4 + e]); }
+                pf[t] = __builtin_bit_cast(bf16x8, x);
+                dsf[t] = __builtin_bit_cast(bf16x8, y);
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                if (PARTS & 1) {
+                    dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[t], dotr[dt][t], dv[dt], 0, 0, 0);
+                    dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[t], qtr[dt][t], dk[dt], 0, 0, 0);
+                } else { dv[dt][t] += (float)pf[t][0] * (float)dotr[dt][t][0]; dk[dt][t] += (float)dsf[t][0] * (float)qtr[dt][t][0]; }
+            }
+    }
+    wait_direct_loads();
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) t += dk[k][v] + dv[k][v];
+    if (t == 12345.678f) sink[blockIdx.x * 256 + threadIdx.x] = t;  // keeps the loop alive; never true for these operands
+}
+
 }  // namespace
 
 extern "C" int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma, int iters, double* tflops_out) {
@@ -93,5 +222,50 @@ extern "C" int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma,
     if (err != hipSuccess) return eisen_set_error(ctx, (int)err, "mfma_ceiling: %s", hipGetErrorString(err));
     const double flops = (double)blocks * 8.0 * (double)iters * 16.0 * 32768.0;  // waves x iterations x MFMAs x flop per MFMA
     *tflops_out = ms > 0.f ? flops / (ms * 1e-3) / 1e12 : 0.0;
+    return 0;
+}
+
+extern "C" int eisen_hip_attention_tile_model(eisen_ctx* ctx, int parts, int waves_per_simd, int iters, double* ns_per_tile_out) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, ns_per_tile_out != nullptr, EISEN_E_ARG, "attention_tile_model: ns_per_tile_out is null");
+    EISEN_REQUIRE(ctx, parts == 1 || parts == 3 || parts == 7 || parts == 8 || parts == 15, EISEN_E_ARG,
+                  "attention_tile_model: parts must be 1, 3, 7, 8 or 15, got %d", parts);
+    EISEN_REQUIRE(ctx, waves_per_simd == 1 || waves_per_simd == 2, EISEN_E_ARG, "attention_tile_model: waves_per_simd must be 1 or 2, got %d", waves_per_simd);
+    EISEN_REQUIRE(ctx, iters > 0 && iters <= (1 << 20), EISEN_E_ARG, "attention_tile_model: iters %d outside (0, 2^20]", iters);
+    hipDeviceProp_t prop;
+    EISEN_HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    const int blocks = prop.multiProcessorCount * waves_per_simd;  // four waves per block, one per SIMD
+    const size_t src_bytes = (size_t)8 * 4 * 16 * 8192, sink_bytes = (size_t)blocks * 256 * sizeof(float);
+    void* ws = nullptr;
+    int rc = eisen_workspace(ctx, src_bytes + sink_bytes, &ws);
+    if (rc) return rc;
+    char* src = static_cast<char*>(ws);
+    float* sink = reinterpret_cast<float*>(src + src_bytes);
+    rc = eisen_hip_fill(ctx, src, EISEN_F32, 0.f, src_bytes / sizeof(float));
+    if (rc) return rc;
+    hipEvent_t e0, e1;
+    EISEN_HIP_TRY(ctx, hipEventCreate(&e0));
+    EISEN_HIP_TRY(ctx, hipEventCreate(&e1));
+    auto launch = [&](int n) {
+        switch (parts) {
+            case 1: tile_model_kernel<1><<<blocks, 256, 0, ctx->stream>>>(n, src, sink); break;
+            case 3: tile_model_kernel<3><<<blocks, 256, 0, ctx->stream>>>(n, src, sink); break;
+            case 7: tile_model_kernel<7><<<blocks, 256, 0, ctx->stream>>>(n, src, sink); break;
+            case 8: tile_model_kernel<8><<<blocks, 256, 0, ctx->stream>>>(n, src, sink); break;
+            default: tile_model_kernel<15><<<blocks, 256, 0, ctx->stream>>>(n, src, sink); break;
+        }
+    };
+    launch(iters / 8 + 1);  // warm-up: clocks, code object, the source region into the L2
+    hipError_t err = hipEventRecord(e0, ctx->stream);
+    launch(iters);
+    if (err == hipSuccess) err = hipGetLastError();
+    if (err == hipSuccess) err = hipEventRecord(e1, ctx->stream);
+    if (err == hipSuccess) err = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (err != hipSuccess) return eisen_set_error(ctx, (int)err, "attention_tile_model: %s", hipGetErrorString(err));
+    *ns_per_tile_out = (double)ms * 1e6 / (double)iters / (double)waves_per_simd;  // a SIMD finishes waves_per_simd tiles per iteration
     return 0;
 }

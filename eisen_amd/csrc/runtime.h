@@ -67,6 +67,8 @@ struct eisen_ctx {
     std::vector<eisen_rope_table> rope_tables;
     float* attn_scratch = nullptr;  // this device's copy of the file-scope scratch array in attention.hip (never freed)
     int attn_ablation = 0;  // measurement only: the part of the attention backward kernels' tile loop to leave out (0 = none)
+    long long* attn_stamps = nullptr;  // measurement only: where the attention kernels drop time stamps (eisen_hip_attention_timeline)
+    int attn_stamp_waves = 0;
     eisen_prof prof;
     char last_error[512] = {0};
 };

@@ -393,6 +393,16 @@ class Context:
         """Measurement only: leave one part of the backward kernels' tile loop out (0 = the real kernels)."""
         self._call("eisen_hip_attention_ablation", _i(part))
 
+    def attention_timeline(self, stamps=None, waves=0):
+        """Measurement only: the hd-64 attention kernels drop time stamps into `stamps` (3 * waves * 16 int64) until called with None."""
+        self._call("eisen_hip_attention_timeline", _ptr(stamps), _sz(waves))
+
+    def attention_tile_model(self, parts, waves_per_simd=2, iters=4000):
+        """Measurement only: ns per tile and SIMD of a model of the dK/dV kernel's tile loop (parts: 1 MFMA, 3 +VALU, 7 +LDS, 8 loads, 15 all)."""
+        out = C.c_double(0.0)
+        self._call("eisen_hip_attention_tile_model", _i(parts), _i(waves_per_simd), _i(iters), C.byref(out))
+        return out.value
+
     def attention_rope_backward(self, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, scale, causal=True):
         """Backward for rotary-embedded q, k: dq, dk come out as gradients of the un-rotated projections."""
         self._call("eisen_hip_attention_rope_backward", _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(dq), _ptr(dk),

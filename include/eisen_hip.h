@@ -363,6 +363,21 @@ int eisen_hip_attention_backward_noalloc(eisen_ctx* ctx, const void* q, const vo
  * 4 the global-to-LDS loads of every tile after the first, 5 the softmax arithmetic, 6 the S and dP MFMAs; 0 none. */
 int eisen_hip_attention_ablation(eisen_ctx* ctx, int part);
 
+/* Measurement aid for the three bf16 attention kernels at head_dim 64 with four query heads per KV head (no counterpart in
+ * the reference): while a buffer is set, every wave of those kernels drops time stamps of its progress, the results are
+ * the usual ones.  stamps: device memory for 3 * waves * 16 values of 8 bytes, laid out [kernel: 0 forward, 1 dQ,
+ * 2 dK/dV][wave = block * 4 + wave of the block][stamp 0..7][0: the GPU's 100 MHz counter, 1: its shader clock]; waves
+ * beyond `waves` drop nothing.  Stamp 0: kernel entered; 1, 2: first tile loop begins, ends; 3: its results stored; 4, 5,
+ * 6: the same for the second query (key) block of a paired workgroup, zero where there is none.  (nullptr, 0) ends it. */
+int eisen_hip_attention_timeline(eisen_ctx* ctx, long long* stamps, size_t waves);
+
+/* Measurement aid (no counterpart in the reference): a model of the tile loop of the key-stationary attention-backward
+ * kernel at head_dim 64, built from the same instructions on made-up data, timed with any of its parts alone or together.
+ * parts: 1 the sixteen MFMAs of a tile; 3 those and the vector work between them; 7 those and the tile's LDS reads; 8 only
+ * the eight 1 KB direct-to-LDS loads that bring a wave's next tile (from a region that stays in the L2); 15 everything.
+ * waves_per_simd: 1 or 2 (the kernel runs two).  *ns_per_tile_out: time per tile and SIMD over `iters` tiles per wave. */
+int eisen_hip_attention_tile_model(eisen_ctx* ctx, int parts, int waves_per_simd, int iters, double* ns_per_tile_out);
+
 /* eisen_hip_attention_backward for q and k that are rotary-embedded projections, q = rope(q0), k = rope(k0)
  * (src/nn/attention.rs:316-317 applies `g.rope` to both before the attention chain): dq and dk receive the
  * gradients of q0 and k0, i.e. the rotary backward (src/graph/ops/transform.rs:592-595) is applied to the f32
