@@ -1071,7 +1071,7 @@ def test_bmm_batched(ctx):
 oracle_attention = R.attention_chain
 
 
-def _attn_case(ctx, dtype, B, S, Hq, Hkv, hd, causal=True, seed=500, layout="bshd"):
+def _attn_case(ctx, dtype, B, S, Hq, Hkv, hd, causal=True, seed=500, layout="bshd", dq_bounds=None):
     sd = 1.0 / np.sqrt(hd)
     q, do = prep(gen.normal(seed, (B, S, Hq, hd), sd), dtype), prep(gen.normal(seed + 1, (B, S, Hq, hd), sd), dtype)
     k, v = prep(gen.normal(seed + 2, (B, S, Hkv, hd), sd), dtype), prep(gen.normal(seed + 3, (B, S, Hkv, hd), sd), dtype)
@@ -1095,7 +1095,7 @@ def _attn_case(ctx, dtype, B, S, Hq, Hkv, hd, causal=True, seed=500, layout="bsh
     # backward takes the forward's own O (as the graph does)
     gq, gk, gv = ctx.malloc(q.size * 4), ctx.malloc(k.size * 4), ctx.malloc(k.size * 4)
     ctx.attention_backward(dq_, dk_, dv_, out, ddo, lse, gq, gk, gv, dtype, B, S, Hq, Hkv, hd, float(scale), causal, qs, ks)
-    assert_close(back(dn(ctx, gq, shape_q, dtype)), edq, tol, "attn dQ")
+    assert_close(back(dn(ctx, gq, shape_q, dtype)), edq, tol, "attn dQ", **(dq_bounds or {}))
     assert_close(back(dn(ctx, gk, shape_k, dtype)), edk, tol, "attn dK")
     assert_close(back(dn(ctx, gv, shape_k, dtype)), edv, tol, "attn dV")
     # LSE closed form on a few rows: log sum_j exp(scale q.k_j) over visible keys
@@ -1129,6 +1129,17 @@ def test_attention_f32_non_causal_and_reference_vector(ctx):
                                            (1, 130, 2, 1, 128), (1, 96, 6, 2, 64), (1, 257, 4, 1, 64)])
 def test_attention_bf16_mfma(ctx, B, S, Hq, Hkv, hd):
     _attn_case(ctx, BF16, B, S, Hq, Hkv, hd)
+
+
+@pytest.mark.parametrize("B,S,Hq,Hkv,hd,layout", [(64, 96, 32, 8, 64, "bshd"), (129, 64, 16, 4, 64, "bhsd"), (64, 128, 16, 4, 32, "bshd")])
+def test_attention_bf16_many_short_sequences(ctx, B, S, Hq, Hkv, hd, layout):
+    """Grids of a thousand workgroups and more over short sequences: the dQ kernel then pairs a long query block with its short mirror
+    image and runs both as one stream of K / V tiles, here with one tile per block and (S = 96) a middle block without a mirror; the
+    forward starts the longest blocks first where the grid divides evenly over the XCDs and falls back to pairs where it does not
+    (129 x 4 KV heads).  dQ of the second query of a sequence is a difference of two nearly equal terms whose D = rowsum(dO o O)
+    comes from the bf16 O (as in the reference's chain, where O is a bf16 tensor): with thousands of sequences a few such elements in
+    100,000 pass the bound 2e-2 (|e| + rms), the worst observed at 2.6 x; the bounds are those of the full-size config-3 test."""
+    _attn_case(ctx, BF16, B, S, Hq, Hkv, hd, layout=layout, dq_bounds=dict(outliers=2e-4, worst_cap=3.0))
 
 
 def test_attention_bf16_layout_bhsd_and_non_causal(ctx):
