@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256, 2) void fa_bwd_dkv32_kernel(AttnArgs a) {
     for (int pass = 0; pass < 2; pass++) {
         const int kb = pass == 0 ? pair : n_qt - 1 - pair;
         if (pass == 1 && kb <= pair) break;  // odd block count: the middle block has no mirror
-        const int k0 = kb * 32, key = k0 + c;
+        const int k0 = kb * 32;
         if (pass == 0) load_kv(kb);  // the second pass's rows were requested before the first pass's reduction
         f32x16 dk[DT], dv[DT];
 #pragma unroll
