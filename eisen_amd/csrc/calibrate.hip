@@ -91,6 +91,9 @@ __global__ __launch_bounds__(256, 2) void tile_model_kernel(int iters, const cha
     // 16 tiles of 8 KB per wave; the blocks of an XCD share one 512 KB set
     const char* gbase = gsrc + (size_t)((blockIdx.x % 8) * 4 + wave) * 16 * 8192;
     const unsigned loff = lane * 16;
+    f32x16 s, dp;
+#pragma unroll
+    for (int v = 0; v < 16; v++) { s[v] = -3.f - 0.01f * v; dp[v] = 0.5f; }
     if (PARTS & 8) {
 #pragma unroll
         for (int r = 0; r < 8; r++) load_lds_16(gbase, loff + r * 1024, ring + r * 1024);
@@ -100,7 +103,6 @@ __global__ __launch_bounds__(256, 2) void tile_model_kernel(int iters, const cha
         if (PARTS & 8) wait_direct_loads();
 #pragma unroll
         for (int j = 0; j < 4; j++) asm volatile("" : "+v"(kf[j]), "+v"(vn[j]));  // nothing is hoisted out of the loop
-        f32x16 s, dp;
         if (PARTS & 4) {
             const float* st = reinterpret_cast<const float*>(stage + 8192);
 #pragma unroll
@@ -110,11 +112,7 @@ __global__ __launch_bounds__(256, 2) void tile_model_kernel(int iters, const cha
                 s[4 * vg] = l4.x; s[4 * vg + 1] = l4.y; s[4 * vg + 2] = l4.z; s[4 * vg + 3] = l4.w;
                 dp[4 * vg] = d4.x; dp[4 * vg + 1] = d4.y; dp[4 * vg + 2] = d4.z; dp[4 * vg + 3] = d4.w;
             }
-        } else {
-#pragma unroll
-            for (int v = 0; v < 16; v++) { s[v] = -3.f - 0.01f * v; dp[v] = 0.5f; }
-            asm volatile("" : "+v"(s), "+v"(dp));
-        }
+        }  // without the LDS reads the two score accumulators keep running: no start values to set up, nothing but the MFMAs
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
             bf16x8 qa = kf[(ks + 1) & 3], da = vn[(ks + 1) & 3];
