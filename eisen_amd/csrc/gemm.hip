@@ -268,12 +268,27 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-    // this lane's chunk of each of its wave's loads (the same for every slab)
+    // this lane's chunk of each of its wave's loads (the same for every slab), as a byte offset from the slab's origin for
+    // the leading dimensions in force; a segment of the contraction with other leading dimensions recomputes them
     int a_row[TA::LOADS], a_chunk[TA::LOADS], b_row[TB::LOADS], b_chunk[TB::LOADS];
+    unsigned a_off[TA::LOADS], b_off[TB::LOADS];
 #pragma unroll
     for (int i = 0; i < TA::LOADS; i++) TA::lane_chunk(i, wave, lane, a_row[i], a_chunk[i]);
 #pragma unroll
     for (int i = 0; i < TB::LOADS; i++) TB::lane_chunk(i, wave, lane, b_row[i], b_chunk[i]);
+    int off_lda = -1, off_ldb = -1;
+    auto set_offsets = [&](int lda, int ldb) {
+        if (lda != off_lda) {
+#pragma unroll
+            for (int i = 0; i < TA::LOADS; i++) a_off[i] = (unsigned)(a_row[i] * lda + a_chunk[i] * 8) * 2u;
+            off_lda = lda;
+        }
+        if (ldb != off_ldb) {
+#pragma unroll
+            for (int i = 0; i < TB::LOADS; i++) b_off[i] = (unsigned)(b_row[i] * ldb + b_chunk[i] * 8) * 2u;
+            off_ldb = ldb;
+        }
+    };
 
     // Where a slab's loads come from and go to (uniform values): the slab's K segment is picked with scalar selects.
     struct SlabSource {
@@ -299,6 +314,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
         src.b0 = B_KC ? Bp + (long long)n0 * ldb + k0 : Bp + (long long)k0 * ldb + n0;
         src.lda = lda;
         src.ldb = ldb;
+        set_offsets(lda, ldb);  // (uniform; changes only where a segment with other leading dimensions begins)
         src.As = lds[stage];
         src.Bs = lds[stage] + TA::ELEMS;
         return src;
@@ -308,8 +324,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_direct_kernel(GemmAr
         constexpr int h_lo = decltype(h_lo_c)::value, h_hi = decltype(h_hi_c)::value;
 #pragma unroll
         for (int h = h_lo; h < h_hi; h++) {
-            if (h < TA::LOADS) load_to_lds_16(src.a0 + (long long)a_row[h] * src.lda + a_chunk[h] * 8, src.As + TA::lds_block(h, wave));
-            else load_to_lds_16(src.b0 + (long long)b_row[h - TA::LOADS] * src.ldb + b_chunk[h - TA::LOADS] * 8, src.Bs + TB::lds_block(h - TA::LOADS, wave));
+            if (h < TA::LOADS) load_to_lds_16(src.a0, a_off[h], src.As + TA::lds_block(h, wave));
+            else load_to_lds_16(src.b0, b_off[h - TA::LOADS], src.Bs + TB::lds_block(h - TA::LOADS, wave));
         }
     };
     using I0 = std::integral_constant<int, 0>;
@@ -839,11 +855,14 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
             while (split < 32 && tiles * split * 2 <= 256 && K / (split * 2) >= min_part && K % (split * 2 * slab) == 0) split *= 2;
     }
     const bool split128 = split > 1 && M >= 128 && N >= 128;
+    // the direct-to-LDS kernels address a slab by a scalar base and a 32-bit byte offset per lane (up to 256 rows of a leading dimension)
+    bool ld_small = g.lda < (1 << 22) && g.ldb < (1 << 22);
+    for (int i = 0; i + 1 < g.nseg; i++) ld_small = ld_small && g.lda_seg[i] < (1 << 22) && g.ldb_seg[i] < (1 << 22);
     // 256x128 tiles only when they fill whole rounds of the 256 CUs well (one workgroup per CU)
     const long long wide_tiles = (long long)(M / 256) * (N / 128) * batch;
-    const bool wide = mfma_ok && split == 1 && big_tile && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && wide_tiles >= 256 &&
+    const bool wide = mfma_ok && ld_small && split == 1 && big_tile && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 && wide_tiles >= 256 &&
                       (double)wide_tiles / (double)(256 * ((wide_tiles + 255) / 256)) >= 0.85;
-    const bool wide32 = mfma_ok && split == 1 && n_more == 0 && !a_kc && !b_kc && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 &&
+    const bool wide32 = mfma_ok && ld_small && split == 1 && n_more == 0 && !a_kc && !b_kc && M % 256 == 0 && N % 128 == 0 && K % 64 == 0 &&
                         (wide_tiles >= 512 || (wide_tiles >= 300 && !wide));
     // 256 x 256 tiles (the gate/up kernel's main loop: an A operand register feeds twice the MFMAs) where the grid still
     // has three rounds of them: the lm_head forward (1035 against 980 TFLOP/s at 4096 x 32000 x 2048)
@@ -919,7 +938,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         } else if (big_tile || split128) {
             // whole tiles: the direct-to-LDS kernel (one workgroup per CU) is up to 16 % ahead when the grid has at most
             // one tile per CU and level with the register-staged kernel (two workgroups per CU) beyond that
-            const bool whole = M % 128 == 0 && N % 128 == 0 && K % 64 == 0 && (split == 1 || g.k_part % 64 == 0);
+            const bool whole = ld_small && M % 128 == 0 && N % 128 == 0 && K % 64 == 0 && (split == 1 || g.k_part % 64 == 0);
             // both operands through the transposing LDS reads and at least two tiles per CU: slabs of 32 let three
             // workgroups share a CU (down-projection dW 20 % faster)
             if (whole && !a_kc && !b_kc && tiles128 * split >= 512) launch_mfma_direct<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
@@ -1042,11 +1061,12 @@ extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* cons
     EISEN_REQUIRE(ctx, n >= 1 && n <= (size_t)kMaxGroup && A && B && C && N, EISEN_E_ARG, "eisen_hip_gemm_grouped: 1 to 8 products, no null pointers");
     // One launch when every product is a whole number of 128x128 tiles of the dW form (bf16 operands stored [K][M] and
     // [K][N], f32 result) and together they give every CU at least two tiles; otherwise one launch per product.
+    // (leading dimensions below 2^22: the direct-to-LDS kernels address a slab by a scalar base and a 32-bit byte offset per lane)
     bool grouped = n >= 2 && dtype_ab == EISEN_BF16 && dtype_c == EISEN_F32 && trans_a && !trans_b && M % 128 == 0 && K % 64 == 0 && K > 0 &&
-                   M < (size_t(1) << 30) && K < (size_t(1) << 30);
+                   M < (size_t(1) << 22) && K < (size_t(1) << 30);
     long long tiles = 0;
     for (size_t p = 0; p < n && grouped; p++) {
-        grouped = A[p] && B[p] && C[p] && N[p] > 0 && N[p] % 128 == 0 && N[p] < (size_t(1) << 30) && eisen_aligned(A[p], 16) && eisen_aligned(B[p], 16) &&
+        grouped = A[p] && B[p] && C[p] && N[p] > 0 && N[p] % 128 == 0 && N[p] < (size_t(1) << 22) && eisen_aligned(A[p], 16) && eisen_aligned(B[p], 16) &&
                   eisen_aligned(C[p], 16);
         tiles += (long long)(M / 128) * (long long)(N[p] / 128);
     }
@@ -1108,11 +1128,11 @@ extern "C" int eisen_hip_gemm_grouped(eisen_ctx* ctx, size_t n, const void* cons
     // tokens): one launch of 64 x 64 tiles over every product and every part of a split contraction, then one launch
     // that adds each product's partial results in part order.  Instead of a GEMM and a reduction per product.
     bool small = n >= 2 && dtype_ab == EISEN_BF16 && dtype_c == EISEN_F32 && trans_a && !trans_b && M % 64 == 0 && K % 32 == 0 && K >= 1024 &&
-                 M < (size_t(1) << 30) && K < (size_t(1) << 30);
+                 M < (size_t(1) << 22) && K < (size_t(1) << 30);
     long long tiles64 = 0, out_elems = 0;
     size_t max_n = 0;
     for (size_t p = 0; p < n && small; p++) {
-        small = A[p] && B[p] && C[p] && N[p] > 0 && N[p] % 64 == 0 && N[p] < (size_t(1) << 30) && eisen_aligned(A[p], 16) && eisen_aligned(B[p], 16) &&
+        small = A[p] && B[p] && C[p] && N[p] > 0 && N[p] % 64 == 0 && N[p] < (size_t(1) << 22) && eisen_aligned(A[p], 16) && eisen_aligned(B[p], 16) &&
                 eisen_aligned(C[p], 16);
         tiles64 += (long long)(M / 64) * (long long)(N[p] / 64);
         out_elems += (long long)M * (long long)N[p];

@@ -360,6 +360,12 @@ __device__ __forceinline__ void load_to_lds_16(const void* src, bf16_t* lds_dst)
     const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
 }
+// the same with a wave-uniform 64-bit base and a 32-bit byte offset per lane (below 2 GiB): the base is two scalar
+// registers and the offset does not change from slab to slab, so a load costs no vector arithmetic
+__device__ __forceinline__ void load_to_lds_16(const void* base, unsigned lane_offset, bf16_t* lds_dst) {
+    const unsigned lds_addr = (unsigned)(size_t)(lds_void_ptr)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_offset), "s"(base) : "m0");
+}
 template <int N>
 __device__ __forceinline__ void wait_loads_but() {  // until at most N of this wave's vector memory loads are outstanding
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
