@@ -463,25 +463,37 @@ __global__ __launch_bounds__(512) void gemm_swiglu_forward_kernel(SwigluForwardA
 #pragma unroll
             for (int v = 0; v < 16; v++) { accg[i][j][v] = 0.f; accu[i][j][v] = 0.f; }
 
-    int a_row[TA::LOADS], a_chunk[TA::LOADS], b_row[TB::LOADS], b_chunk[TB::LOADS];
+    // this lane's chunk of each of its wave's loads, as a byte offset from the slab's origin (the same for every slab: a load
+    // takes the slab's origin in scalar registers and this offset, no vector arithmetic)
+    unsigned a_off[TA::LOADS], b_off[TB::LOADS];
 #pragma unroll
-    for (int i = 0; i < TA::LOADS; i++) TA::lane_chunk(i, wave, lane, a_row[i], a_chunk[i]);
+    for (int i = 0; i < TA::LOADS; i++) {
+        int row, chunk;
+        TA::lane_chunk(i, wave, lane, row, chunk);
+        a_off[i] = (unsigned)(row * g.K + chunk * 8) * 2u;
+    }
 #pragma unroll
-    for (int i = 0; i < TB::LOADS; i++) TB::lane_chunk(i, wave, lane, b_row[i], b_chunk[i]);
+    for (int i = 0; i < TB::LOADS; i++) {
+        int row, chunk;
+        TB::lane_chunk(i, wave, lane, row, chunk);
+        b_off[i] = (unsigned)(row * g.N + chunk * 8) * 2u;
+    }
     // loads h_lo..h_hi-1 of the NLOADS this wave issues per slab: X rows, then the Wg and Wu slabs
     auto issue = [&](int slab, int stage, auto h_lo_c, auto h_hi_c) {
         constexpr int h_lo = decltype(h_lo_c)::value, h_hi = decltype(h_hi_c)::value;
         const int k0 = slab * BK;
         bf16_t* st = lds[stage];
+        const bf16_t* x0 = g.X + (long long)m0 * g.K + k0;
+        const long long w_origin = (long long)k0 * g.N + n0;
 #pragma unroll
         for (int h = h_lo; h < h_hi; h++) {
             if (h < TA::LOADS) {
-                load_to_lds_16(g.X + (long long)(m0 + a_row[h]) * g.K + k0 + a_chunk[h] * 8, st + TA::lds_block(h, wave));
+                load_to_lds_16(x0, a_off[h], st + TA::lds_block(h, wave));
             } else {
                 const int hb = (h - TA::LOADS) % TB::LOADS;
                 const bool second = h - TA::LOADS >= TB::LOADS;
                 const bf16_t* W = second ? g.Wu : g.Wg;
-                load_to_lds_16(W + (long long)(k0 + b_row[hb]) * g.N + n0 + b_chunk[hb] * 8, st + TA::ELEMS + (second ? TB::ELEMS : 0) + TB::lds_block(hb, wave));
+                load_to_lds_16(W + w_origin, b_off[hb], st + TA::ELEMS + (second ? TB::ELEMS : 0) + TB::lds_block(hb, wave));
             }
         }
     };
@@ -884,7 +896,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         g.rope_head_dim = (int)rope->head_dim;
         g.rope_members = (int)std::min<size_t>(rope->members, batch);
     }
-    const bool wide256 = mfma_ok && split == 1 && n_more == 0 && a_kc && !b_kc && batch == 1 && dtype_c == EISEN_BF16 && !residual && !swiglu && !rope &&
+    const bool wide256 = mfma_ok && ld_small && split == 1 && n_more == 0 && a_kc && !b_kc && batch == 1 && dtype_c == EISEN_BF16 && !residual && !swiglu && !rope &&
                          !accumulate && M % 256 == 0 && N % 256 == 0 && K % 32 == 0 && (M / 256) * (N / 256) >= 768 && eisen_aligned(C, 16);
     if (wide256) {
         SwigluForwardArgs a{static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(B), static_cast<const bf16_t*>(B) + 128, static_cast<bf16_t*>(C),
@@ -1039,7 +1051,7 @@ extern "C" int eisen_hip_gemm_swiglu_forward(eisen_ctx* ctx, const void* X, cons
     EISEN_REQUIRE(ctx, eisen_dtype_ok(dtype), EISEN_E_ARG, "eisen_hip_gemm_swiglu_forward: unknown dtype %d", dtype);
     if (M * N == 0) return 0;
     const bool fused = dtype == EISEN_BF16 && M % 256 == 0 && N % 128 == 0 && K % 32 == 0 && K >= 32 && (M / 256) * (N / 128) >= 256 &&
-                       M / 256 <= 65535 && M < (size_t(1) << 30) && N < (size_t(1) << 30) && K < (size_t(1) << 30) && eisen_aligned(X, 16) && eisen_aligned(Wg, 16) &&
+                       M / 256 <= 65535 && M < (size_t(1) << 30) && N < (size_t(1) << 22) && K < (size_t(1) << 22) && eisen_aligned(X, 16) && eisen_aligned(Wg, 16) &&
                        eisen_aligned(Wu, 16) && eisen_aligned(G, 16) && eisen_aligned(U, 16) && eisen_aligned(H, 16);
     if (fused) {
         SwigluForwardArgs a{static_cast<const bf16_t*>(X), static_cast<const bf16_t*>(Wg), static_cast<const bf16_t*>(Wu), static_cast<bf16_t*>(G),
