@@ -112,7 +112,8 @@ def mfma_ceiling(ctx):
     """What this GPU sustains on nothing but bf16 MFMAs, measured now, next to the published peak the fractions use:
     operands in registers, and re-read from LDS at the ratio of a 128x128 and of a 64x64 wave tile."""
     return dict(unit="TFLOP/s", registers_only=round(ctx.mfma_ceiling(0), 1), lds_fed_128x128_wave_tile=round(ctx.mfma_ceiling(8), 1),
-                lds_fed_64x64_wave_tile=round(ctx.mfma_ceiling(16), 1))
+                lds_fed_64x64_wave_tile=round(ctx.mfma_ceiling(16), 1), lds_fed_24_reads_per_16_mfma=round(ctx.mfma_ceiling(24), 1),
+                lds_fed_32_reads_per_16_mfma=round(ctx.mfma_ceiling(32), 1))
 
 
 def pick_dominant(prof, workload):

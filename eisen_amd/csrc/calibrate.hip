@@ -11,7 +11,9 @@ namespace {
 
 // Each wave: four independent 32x32 accumulators (a 64x64 wave tile), 16 MFMAs per iteration = four contraction steps.
 // READS: 16-byte LDS operand reads (1 KB per wave instruction) per 16 MFMAs: 0 = operands stay in registers; 16 = the
-// 64x64 wave tile of the 8-wave GEMM kernels (two A and two B reads per step); 8 = the ratio of a 128x128 wave tile.
+// 64x64 wave tile of the 8-wave GEMM kernels (two A and two B reads per step); 8 = the ratio of a 128x128 wave tile;
+// 24 and 32 = more than any kernel here issues in 16-byte reads (a 64x64 wave tile whose second operand comes through
+// 8-byte transposing reads issues 24 read instructions for the same bytes): where the LDS starts to hold the MFMAs back.
 template <int READS>
 __global__ __launch_bounds__(512) void mfma_ceiling_kernel(int iters, float* sink) {
     __shared__ __attribute__((aligned(16))) bf16_t tile[16 * 512];  // 16 operand reads' worth of chunks
@@ -36,13 +38,14 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(int iters, float* sin
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             if (READS > 0) {
-                constexpr int PER_STEP = READS / 4;  // 4 or 2
+                constexpr int PER_STEP = READS / 4;  // 2, 4, 6 or 8
                 const int base = ((it * 4 + s) * PER_STEP) & 15;
 #pragma unroll
                 for (int r = 0; r < PER_STEP; r++) {
                     const bf16x8 x = src[((base + r) & 15) * 64];
                     if (r & 1) b[(s + (r >> 1)) & 3] = x;
                     else a[(s + (r >> 1)) & 3] = x;
+                    if (r >= 4) asm volatile("" ::"v"(x));  // (a read whose value a later read of the step overwrites is still made)
                 }
             }
             acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s], b[s], acc[0], 0, 0, 0);
@@ -190,8 +193,8 @@ __global__ __launch_bounds__(256, 2) void tile_model_kernel(int iters, const cha
 extern "C" int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma, int iters, double* tflops_out) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, tflops_out != nullptr, EISEN_E_ARG, "mfma_ceiling: tflops_out is null");
-    EISEN_REQUIRE(ctx, lds_reads_per_16_mfma == 0 || lds_reads_per_16_mfma == 8 || lds_reads_per_16_mfma == 16, EISEN_E_ARG,
-                  "mfma_ceiling: lds_reads_per_16_mfma must be 0, 8 or 16, got %d", lds_reads_per_16_mfma);
+    EISEN_REQUIRE(ctx, lds_reads_per_16_mfma == 0 || lds_reads_per_16_mfma == 8 || lds_reads_per_16_mfma == 16 || lds_reads_per_16_mfma == 24 || lds_reads_per_16_mfma == 32, EISEN_E_ARG,
+                  "mfma_ceiling: lds_reads_per_16_mfma must be 0, 8, 16, 24 or 32, got %d", lds_reads_per_16_mfma);
     EISEN_REQUIRE(ctx, iters > 0 && iters <= (1 << 20), EISEN_E_ARG, "mfma_ceiling: iters %d outside (0, 2^20]", iters);
     hipDeviceProp_t prop;
     EISEN_HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
@@ -205,7 +208,9 @@ extern "C" int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma,
     auto launch = [&](int n) {
         if (lds_reads_per_16_mfma == 0) mfma_ceiling_kernel<0><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
         else if (lds_reads_per_16_mfma == 8) mfma_ceiling_kernel<8><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
-        else mfma_ceiling_kernel<16><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
+        else if (lds_reads_per_16_mfma == 16) mfma_ceiling_kernel<16><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
+        else if (lds_reads_per_16_mfma == 24) mfma_ceiling_kernel<24><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
+        else mfma_ceiling_kernel<32><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
     };
     launch(iters);  // warm-up: clocks and code object
     hipError_t err = hipEventRecord(e0, ctx->stream);

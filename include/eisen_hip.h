@@ -131,7 +131,8 @@ int eisen_hip_profile_stop(eisen_ctx* ctx, eisen_prof_entry* out, size_t capacit
  * instructions): runs a kernel of nothing but v_mfma_f32_32x32x16_bf16 on every CU (two waves per SIMD, four independent
  * 32x32 accumulators per wave, `iters` x 16 MFMAs per wave), once untimed and once between two events on the context's
  * stream, and returns the achieved TFLOP/s.  lds_reads_per_16_mfma = 0: operands stay in registers; 16: every contraction
- * step re-reads two A and two B operands from LDS (the ratio of a 64x64 wave tile); 8: the ratio of a 128x128 wave tile.
+ * step re-reads two A and two B operands from LDS (the ratio of a 64x64 wave tile); 8: the ratio of a 128x128 wave tile;
+ * 24, 32: one and a half times and twice the reads of a 64x64 wave tile (where the LDS begins to hold the MFMAs back).
  * Synchronises the stream. */
 int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma, int iters, double* tflops_out);
 
