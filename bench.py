@@ -43,7 +43,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # `symbol_of` names it; the summaries (command, calibration factors, per-kernel rows) are the files named here.
 TRAFFIC_SOURCE = {"c5": "profiles/c5_step_hbm_traffic_pmc.md", "c4": "profiles/c4_step_hbm_traffic_pmc.md", "c3": "profiles/c2_c3_hbm_traffic_pmc.md", "c2": "profiles/c2_c3_hbm_traffic_pmc.md"}
 MEASURED_TRAFFIC = {
-    "c5": {"gemm_tn_bf16_f32out_256x256x32_window": 24423.6e6, "gemm_tn_bf16_f32out_256x256x32": 902.8e6, "gemm_nt_bf16_bf16out_256x128x64": 213.4e6},
+    "c5": {"gemm_tn_bf16_f32out_256x256x32_window": 18263.6e6, "gemm_tn_bf16_f32out_256x256x32": 902.8e6, "gemm_nt_bf16_bf16out_256x128x64": 213.4e6},
     "c4": {"gemm_tn_bf16_f32out_128x128x64_splitk": 57.7e6, "gemm_nt_bf16_bf16out_128x128x64": 35.7e6, "gemm_nt_bf16_bf16out_256x128x64_swiglu_bwd": 101.4e6,
            "gemm_tn_bf16_f32out_64x64x32_grouped_splitk": 40.1e6, "gemm_nn_bf16_bf16out_128x128x64_splitk": 54.2e6, "gemm_nn_bf16_swiglu_256x128x32": 85.1e6},
     "c3": {"attn_bwd": 78.7e6 + 52.4e6},
@@ -178,11 +178,13 @@ def cpu_baseline_lm(c, seq, mb=1):
 # workloads
 # ---------------------------------------------------------------------------------------------
 
-def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True, beside=True):
+def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True, beside=True, meet_us=None):
     from eisen_amd import graph as G
     from eisen_amd import hip
     c = CONFIGS[name]
     ctx = hip.Context(0)
+    if meet_us is not None:   # A/B of the windowed weight-gradient GEMM's meeting points (library default: 40 us; 0 = none)
+        ctx.gemm_window_meet(meet_us)
     g = G.Graph(ctx, G.BF16_MIXED)
     lm = G.TransformerLM(g, **arch(c))
     rng = np.random.default_rng(1234)
@@ -482,6 +484,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
     ap.add_argument("--no-window", action="store_true", help="c5: form every micro-batch's weight gradients in its own backward pass, as the reference does, "
                     "instead of once per optimizer step over the whole accumulation window")
+    ap.add_argument("--window-meet-us", type=int, default=None, help="c5: longest wait at the meeting points of the windowed weight-gradient GEMM "
+                    "(library default 40; 0 switches them off)")
     ap.add_argument("--no-beside", action="store_true", help="c4: keep the weight-gradient GEMMs of narrow layers on the main stream, in tape order")
     ap.add_argument("--recompute", action="store_true", help="c5 / c4: per-block recompute (lower activation memory, one more forward pass per block)")
     args = ap.parse_args()
@@ -490,7 +494,7 @@ def main():
         sys.exit(2)
     w = args.workload
     if w in ("all", "c5"):
-        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside)
+        out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside, args.window_meet_us)
         if w == "all":
             out["other_configs"] = dict(c4=brief(bench_lm("c4", 20, 3, not args.no_cpu)), c3=brief(bench_c3(20, 3)), c2=brief(bench_c2(20, 3)))
             if not args.no_window:   # the same step in the reference's accumulation order: every pass forms and adds its own dW

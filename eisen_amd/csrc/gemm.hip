@@ -1240,12 +1240,22 @@ extern "C" int eisen_hip_gemm_grouped_ksegments(eisen_ctx* ctx, size_t n_product
         // fewer tiles than CUs would leave most of the chip idle for the whole contraction
         one = one && tiles >= 176 && eisen_gemm_wide_window_supports(w, rows.data());
         if (one) {
+            // the table, and behind it the (zeroed) counters of the meeting points: one per XCD and 32 tiles of its range
+            const int meet_us = ctx->window_meet_us;
+            const size_t ngrp = (size_t)((tiles / 8 + 31) / 32);
+            const size_t table_bytes = rows.size() * sizeof(WideWindowRow), meet_bytes = meet_us > 0 ? 8 * ngrp * sizeof(int) : 0;
+            std::vector<char> host(table_bytes + meet_bytes, 0);
+            memcpy(host.data(), rows.data(), table_bytes);
             void* table = nullptr;
-            int rc = eisen_hip_malloc(ctx, rows.size() * sizeof(WideWindowRow), &table);
+            int rc = eisen_hip_malloc(ctx, host.size(), &table);
             if (rc) return rc;
-            rc = eisen_hip_htod(ctx, table, rows.data(), rows.size() * sizeof(WideWindowRow));
+            rc = eisen_hip_htod(ctx, table, host.data(), host.size());
             if (!rc) {
                 w.rows = static_cast<const WideWindowRow*>(table);
+                if (meet_us > 0) {
+                    w.meet = reinterpret_cast<int*>(static_cast<char*>(table) + table_bytes);
+                    w.meet_ticks = meet_us * 100;
+                }
                 EisenProfScope prof(ctx, "gemm_tn_bf16_f32out_256x256x32_window", flops, true);
                 eisen_gemm_launch_wide_window(ctx, w, (unsigned)tiles);
             }
@@ -1262,6 +1272,13 @@ extern "C" int eisen_hip_gemm_grouped_ksegments(eisen_ctx* ctx, size_t n_product
                                        s == 0 ? accumulate : 1, "eisen_hip_gemm_grouped_ksegments");
             if (rc) return rc;
         }
+    return 0;
+}
+
+extern "C" int eisen_hip_gemm_window_meet(eisen_ctx* ctx, int microseconds) {
+    EISEN_CHECK_CTX(ctx);
+    EISEN_REQUIRE(ctx, microseconds >= 0 && microseconds <= 1000, EISEN_E_ARG, "eisen_hip_gemm_window_meet: %d us outside [0, 1000]", microseconds);
+    ctx->window_meet_us = microseconds;
     return 0;
 }
 

@@ -71,6 +71,12 @@ struct WideWindow {
     int seg_slabs;  // 32-deep slabs per piece, a multiple of 4
     int accumulate;
     const WideWindowRow* rows;  // device memory, nprod entries
+    // Optional meeting point for the workgroups an XCD runs at one time (null: none).  One counter per XCD and group of 32
+    // consecutive tiles of its range, zero at launch.  A workgroup counts itself in and waits until its group is complete or
+    // `meet_ticks` of the 100 MHz clock have passed, whichever comes first: the wait only keeps the group's tiles close enough
+    // in time to share their operand panels in the L2, and no result depends on it.
+    int* meet;
+    int meet_ticks;
 };
 // the host's copy of the table: shapes the kernel takes?
 bool eisen_gemm_wide_window_supports(const WideWindow& w, const WideWindowRow* host_rows);

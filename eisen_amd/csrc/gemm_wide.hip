@@ -107,6 +107,21 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, std::conditi
         }
     }
     const int m0 = mt * WBM, n0 = nt * WBN;
+    if constexpr (WIN) {
+        const int per = gridDim.x / 8;
+        if (w.meet != nullptr && (int)blockIdx.x < per * 8) {
+            if (tid == 0) {
+                const int local = blockIdx.x / 8, grp = local / 32, ngrp = (per + 31) / 32;
+                const int expect = min(32, per - grp * 32);
+                int* c = w.meet + (blockIdx.x % 8) * ngrp + grp;
+                __hip_atomic_fetch_add(c, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const long long t0 = wall_clock64();
+                while (__hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < expect && wall_clock64() - t0 < w.meet_ticks)
+                    __builtin_amdgcn_s_sleep(16);
+            }
+            __syncthreads();
+        }
+    }
     const bf16_t* A = static_cast<const bf16_t*>(g.A);
     const bf16_t* B = static_cast<const bf16_t*>(g.B);
     TC* C = static_cast<TC*>(g.C);

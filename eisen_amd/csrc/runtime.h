@@ -69,6 +69,7 @@ struct eisen_ctx {
     int attn_ablation = 0;  // measurement only: the part of the attention backward kernels' tile loop to leave out (0 = none)
     long long* attn_stamps = nullptr;  // measurement only: where the attention kernels drop time stamps (eisen_hip_attention_timeline)
     int attn_stamp_waves = 0;
+    int window_meet_us = 40;  // longest wait at a meeting point of the windowed weight-gradient GEMM (eisen_hip_gemm_window_meet); 0 = none
     eisen_prof prof;
     char last_error[512] = {0};
 };

@@ -359,6 +359,10 @@ class Context:
         self._call("eisen_hip_gemm_swiglu_backward", _ptr(A), _ptr(B), _ptr(gate), _ptr(up), _ptr(dgate), _ptr(dup), _i(dtype), _i(trans_a), _i(trans_b),
                    _sz(M), _sz(N), _sz(K))
 
+    def gemm_window_meet(self, microseconds):
+        """Longest wait at the meeting points of gemm_grouped_ksegments' one-launch form (0 = no meeting points)."""
+        self._call("eisen_hip_gemm_window_meet", _i(microseconds))
+
     def gemm_ksegments(self, As, Bs, Ks, Cbuf, dtype_ab, dtype_c, trans_a, trans_b, M, N, accumulate=0):
         """C (+)= sum_s op(A_s) op(B_s) over up to three (A, B, K) segments."""
         n = len(Ks)

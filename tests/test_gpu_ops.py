@@ -930,6 +930,37 @@ def test_gemm_grouped_ksegments_weight_gradients_over_micro_batches(ctx, shapes,
         x.free()
 
 
+def test_gemm_window_meeting_points_change_no_bit(ctx):
+    # 352 tiles of 256x256 = 44 per XCD: a full group of 32 and a group of 12 on every XCD.  The wait at a group's meeting point
+    # is bounded (40 us by default; 1 us here makes every early workgroup give up waiting) and must not show in the results.
+    shapes, seg_k, nseg = ((2048, 5632), (2048, 5632)), 128, 2
+    xs = [[_rand_bf16(1200 + 16 * p + s, (seg_k, m), 0.5) for s in range(nseg)] for p, (m, n) in enumerate(shapes)]
+    dys = [[_rand_bf16(1300 + 16 * p + s, (seg_k, n), 0.5) for s in range(nseg)] for p, (m, n) in enumerate(shapes)]
+    dA = [[up(ctx, x, BF16) for x in row] for row in xs]
+    dB = [[up(ctx, d, BF16) for d in row] for row in dys]
+    Ms, Ns = [m for m, n in shapes], [n for m, n in shapes]
+    results = []
+    try:
+        for us in (40, 0, 1):
+            ctx.gemm_window_meet(us)
+            dC = [up(ctx, np.zeros(sh, np.float32), F32) for sh in shapes]
+            ctx.gemm_grouped_ksegments(dA, dB, dC, Ms, Ns, seg_k, 0)
+            results.append([dn(ctx, dC[p], shapes[p], F32) for p in range(len(shapes))])
+            for c in dC:
+                c.free()
+    finally:
+        ctx.gemm_window_meet(40)
+    for p, (m, n) in enumerate(shapes):
+        exp = sum(xs[p][s].astype(np.float64).T @ dys[p][s].astype(np.float64) for s in range(nseg))
+        assert_close(results[0][p], exp, 1e-3, f"product {p}")
+        assert np.array_equal(results[0][p], results[1][p]), f"product {p}: meeting points changed the result"
+        assert np.array_equal(results[0][p], results[2][p]), f"product {p}: a timed-out meeting point changed the result"
+    with pytest.raises(hip.EisenHipError):
+        ctx.gemm_window_meet(-1)
+    for x in [t for row in dA + dB for t in row]:
+        x.free()
+
+
 def _rand_bf16(seed, shape, scale=1.0):
     """bf16-representable normal values, generated fast enough for the config-5 operand sizes."""
     return hip.round_bf16(np.random.default_rng(seed).standard_normal(shape, dtype=np.float32) * np.float32(scale))
