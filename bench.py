@@ -462,6 +462,14 @@ def bench_c3_timeline(steps, warmup):
     for label, parts in (("mfma", 1), ("mfma_valu", 3), ("mfma_valu_lds", 7), ("tile_loads", 8), ("all", 15)):
         for wps in (1, 2):
             model[f"{label}_{wps}_per_simd"] = round(ctx.attention_tile_model(parts, wps, 4000), 1)
+    # the tile loop of a one-pass backward (S and dP once, dQ partials per 128-key chunk), and the two kernels it would need around it
+    onepass = {}
+    for label, parts in (("tile_with_partial_stores", 16), ("tile_without_partial_stores", 32)):
+        onepass[f"{label}_ns_per_tile_and_simd"] = round(ctx.attention_tile_model(parts, 2, 4000), 1)
+    for chunk in (128, 256):
+        d_us, sum_us = ctx.attention_onepass_parts(8 * 16 * 1024, 1024, chunk)
+        onepass["rowdot_prepass_us"] = round(d_us, 2)
+        onepass[f"partial_sum_chunk{chunk}_us"] = round(sum_us, 2)
     ctx.close()
     names = ["attn_fwd_bf16", "attn_bwd_dq_bf16", "attn_bwd_dkv_bf16"]
     keys = ["waves", "entry_to_first_loop_us", "tile_loops_us", "first_block_stored_us", "to_second_loop_us", "second_block_stored_us",
@@ -469,7 +477,7 @@ def bench_c3_timeline(steps, warmup):
     return dict(metric="config-3 attention kernels: a wave's life by phase (in-kernel time stamps, mean over waves)", unit="us", steps=steps, warmup=warmup,
                 config=dict(workload="config3 causal GQA flash attention fwd+bwd, B8 S1024 Hq16 Hkv4 hd64, [B,H,S,hd]"),
                 rows=[dict(kernel=n, **{k_: round(float(x), 2) for k_, x in zip(keys, r)}) for n, r in zip(names, acc)],
-                dkv_tile_loop_model_ns_per_tile_and_simd=model)
+                dkv_tile_loop_model_ns_per_tile_and_simd=model, one_pass_model=onepass)
 
 
 def main():

@@ -402,10 +402,16 @@ class Context:
         self._call("eisen_hip_attention_timeline", _ptr(stamps), _sz(waves))
 
     def attention_tile_model(self, parts, waves_per_simd=2, iters=4000):
-        """Measurement only: ns per tile and SIMD of a model of the dK/dV kernel's tile loop (parts: 1 MFMA, 3 +VALU, 7 +LDS, 8 loads, 15 all)."""
+        """Measurement only: ns per tile and SIMD of a model of the dK/dV kernel's tile loop (parts: 1 MFMA, 3 +VALU, 7 +LDS, 8 loads, 15 all; 16 / 32 the one-pass tile with / without its dQ partial stores)."""
         out = C.c_double(0.0)
         self._call("eisen_hip_attention_tile_model", _i(parts), _i(waves_per_simd), _i(iters), C.byref(out))
         return out.value
+
+    def attention_onepass_parts(self, rows, seq, chunk):
+        """Measurement only: us of the D = rowsum(dO o O) pre-pass and of the ordered sum of causal dQ partials (key chunks of `chunk`)."""
+        a, b = C.c_double(0.0), C.c_double(0.0)
+        self._call("eisen_hip_attention_onepass_parts", _sz(rows), _i(seq), _i(chunk), C.byref(a), C.byref(b))
+        return a.value, b.value
 
     def attention_rope_backward(self, q, k, v, out, dout, lse, dq, dk, dv, dtype, B, S, Hq, Hkv, hd, scale, causal=True):
         """Backward for rotary-embedded q, k: dq, dk come out as gradients of the un-rotated projections."""

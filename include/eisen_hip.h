@@ -384,8 +384,18 @@ int eisen_hip_attention_timeline(eisen_ctx* ctx, long long* stamps, size_t waves
  * kernel at head_dim 64, built from the same instructions on made-up data, timed with any of its parts alone or together.
  * parts: 1 the sixteen MFMAs of a tile; 3 those and the vector work between them; 7 those and the tile's LDS reads; 8 only
  * the eight 1 KB direct-to-LDS loads that bring a wave's next tile (from a region that stays in the L2); 15 everything.
+ * parts 16: the tile loop a one-pass backward would have instead (score tile and dP computed once; the four waves of a
+ * workgroup own 128 keys, work on one 32-query tile at a time, share its Q / dO tile, exchange their dS tiles through LDS
+ * behind one barrier per tile and write a dQ partial of 8 KB per workgroup and tile); 32: the same without those writes.
  * waves_per_simd: 1 or 2 (the kernel runs two).  *ns_per_tile_out: time per tile and SIMD over `iters` tiles per wave. */
 int eisen_hip_attention_tile_model(eisen_ctx* ctx, int parts, int waves_per_simd, int iters, double* ns_per_tile_out);
+
+/* Measurement aid (no counterpart in the reference): the two small kernels that a one-pass attention backward would need
+ * around its main kernel, timed on made-up data at head_dim 64, to be set beside the one-pass tile model
+ * (eisen_hip_attention_tile_model, parts 16 / 32).  *rowdot_us_out: D = rowsum(dO o O) over `rows` bf16 rows of 64.
+ * *partial_sum_us_out: dQ as the sum, in a fixed order, of the f32 partials of the key chunks a causal query sees
+ * (position / chunk + 1 of them; rows = whole sequences of `seq`), stored as bf16.  Averages over 10 launches. */
+int eisen_hip_attention_onepass_parts(eisen_ctx* ctx, size_t rows, int seq, int chunk, double* rowdot_us_out, double* partial_sum_us_out);
 
 /* eisen_hip_attention_backward for q and k that are rotary-embedded projections, q = rope(q0), k = rope(k0)
  * (src/nn/attention.rs:316-317 applies `g.rope` to both before the attention chain): dq and dk receive the

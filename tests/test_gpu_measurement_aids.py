@@ -88,5 +88,12 @@ def test_tile_model_and_mfma_ceiling_report_sane_figures(ctx):
     assert everything >= 0.9 * mfma and 20.0 < loads < 2000.0, (mfma, everything, loads)
     with pytest.raises(EisenHipError):
         ctx.attention_tile_model(2, 2, 1000)
+    # the one-pass tile: 16 + 4 MFMAs' worth of matrix time, never less than 266 ns at the boost clock
+    one_pass = ctx.attention_tile_model(32, 2, 1000)
+    assert 266.0 <= one_pass < 3000.0 and ctx.attention_tile_model(16, 2, 1000) >= 0.9 * one_pass, one_pass
+    d_us, sum_us = ctx.attention_onepass_parts(4 * 1024, 1024, 128)
+    assert 0.5 < d_us < 500.0 and 0.5 < sum_us < 500.0, (d_us, sum_us)
+    with pytest.raises(EisenHipError):
+        ctx.attention_onepass_parts(1000, 1024, 128)
     ceiling = ctx.mfma_ceiling(0, 5000)
     assert 1250.0 < ceiling < 2500.0, ceiling
