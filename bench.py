@@ -113,7 +113,54 @@ def mfma_ceiling(ctx):
     operands in registers, and re-read from LDS at the ratio of a 128x128 and of a 64x64 wave tile."""
     return dict(unit="TFLOP/s", registers_only=round(ctx.mfma_ceiling(0), 1), lds_fed_128x128_wave_tile=round(ctx.mfma_ceiling(8), 1),
                 lds_fed_64x64_wave_tile=round(ctx.mfma_ceiling(16), 1), lds_fed_24_reads_per_16_mfma=round(ctx.mfma_ceiling(24), 1),
-                lds_fed_32_reads_per_16_mfma=round(ctx.mfma_ceiling(32), 1))
+                lds_fed_32_reads_per_16_mfma=round(ctx.mfma_ceiling(32), 1),
+                # the same loops on operands whose bits change from MFMA to MFMA (random sign, exponent, mantissa), as a layer's
+                # activations and gradients do: the clock the part holds under matrix load depends on the data
+                random_operands_registers_only=round(ctx.mfma_ceiling(0, random_operands=True), 1),
+                random_operands_lds_fed_128x128_wave_tile=round(ctx.mfma_ceiling(8, random_operands=True), 1),
+                random_operands_lds_fed_64x64_wave_tile=round(ctx.mfma_ceiling(16, random_operands=True), 1))
+
+
+def gemms_by_operand_data(ctx):
+    """The step's GEMM kernels alone on the GPU at config-5 shapes, once on all-zero operands and once on N(0,1) operands (the same
+    code objects; only the bits of the data differ).  The clock this GPU holds under matrix load depends on the operands, so the
+    zero-operand figure is what a kernel's structure allows and the other what the part's power management then leaves of it."""
+    from eisen_amd import hip
+    BF16 = hip.BF16
+    rng = np.random.default_rng(7)
+    M = 4096
+    wm, wn, nprod, nseg = 2048, 5632, 32, 8
+    Cs = [ctx.malloc(wm * wn * 4) for _ in range(nprod)]
+    c2, G, U, H = (ctx.malloc(M * cols * 2) for cols in (2048, 5632, 5632, 5632))
+    out = dict(unit="TFLOP/s")
+
+    def rate(fn, flop, reps):
+        for _ in range(2):
+            fn()
+        ctx.sync()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        ctx.sync()
+        return round(flop * reps / (time.perf_counter() - t0) / 1e12, 1)
+
+    for label in ("zero_operands", "normal_operands"):
+        mk = (lambda shape: np.zeros(shape, np.float32)) if label == "zero_operands" else (lambda shape: hip.round_bf16(rng.standard_normal(shape, dtype=np.float32)))
+        x2, x5 = ctx.upload(mk((M, 2048)), BF16), ctx.upload(mk((M, 5632)), BF16)
+        w22, w52, wg, wu = (ctx.upload(mk(sh), BF16) for sh in ((2048, 2048), (5632, 2048), (2048, 5632), (2048, 5632)))
+        A, B = [[x2] * nseg] * nprod, [[x5] * nseg] * nprod
+        out[label] = {
+            "gemm_tn_bf16_f32out_256x256x32_window, 32 x [2048 x 5632] over 8 x 4096 rows":
+                rate(lambda: ctx.gemm_grouped_ksegments(A, B, Cs, [wm] * nprod, [wn] * nprod, M, 0), 2.0 * wm * wn * M * nseg * nprod, 2),
+            "gemm_nn_bf16_bf16out_256x128x64, 4096 x 2048 x 5632": rate(lambda: ctx.gemm(x5, w52, c2, BF16, BF16, 0, 0, M, 2048, 5632), 2.0 * M * 2048 * 5632, 30),
+            "gemm_nt_bf16_bf16out_256x128x64, 4096 x 2048 x 2048": rate(lambda: ctx.gemm(x2, w22, c2, BF16, BF16, 0, 1, M, 2048, 2048), 2.0 * M * 2048 * 2048, 30),
+            "gemm_nn_bf16_swiglu_fwd, 4096 x (5632 + 5632) x 2048": rate(lambda: ctx.gemm_swiglu_forward(x2, wg, wu, G, U, H, BF16, M, 5632, 2048), 4.0 * M * 5632 * 2048, 20),
+        }
+        for b in (x2, x5, w22, w52, wg, wu):
+            b.free()
+    for b in Cs + [c2, G, U, H]:
+        b.free()
+    return out
 
 
 def pick_dominant(prof, workload):
@@ -245,6 +292,8 @@ def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True, b
                            mfma_frac_of_step=round(step_flops / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 4), last_loss=round(float(last_loss), 4)),
                roofline=pick_dominant(prof, name), kernels=kernel_table(prof))
     out["roofline"]["mfma_ceiling"] = mfma_ceiling(ctx)
+    if name == "c5" and win_passes:
+        out["roofline"]["gemms_alone_by_operand_data"] = gemms_by_operand_data(ctx)
     ctx.close()
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline_lm(c, c["seq"], 1 if name == "c5" else 8)

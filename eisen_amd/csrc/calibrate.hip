@@ -14,19 +14,34 @@ namespace {
 // 64x64 wave tile of the 8-wave GEMM kernels (two A and two B reads per step); 8 = the ratio of a 128x128 wave tile;
 // 24 and 32 = more than any kernel here issues in 16-byte reads (a 64x64 wave tile whose second operand comes through
 // 8-byte transposing reads issues 24 read instructions for the same bytes): where the LDS starts to hold the MFMAs back.
+// a bf16 with random sign and mantissa and an exponent spread over 2^-4 .. 2^-1: operands whose bits change from one MFMA to
+// the next the way those of a trained layer's activations and gradients do
+__device__ __forceinline__ bf16_t random_operand(unsigned i) {
+    unsigned h = i * 2654435761u;
+    h ^= h >> 15; h *= 2246822519u; h ^= h >> 13; h *= 3266489917u; h ^= h >> 16;
+    const unsigned short bits = (unsigned short)((h & 0x8000u) | ((123u + ((h >> 7) & 3u)) << 7) | (h & 0x7Fu));
+    return __builtin_bit_cast(bf16_t, bits);
+}
+
+// RANDOM_DATA: what the operands hold.  The part's clock under matrix load depends on how many operand bits toggle between
+// consecutive MFMAs: a GEMM on all-zero or constant matrices runs a third faster than on random ones.  false: a
+// few dozen distinct small values (the optimistic ceiling); true: random signs, mantissas and exponents.
 template <int READS>
-__global__ __launch_bounds__(512) void mfma_ceiling_kernel(int iters, float* sink) {
+__global__ __launch_bounds__(512) void mfma_ceiling_kernel(int iters, float* sink, int random_data) {
     __shared__ __attribute__((aligned(16))) bf16_t tile[16 * 512];  // 16 operand reads' worth of chunks
     const int lane = threadIdx.x & 63;
-    for (int i = threadIdx.x; i < 16 * 512; i += 512) tile[i] = (bf16_t)(0.002f * (float)((i * 37) % 113) - 0.11f);
+    for (int i = threadIdx.x; i < 16 * 512; i += 512)
+        tile[i] = random_data ? random_operand(blockIdx.x * 8192u + i) : (bf16_t)(0.002f * (float)((i * 37) % 113) - 0.11f);
     __syncthreads();
     bf16x8 a[4], b[4];
 #pragma unroll
     for (int j = 0; j < 4; j++)
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            a[j][e] = (bf16_t)(0.003f * (float)((lane * 7 + j * 13 + e * 5) % 61) - 0.09f);
-            b[j][e] = (bf16_t)(0.004f * (float)((lane * 11 + j * 3 + e * 17) % 53) - 0.10f);
+            a[j][e] = random_data ? random_operand(0x10000000u + (blockIdx.x * 512u + threadIdx.x) * 64u + j * 8 + e)
+                                  : (bf16_t)(0.003f * (float)((lane * 7 + j * 13 + e * 5) % 61) - 0.09f);
+            b[j][e] = random_data ? random_operand(0x20000000u + (blockIdx.x * 512u + threadIdx.x) * 64u + j * 8 + e)
+                                  : (bf16_t)(0.004f * (float)((lane * 11 + j * 3 + e * 17) % 53) - 0.10f);
         }
     f32x16 acc[4];
 #pragma unroll
@@ -373,7 +388,14 @@ __global__ __launch_bounds__(256) void partial_sum_model_kernel(const float* __r
 
 }  // namespace
 
+static int mfma_ceiling_run(eisen_ctx* ctx, int lds_reads_per_16_mfma, int random_data, int iters, double* tflops_out);
 extern "C" int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma, int iters, double* tflops_out) {
+    return mfma_ceiling_run(ctx, lds_reads_per_16_mfma, 0, iters, tflops_out);
+}
+extern "C" int eisen_hip_mfma_ceiling_random(eisen_ctx* ctx, int lds_reads_per_16_mfma, int iters, double* tflops_out) {
+    return mfma_ceiling_run(ctx, lds_reads_per_16_mfma, 1, iters, tflops_out);
+}
+static int mfma_ceiling_run(eisen_ctx* ctx, int lds_reads_per_16_mfma, int random_data, int iters, double* tflops_out) {
     EISEN_CHECK_CTX(ctx);
     EISEN_REQUIRE(ctx, tflops_out != nullptr, EISEN_E_ARG, "mfma_ceiling: tflops_out is null");
     EISEN_REQUIRE(ctx, lds_reads_per_16_mfma == 0 || lds_reads_per_16_mfma == 8 || lds_reads_per_16_mfma == 16 || lds_reads_per_16_mfma == 24 || lds_reads_per_16_mfma == 32, EISEN_E_ARG,
@@ -389,11 +411,11 @@ extern "C" int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma,
     EISEN_HIP_TRY(ctx, hipEventCreate(&e0));
     EISEN_HIP_TRY(ctx, hipEventCreate(&e1));
     auto launch = [&](int n) {
-        if (lds_reads_per_16_mfma == 0) mfma_ceiling_kernel<0><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
-        else if (lds_reads_per_16_mfma == 8) mfma_ceiling_kernel<8><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
-        else if (lds_reads_per_16_mfma == 16) mfma_ceiling_kernel<16><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
-        else if (lds_reads_per_16_mfma == 24) mfma_ceiling_kernel<24><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
-        else mfma_ceiling_kernel<32><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink);
+        if (lds_reads_per_16_mfma == 0) mfma_ceiling_kernel<0><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink, random_data);
+        else if (lds_reads_per_16_mfma == 8) mfma_ceiling_kernel<8><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink, random_data);
+        else if (lds_reads_per_16_mfma == 16) mfma_ceiling_kernel<16><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink, random_data);
+        else if (lds_reads_per_16_mfma == 24) mfma_ceiling_kernel<24><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink, random_data);
+        else mfma_ceiling_kernel<32><<<blocks, 512, 0, ctx->stream>>>(n, (float*)sink, random_data);
     };
     launch(iters);  // warm-up: clocks and code object
     hipError_t err = hipEventRecord(e0, ctx->stream);

@@ -190,10 +190,11 @@ class Context:
             out[e.name.decode()] = dict(ms=e.ms, launches=int(e.launches), work=e.work, unit="flop" if e.work_is_flops else "byte")
         return out
 
-    def mfma_ceiling(self, lds_reads_per_16_mfma=0, iters=20000):
-        """TFLOP/s of a loop of nothing but bf16 MFMAs on every CU (operands in registers, or re-read from LDS)."""
+    def mfma_ceiling(self, lds_reads_per_16_mfma=0, iters=20000, random_operands=False):
+        """TFLOP/s of a loop of nothing but bf16 MFMAs on every CU (operands in registers, or re-read from LDS); with
+        random_operands the operands' bits change from MFMA to MFMA as real data's do, which lowers the clock the part holds."""
         out = C.c_double()
-        self._call("eisen_hip_mfma_ceiling", _i(lds_reads_per_16_mfma), _i(iters), C.byref(out))
+        self._call("eisen_hip_mfma_ceiling_random" if random_operands else "eisen_hip_mfma_ceiling", _i(lds_reads_per_16_mfma), _i(iters), C.byref(out))
         return out.value
 
     # ---- by-name launch ---------------------------------------------------------------

@@ -135,6 +135,11 @@ int eisen_hip_profile_stop(eisen_ctx* ctx, eisen_prof_entry* out, size_t capacit
  * 24, 32: one and a half times and twice the reads of a 64x64 wave tile (where the LDS begins to hold the MFMAs back).
  * Synchronises the stream. */
 int eisen_hip_mfma_ceiling(eisen_ctx* ctx, int lds_reads_per_16_mfma, int iters, double* tflops_out);
+/* The same loops on operands whose bits change from one MFMA to the next (random sign, exponent and mantissa) instead
+ * of a few dozen distinct small values.  The clock this GPU holds under matrix load depends on the operands: the same GEMM
+ * runs a third faster on all-zero or constant matrices than on random ones, so this is the ceiling to read a kernel on
+ * real data against. */
+int eisen_hip_mfma_ceiling_random(eisen_ctx* ctx, int lds_reads_per_16_mfma, int iters, double* tflops_out);
 
 /* ---- elementwise ---------------------------------------------------------------------- */
 

@@ -97,3 +97,5 @@ def test_tile_model_and_mfma_ceiling_report_sane_figures(ctx):
         ctx.attention_onepass_parts(1000, 1024, 128)
     ceiling = ctx.mfma_ceiling(0, 5000)
     assert 1250.0 < ceiling < 2500.0, ceiling
+    on_random_operands = ctx.mfma_ceiling(16, 5000, random_operands=True)
+    assert 900.0 < on_random_operands < 2500.0, on_random_operands
