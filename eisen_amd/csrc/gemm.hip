@@ -936,7 +936,7 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
         // Tile choice (measured on MI355X at the config-5 shapes): 256x128 with 8 waves and operands loaded
         // straight into three LDS stages is the fastest kernel whenever the shape is a whole number of such tiles
         // and they fill the CUs evenly (it is 5-13 % ahead of the same tile staged through registers); other
-        // large shapes run 128x128 with 4 waves, two workgroups per CU.  64x64 is for problems with few tiles.
+        // large shapes run 128x128 (direct-to-LDS with 8 waves when the shape is whole tiles, else register-staged with 4).  64x64 is for problems with few tiles.
         if (wide32) {
             // both operands through the (slower) transposing LDS reads and more than one tile per CU: slabs of 32 need
             // half the LDS, so two workgroups share a CU and cover each other's barrier waits and epilogues (6-7 % faster
@@ -954,7 +954,9 @@ static int gemm_common(eisen_ctx* ctx, const void* A, const void* B, void* C, in
             // both operands through the transposing LDS reads and at least two tiles per CU: slabs of 32 let three
             // workgroups share a CU (down-projection dW 20 % faster)
             if (whole && !a_kc && !b_kc && tiles128 * split >= 512) launch_mfma_direct<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
-            else if (whole) launch_mfma_direct<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
+            // (slabs of 64: three stages fill most of a CU's LDS, so one workgroup per CU either way; eight waves of 32 x 64 cover
+            // each other's waits where four of 64 x 64 cannot: config 4 -2 % per step, config 5's K|V launch -4 %)
+            else if (whole) launch_mfma_direct<128, 128, 64, 4, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
             else if (K % 64 == 0) launch_mfma_c<128, 128, 64, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
             else launch_mfma_c<128, 128, 32, 2, 2>(ctx, g, a_kc, b_kc, (int)batch, dtype_c);
         } else {
