@@ -108,7 +108,16 @@ def roofline_of(name, e, workload, strict=False):
     return r
 
 
+PROBES = True   # --no-probes: leave out the launches that only measure the GPU (MFMA ceilings, GEMMs by operand data), for kernel traces
+
+
 def mfma_ceiling(ctx):
+    if not PROBES:
+        return None
+    return _mfma_ceiling(ctx)
+
+
+def _mfma_ceiling(ctx):
     """What this GPU sustains on nothing but bf16 MFMAs, measured now, next to the published peak the fractions use:
     operands in registers, and re-read from LDS at the ratio of a 128x128 and of a 64x64 wave tile."""
     return dict(unit="TFLOP/s", registers_only=round(ctx.mfma_ceiling(0), 1), lds_fed_128x128_wave_tile=round(ctx.mfma_ceiling(8), 1),
@@ -292,7 +301,7 @@ def bench_lm(name, steps, warmup, with_cpu=True, recompute=False, window=True, b
                            mfma_frac_of_step=round(step_flops / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 4), last_loss=round(float(last_loss), 4)),
                roofline=pick_dominant(prof, name), kernels=kernel_table(prof))
     out["roofline"]["mfma_ceiling"] = mfma_ceiling(ctx)
-    if name == "c5" and win_passes:
+    if name == "c5" and win_passes and PROBES:
         out["roofline"]["gemms_alone_by_operand_data"] = gemms_by_operand_data(ctx)
     ctx.close()
     if with_cpu:
@@ -539,6 +548,8 @@ def main():
     ap.add_argument("--ablation", action="store_true", help="c3: time the backward kernels with one part of their tile loop left out at a time")
     ap.add_argument("--timeline", action="store_true", help="c3: where a wave of the three kernels spends its life (time stamps dropped inside the kernels)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg (profiling runs)")
+    ap.add_argument("--no-probes", action="store_true", help="skip the launches that only measure the GPU (roofline.mfma_ceiling, roofline.gemms_alone_by_operand_data): "
+                    "for kernel traces, whose per-kernel averages they would enter")
     ap.add_argument("--no-window", action="store_true", help="c5: form every micro-batch's weight gradients in its own backward pass, as the reference does, "
                     "instead of once per optimizer step over the whole accumulation window")
     ap.add_argument("--window-meet-us", type=int, default=None, help="c5: longest wait at the meeting points of the windowed weight-gradient GEMM "
@@ -549,6 +560,8 @@ def main():
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    global PROBES
+    PROBES = not args.no_probes
     w = args.workload
     if w in ("all", "c5"):
         out = bench_lm("c5", args.steps if args.steps is not None else 3, args.warmup if args.warmup is not None else 1, not args.no_cpu, args.recompute, not args.no_window, not args.no_beside, args.window_meet_us)
