@@ -189,8 +189,25 @@ __device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)
         constexpr int LPR = WN / 8, PASSES = 32 * LPR / 64;  // lanes per row, passes per band
         static_assert(32 * LPR % 64 == 0, "band must split evenly over the wave");
         const int c = lane & 31, gh = lane >> 5;
+        const bool rotate = sizeof(TC) == 2 && g.rope && bz < g.rope_members;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
+            // rotary epilogue: the band's cos / sin values are requested before the accumulators go through the LDS, so that they
+            // arrive while the band is staged (four pairs = 32 bytes per lane and pass)
+            float4 cs[PASSES][2];
+            if constexpr (sizeof(TC) == 2) {
+                if (rotate) {
+#pragma unroll
+                    for (int ps = 0; ps < PASSES; ps++) {
+                        const int idx = ps * 64 + lane, r = idx / LPR, cg = idx % LPR;
+                        const int m = m0 + wm * WM + i * 32 + r, n = n0 + wn * WN + cg * 8;
+                        const float4* src = reinterpret_cast<const float4*>(g.rope + (long long)(m % g.rope_seq) * (g.rope_head_dim >> 1) +
+                                                                            ((n % g.rope_head_dim) >> 1));
+                        cs[ps][0] = src[0];
+                        cs[ps][1] = src[1];
+                    }
+                }
+            }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -249,13 +266,11 @@ __device__ __forceinline__ void gemm_store_tile(const GemmArgs& g, f32x16 (&acc)
                     TC* dst = C + (long long)m * g.ldc + n;
                     Pack<TC> o[8 / Pack<TC>::N];
                     if constexpr (sizeof(TC) == 2) {
-                        if (g.rope && bz < g.rope_members) {
+                        if (rotate) {
                             // the product rounded to bf16 and then rotated, as the separate rotary kernel would find it
-                            const float4* cs = reinterpret_cast<const float4*>(g.rope + (long long)(m % g.rope_seq) * (g.rope_head_dim >> 1) +
-                                                                               ((n % g.rope_head_dim) >> 1));
 #pragma unroll
                             for (int q = 0; q < 2; q++) {
-                                const float4 t = cs[q];
+                                const float4 t = cs[ps][q];
                                 const float a0 = to_f32(from_f32<TC>(val[4 * q])), b0 = to_f32(from_f32<TC>(val[4 * q + 1]));
                                 const float a1 = to_f32(from_f32<TC>(val[4 * q + 2])), b1 = to_f32(from_f32<TC>(val[4 * q + 3]));
                                 rope_rotate_forward(a0, b0, make_float2(t.x, t.y), val[4 * q], val[4 * q + 1]);
