@@ -930,6 +930,39 @@ def test_gemm_grouped_ksegments_weight_gradients_over_micro_batches(ctx, shapes,
         x.free()
 
 
+@pytest.mark.parametrize("trans_b", [1, 0])
+def test_gemm_leading_dimension_beyond_32_bit_lane_offsets(ctx, trans_b):
+    # The direct-to-LDS kernels address a slab with 32-bit byte offsets per lane, which holds for leading dimensions below
+    # 2^22; a row-major operand with a longer row (here K = 2^22 + 64, 128 tiles of 128 x 128) has to take the kernels with
+    # 64-bit addresses.  Rows hold powers of two, so every sum is exact in f32 whatever its order: C[i][j] = K a_i b_j.
+    M, N, K = 2048, 1024, (1 << 22) + 64
+    a_row = [2.0 ** ((i % 5) - 2) for i in range(M)]
+    b_row = [2.0 ** ((j % 3) - 1) for j in range(N)]
+    A, C = ctx.malloc(M * K * 2), ctx.malloc(M * N * 4)
+    for i in range(M):
+        ctx.fill(A.ptr + i * K * 2, BF16, a_row[i], K)
+    if trans_b:   # B [N, K]
+        B = ctx.malloc(N * K * 2)
+        for j in range(N):
+            ctx.fill(B.ptr + j * K * 2, BF16, b_row[j], K)
+    else:         # B [K, N]: K copies of one row
+        B = ctx.upload(np.tile(np.array(b_row, np.float32), (4096, 1)), BF16)   # 4096 rows, then doubled on the device up to K
+        big = ctx.malloc(K * N * 2)
+        done = 0
+        while done < K:
+            n = min(4096, K - done)
+            ctx.dtod(big.ptr + done * N * 2, B, n * N * 2)
+            done += n
+        B.free()
+        B = big
+    ctx.gemm(A, B, C, BF16, F32, 0, trans_b, M, N, K)
+    got = dn(ctx, C, (M, N), F32)
+    exp = np.float32(K) * np.outer(np.array(a_row, np.float32), np.array(b_row, np.float32))
+    assert np.array_equal(got, exp), f"trans_b={trans_b}: {int((got != exp).sum())} of {M * N} elements differ, first at {np.argwhere(got != exp)[:1]}"
+    for x in (A, B, C):
+        x.free()
+
+
 def test_gemm_window_meeting_points_change_no_bit(ctx):
     # 352 tiles of 256x256 = 44 per XCD: a full group of 32 and a group of 12 on every XCD.  The wait at a group's meeting point
     # is bounded (40 us by default; 1 us here makes every early workgroup give up waiting) and must not show in the results.
